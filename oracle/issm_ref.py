@@ -1,0 +1,346 @@
+"""CPU oracle for the interactive-SSM (ISSM) scan and the gated RMSNorm epilogue.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this module; it is
+used by tests/, by the smoke check and by the cpu_baseline leg of bench.py as the
+checker / CPU baseline.  It is a restatement in plain PyTorch (CPU, fp64 by default)
+of the mathematics the reference evaluates, written from the formulas and never
+importing the reference.
+
+What each function restates (paths relative to the reference checkout):
+
+* ``softplus_ref``            issm_triton/softplus.py:7-16 (identity above 20)
+* ``dt_transform``            issm_triton/issm_chunk_state.py:84-99 (bias -> softplus ->
+                              clamp, in that order) and :207-220 for the backward masks
+                              (reproduced by autograd of these same ops)
+* ``issm_scan_sequential``    the recurrence that all five reference stages evaluate:
+                              issm_chunk_state.py:101-104 (a = dt'*A),
+                              issm_state_passing.py:84-104 (h0, final state),
+                              issm_chunk_scan.py:196-210 (D skip, then z gate on y+D*x)
+* ``issm_scan_chunked``       the pure-PyTorch chunked (SSD-style) formulation of
+                              test_issm.py:7-67 (segment sums, intra-chunk C.A.B^T,
+                              per-chunk states, inter-chunk recurrence, state->output),
+                              evaluated per (batch, head) so that the exp(segsum) tensor
+                              stays small.  This is the CPU baseline that is timed.
+* ``issm_chunk_scan_combined_ref``  operator-level semantics of
+                              issm_triton/issm_combined.py:16-92 (argument meaning,
+                              output dtypes) on top of the sequential recurrence
+* ``issm_bwd_closed_form``    closed-form gradients of the chunked algorithm (the sums
+                              evaluated by issm_combined.py:95-179 and the kernels it
+                              calls), used to cross-check autograd and to debug kernels
+* ``gated_rmsnorm_ref``       issm_triton/layernorm_gated.py:8-29
+
+Pinning status: every function here is pinned by tests/test_oracle.py against an
+independent brute-force numpy loop on tiny shapes, against closed forms (A=0, dt=0,
+B=0, N=P=1 by hand), by chunk-size invariance, by time-reversal symmetry and by
+torch.autograd.gradcheck.  The reference holds no golden vectors for this path
+(test_issm.py prints errors, asserts nothing, ships no data).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+INF = float("inf")
+
+
+# --------------------------------------------------------------------------- dt
+def softplus_ref(x: torch.Tensor) -> torch.Tensor:
+    """log(1+exp(x)) for x <= 20, identity above (issm_triton/softplus.py:7-16)."""
+    return torch.where(x <= 20.0, torch.log1p(torch.exp(torch.clamp(x, max=20.0))), x)
+
+
+def dt_transform(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, INF)):
+    """dt' = clamp(softplus?(dt + dt_bias), lo, hi)  (issm_chunk_state.py:84-99).
+
+    dt (B,L,H,N); dt_bias (H,N).  The clamp is always applied, so with the default
+    limits a negative dt becomes 0 (and receives zero gradient).
+    """
+    if dt_bias is not None:
+        dt = dt + dt_bias.to(dt.dtype)[None, None]
+    if dt_softplus:
+        dt = softplus_ref(dt)
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    return torch.clamp(dt, min=lo, max=hi)
+
+
+def _expand_groups(t: torch.Tensor, nheads: int) -> torch.Tensor:
+    """(B,L,G,N) -> (B,L,H,N); head h uses group h // (H/G)."""
+    g = t.shape[2]
+    assert nheads % g == 0
+    return t.repeat_interleave(nheads // g, dim=2)
+
+
+# ------------------------------------------------------------ ground truth scan
+def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
+                         initial_states=None, dt_softplus=False, dt_limit=(0.0, INF),
+                         dtype=torch.float64) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Token-by-token recurrence, differentiable, evaluated in ``dtype``.
+
+        a_t   = dt'_t * A                         (B,H,N)
+        h_t   = exp(a_t) * h_{t-1} + dt'_t * B_t * x_t     (B,H,P,N)
+        y_t   = sum_n C_t * h_t + D * x_t ;  out_t = y_t * silu(z_t) if z given
+
+    Returns (out (B,L,H,P), final_states (B,H,P,N)).
+    """
+    Bsz, L, H, P = x.shape
+    N = dt.shape[-1]
+    x_, dt_, A_, B_, C_ = (t.to(dtype) for t in (x, dt, A, B, C))
+    dtp = dt_transform(dt_, None if dt_bias is None else dt_bias.to(dtype), dt_softplus, dt_limit)
+    Bh = _expand_groups(B_, H)
+    Ch = _expand_groups(C_, H)
+    if initial_states is None:
+        h = torch.zeros(Bsz, H, P, N, dtype=dtype)
+    else:
+        h = initial_states.to(dtype)
+    ys = []
+    for t in range(L):
+        decay = torch.exp(dtp[:, t] * A_[None])                       # (B,H,N)
+        inject = (dtp[:, t] * Bh[:, t])[:, :, None, :] * x_[:, t][..., None]
+        h = decay[:, :, None, :] * h + inject
+        ys.append(torch.einsum("bhpn,bhn->bhp", h, Ch[:, t]))
+    y = torch.stack(ys, dim=1)                                        # (B,L,H,P)
+    if D is not None:
+        D_ = D.to(dtype)
+        y = y + (D_[None, None, :, None] if D_.dim() == 1 else D_[None, None]) * x_
+    if z is not None:
+        y = y * torch.nn.functional.silu(z.to(dtype))
+    return y, h
+
+
+# ------------------------------------------------- chunked formulation (baseline)
+def _segsum(a: torch.Tensor) -> torch.Tensor:
+    """a (..., T) -> S (..., T, T), S[l,s] = sum_{k=s+1..l} a_k for l>=s, -inf above."""
+    T = a.shape[-1]
+    cs = torch.cumsum(a, dim=-1)
+    S = cs[..., :, None] - cs[..., None, :]
+    keep = torch.ones(T, T, dtype=torch.bool, device=a.device).tril()
+    return S.masked_fill(~keep, -INF)
+
+
+def issm_scan_chunked(x, dtp, A, B, C, chunk, initial_states=None):
+    """Chunked evaluation of the recurrence (test_issm.py:18-67), no D / z.
+
+    x (B,L,H,P); dtp = already transformed dt' (B,L,H,N); A (H,N); B,C (B,L,G,N).
+    L must be a multiple of ``chunk`` (test_issm.py:30).  Works in the dtype of x.
+    Evaluated one (batch, head) at a time: the decay tensor exp(segsum) is then
+    (N, nc, chunk, chunk) instead of (B,H,N,nc,chunk,chunk).
+    """
+    Bsz, L, H, P = x.shape
+    N = dtp.shape[-1]
+    assert L % chunk == 0
+    nc = L // chunk
+    G = B.shape[2]
+    y = torch.empty_like(x)
+    final = torch.empty(Bsz, H, P, N, dtype=x.dtype)
+    for b in range(Bsz):
+        for h in range(H):
+            g = h // (H // G)
+            xc = x[b, :, h].reshape(nc, chunk, P)
+            dtc = dtp[b, :, h].reshape(nc, chunk, N)
+            Bc = B[b, :, g].reshape(nc, chunk, N)
+            Cc = C[b, :, g].reshape(nc, chunk, N)
+            a = (dtc * A[h][None, None]).permute(2, 0, 1)            # (N,nc,cs)
+            acs = torch.cumsum(a, dim=-1)
+            # 1. intra-chunk: M[c,l,s] = sum_n C[l,n] B[s,n] dt'[s,n] exp(segsum)[n,l,s]
+            Ldec = torch.exp(_segsum(a))                             # (N,nc,cs,cs)
+            M = torch.einsum("cln,csn,ncls->cls", Cc, Bc * dtc, Ldec)
+            y_diag = torch.bmm(M, xc)
+            # 2. per-chunk states with decay to the chunk end
+            dec_end = torch.exp(acs[..., -1:] - acs).permute(1, 2, 0)  # (nc,cs,N)
+            S = torch.einsum("clp,cln->cpn", xc, Bc * dtc * dec_end)   # (nc,P,N)
+            # 3. inter-chunk recurrence over chunk-end totals
+            h0 = torch.zeros(P, N, dtype=x.dtype) if initial_states is None else initial_states[b, h]
+            allS = torch.cat([h0[None], S], dim=0)                   # (nc+1,P,N)
+            tot = torch.nn.functional.pad(acs[..., -1], (1, 0))      # (N,nc+1)
+            dec_chunk = torch.exp(_segsum(tot))                      # (N,nc+1,nc+1)
+            Hprev = torch.einsum("nzc,cpn->zpn", dec_chunk, allS)    # (nc+1,P,N)
+            # 4. state -> output
+            y_off = torch.einsum("cln,cpn,ncl->clp", Cc, Hprev[:-1], torch.exp(acs))
+            y[b, :, h] = (y_diag + y_off).reshape(L, P)
+            final[b, h] = Hprev[-1]
+    return y, final
+
+
+def issm_chunk_scan_combined_ref(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
+                                 initial_states=None, seq_idx=None, dt_softplus=False,
+                                 dt_limit=(0.0, INF), return_final_states=False,
+                                 dtype=torch.float64):
+    """Operator-level oracle with the signature of issm_combined.py:16.
+
+    ``chunk_size`` does not change the mathematical result; it is accepted for
+    signature parity.  Output ``out`` is cast to x.dtype, final states stay fp32+
+    (issm_state_passing.py:17) -- here they are returned in ``dtype``.
+    """
+    assert seq_idx is None, "seq_idx is not used by DEST (dest_module.py:600-611)"
+    y, fin = issm_scan_sequential(x, dt, A, B, C, D=D, z=z, dt_bias=dt_bias,
+                                  initial_states=initial_states, dt_softplus=dt_softplus,
+                                  dt_limit=dt_limit, dtype=dtype)
+    return (y, fin) if return_final_states else y
+
+
+def issm_biscan_ref(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D=None, initial_states=None,
+                    dt_softplus=False, dt_bias=None, dt_limit=(0.0, INF), dtype=torch.float64):
+    """Bidirectional use of the scan (models/dest_module.py:565-575): the second scan
+    runs over the time-reversed sequence with the same dt, A, D and initial states but
+    its own x/B/C; its output is flipped back.  Returns (y_f, y_b, last_f, last_b); the
+    module averages the pairs."""
+    kw = dict(D=D, dt_bias=dt_bias, initial_states=initial_states, dt_softplus=dt_softplus,
+              dt_limit=dt_limit, dtype=dtype)
+    y_f, l_f = issm_scan_sequential(x_f, dt, A, B_f, C_f, **kw)
+    fl = lambda t: torch.flip(t, dims=[1])
+    y_b, l_b = issm_scan_sequential(fl(x_b), fl(dt), A, fl(B_b), fl(C_b), **kw)
+    return y_f, fl(y_b), l_f, l_b
+
+
+# ------------------------------------------------------- closed-form backward
+def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias=None,
+                         initial_states=None, dt_softplus=False, dt_limit=(0.0, INF),
+                         dtype=torch.float64):
+    """Gradients of the chunked algorithm written out as explicit sums (no autograd).
+
+    Mirrors what issm_combined.py:95-179 assembles from its kernels: dM (chunk_scan.py:
+    790-900), dH (chunk_scan.py:380-512), the reverse state recurrence
+    (state_passing.py:110-278), dx (combined.py:183-395), Q/G based dB and ddt
+    (chunk_state.py:493-652, cabt_bmm.py:454-673, combined.py:398-557), R/F based dC
+    (chunk_scan.py:515-657) and the dt/A reductions (chunk_state.py:107-231).
+    L need not be a multiple of chunk (tail rows have dt'=0, chunk_state.py:99).
+    z is not handled here (gate it outside).  Returns a dict of gradients in ``dtype``.
+    """
+    Bsz, L, H, P = x.shape
+    N = dt.shape[-1]
+    G = B.shape[2]
+    cs = chunk
+    nc = math.ceil(L / cs)
+    Lp = nc * cs
+    f = lambda t: t.to(dtype)
+    x_, dt_, A_, B_, C_, dy_ = map(f, (x, dt, A, B, C, dy))
+    pre = dt_ if dt_bias is None else dt_ + f(dt_bias)[None, None]
+    sp = softplus_ref(pre) if dt_softplus else pre
+    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    dtp = torch.clamp(sp, lo, hi)
+
+    def pad(t):
+        return torch.nn.functional.pad(t, (0, 0, 0, 0, 0, Lp - L)) if Lp != L else t
+
+    xp, dtpp, dyp = pad(x_), pad(dtp), pad(dy_)
+    Bp, Cp = pad(_expand_groups(B_, H)), pad(_expand_groups(C_, H))
+    # chunk views: (B,nc,cs,H,*)
+    xc = xp.reshape(Bsz, nc, cs, H, P)
+    dyc = dyp.reshape(Bsz, nc, cs, H, P)
+    dtc = dtpp.reshape(Bsz, nc, cs, H, N)
+    Bc = Bp.reshape(Bsz, nc, cs, H, N)
+    Cc = Cp.reshape(Bsz, nc, cs, H, N)
+    a = dtc * A_[None, None, None]
+    acs = torch.cumsum(a, dim=2)                                       # cs_[l,n]
+    last = acs[:, :, -1]                                               # (B,nc,H,N)
+    Bd = Bc * dtc
+    dec_end = torch.exp(last[:, :, None] - acs)
+    Bt = Bd * dec_end                                                  # B~
+    Ct = Cc * torch.exp(acs)                                           # C~
+    tril = torch.ones(cs, cs, dtype=torch.bool).tril()
+    # pairwise decay exp(cs_[l]-cs_[s]) for l>=s : (B,nc,l,s,H,N)
+    diff = acs[:, :, :, None] - acs[:, :, None, :]
+    E = torch.where(tril[None, None, :, :, None, None], torch.exp(torch.where(
+        tril[None, None, :, :, None, None], diff, torch.zeros_like(diff))), torch.zeros_like(diff))
+    # forward pieces
+    S = torch.einsum("bclhp,bclhn->bchpn", xc, Bt)
+    h0 = torch.zeros(Bsz, H, P, N, dtype=dtype) if initial_states is None else f(initial_states)
+    Hs = [h0]
+    for c in range(nc):
+        Hs.append(torch.exp(last[:, c])[:, :, None, :] * Hs[-1] + S[:, c])
+    Hprev = torch.stack(Hs[:-1], dim=1)                                # (B,nc,H,P,N)
+    M = torch.einsum("bclhn,bcshn,bclshn->bchls", Cc, Bd, E)           # tril already in E
+    # backward
+    dM = torch.einsum("bclhp,bcshp->bchls", dyc, xc) * tril[None, None, None]
+    dH = torch.einsum("bclhp,bclhn->bchpn", dyc, Ct)
+    dS = [None] * nc
+    carry = torch.zeros(Bsz, H, P, N, dtype=dtype) if dfinal is None else f(dfinal)
+    for c in range(nc - 1, -1, -1):
+        dS[c] = carry
+        carry = torch.exp(last[:, c])[:, :, None, :] * carry + dH[:, c]
+    dh0 = carry
+    dS = torch.stack(dS, dim=1)                                        # (B,nc,H,P,N)
+    g_last = torch.einsum("bchpn,bchpn->bchn", Hprev, dS) * torch.exp(last)
+    dx = (torch.einsum("bcmhn,bchpn->bcmhp", Bt, dS)
+          + torch.einsum("bchlm,bclhp->bcmhp", M, dyc))
+    Q = torch.einsum("bcmhp,bchpn->bcmhn", xc, dS)
+    R = torch.einsum("bclhp,bchpn->bclhn", dyc, Hprev)
+    Gm = torch.einsum("bchlm,bclhn,bclmhn->bcmhn", dM, Cc, E)
+    Fm = torch.einsum("bchls,bcshn,bclshn->bclhn", dM, Bd, E)
+    E1 = dec_end * Q + Gm
+    dBh = dtc * E1
+    ddtp = Bc * E1
+    dCh = torch.exp(acs) * R + Fm
+    dcs = Ct * R - Bt * Q + Cc * Fm - Bd * Gm
+    dcs[:, :, -1] = dcs[:, :, -1] + g_last + (Bt * Q).sum(dim=2)
+    da = torch.flip(torch.cumsum(torch.flip(dcs, dims=[2]), dim=2), dims=[2])
+    ddtp = ddtp + da * A_[None, None, None]
+    unchunk = lambda t: t.reshape(Bsz, Lp, H, -1)[:, :L]
+    dx = unchunk(dx)
+    ddtp = unchunk(ddtp)
+    da_u = unchunk(da)
+    out = {}
+    if D is not None:
+        D_ = f(D)
+        dx = dx + (D_[None, None, :, None] if D_.dim() == 1 else D_[None, None]) * dy_
+        out["dD"] = (dy_ * x_).sum(dim=(0, 1, 3)) if D_.dim() == 1 else (dy_ * x_).sum(dim=(0, 1))
+    clamp_ok = (sp >= lo) & (sp <= hi)
+    ddt = torch.where(clamp_ok, ddtp, torch.zeros_like(ddtp))
+    if dt_softplus:
+        ddt = torch.where(pre <= 20.0, ddt * torch.sigmoid(pre), ddt)
+    out.update(dx=dx, ddt=ddt, dA=(da_u * dtp).sum(dim=(0, 1)),
+               dB=unchunk(dBh).reshape(Bsz, L, G, H // G, N).sum(dim=3),
+               dC=unchunk(dCh).reshape(Bsz, L, G, H // G, N).sum(dim=3),
+               dinitial_states=dh0)
+    if dt_bias is not None:
+        out["ddt_bias"] = ddt.sum(dim=(0, 1))
+    return out
+
+
+# ------------------------------------------------------------- gated RMSNorm
+def gated_rmsnorm_ref(x, weight, z=None, eps=1e-5, norm_before_gate=False, group_size=None,
+                      dtype=torch.float64):
+    """RMSNorm with optional SiLU gate (issm_triton/layernorm_gated.py:8-29).
+
+    norm_before_gate=False (what DEST uses, dest_module.py:512): y = rmsnorm(x*silu(z))*w.
+    norm_before_gate=True: y = rmsnorm(x)*w*silu(z).
+    """
+    x_ = x.to(dtype)
+    w_ = weight.to(dtype)
+    z_ = None if z is None else z.to(dtype)
+    if z_ is not None and not norm_before_gate:
+        x_ = x_ * torch.nn.functional.silu(z_)
+    d = x_.shape[-1]
+    gs = d if group_size is None else group_size
+    xg = x_.reshape(*x_.shape[:-1], d // gs, gs)
+    rstd = torch.rsqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
+    out = (xg * rstd).reshape(x_.shape) * w_
+    if z_ is not None and norm_before_gate:
+        out = out * torch.nn.functional.silu(z_)
+    return out
+
+
+# ------------------------------------------------------ seeded synthetic inputs
+def make_inputs(Bsz, L, H, P, N, G=1, seed=1234, h0_std=0.0, dtype=torch.float32):
+    """Synthetic inputs of the benchmark configurations, generated on CPU in fp32 in a
+    fixed order (x, dt_raw, dt_bias, A, B, C, D, h0, dy, dfinal) and then cast.
+    x~N(0,1); dt_raw~U(-4,-1) (to be softplus'ed); A=-exp(U(ln1,ln16)) per head,
+    broadcast over N; B,C~N(0,1/sqrt(N)); D~N(0,1); h0=0 or N(0,h0_std)."""
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    u = lambda *s: torch.rand(*s, generator=g)
+    x = r(Bsz, L, H, P)
+    dt_raw = u(Bsz, L, H, N) * 3.0 - 4.0
+    dt_bias = torch.zeros(H, N)
+    A = -torch.exp(u(H) * math.log(16.0))[:, None].expand(H, N).contiguous()
+    Bm = r(Bsz, L, G, N) / math.sqrt(N)
+    Cm = r(Bsz, L, G, N) / math.sqrt(N)
+    D = r(H)
+    h0 = r(Bsz, H, P, N) * h0_std
+    dy = r(Bsz, L, H, P)
+    dfinal = r(Bsz, H, P, N)
+    c = lambda t: t.to(dtype)
+    return dict(x=c(x), dt_raw=c(dt_raw), dt_bias=dt_bias, A=A, B=c(Bm), C=c(Cm), D=D,
+                h0=h0, dy=c(dy), dfinal=dfinal)

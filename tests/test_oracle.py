@@ -1,0 +1,214 @@
+"""Pins the CPU oracle (oracle/issm_ref.py) without the reference: brute-force loops,
+closed forms, invariances and gradcheck.  A dropped term, wrong sign/index or a
+transposed operand in the oracle fails at least one of these."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import issm_ref as R
+
+torch.manual_seed(0)
+
+
+def _rand_problem(Bsz=2, L=12, H=4, P=3, N=5, G=2, seed=0, h0=True):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    x = r(Bsz, L, H, P)
+    dt = torch.rand(Bsz, L, H, N, generator=g, dtype=torch.float64) * 0.5
+    A = -torch.exp(torch.rand(H, N, generator=g, dtype=torch.float64) * 2.0)
+    B = r(Bsz, L, G, N)
+    C = r(Bsz, L, G, N)
+    D = r(H)
+    h = r(Bsz, H, P, N) if h0 else None
+    return x, dt, A, B, C, D, h
+
+
+def _brute_numpy(x, dt, A, B, C, D, h0):
+    """Independent statement of the recurrence with scalar loops only."""
+    x, dt, A, B, C = (t.numpy() for t in (x, dt, A, B, C))
+    Bsz, L, H, P = x.shape
+    N = dt.shape[-1]
+    G = B.shape[2]
+    y = np.zeros((Bsz, L, H, P))
+    fin = np.zeros((Bsz, H, P, N))
+    for b in range(Bsz):
+        for h in range(H):
+            g = h // (H // G)
+            for p in range(P):
+                for n in range(N):
+                    s = 0.0 if h0 is None else float(h0[b, h, p, n])
+                    for t in range(L):
+                        s = math.exp(dt[b, t, h, n] * A[h, n]) * s + dt[b, t, h, n] * B[b, t, g, n] * x[b, t, h, p]
+                        y[b, t, h, p] += C[b, t, g, n] * s
+                    fin[b, h, p, n] = s
+    if D is not None:
+        y += D.numpy()[None, None, :, None] * x
+    return y, fin
+
+
+def test_sequential_matches_bruteforce_loops():
+    x, dt, A, B, C, D, h0 = _rand_problem()
+    y, fin = R.issm_scan_sequential(x, dt, A, B, C, D=D, initial_states=h0)
+    yb, fb = _brute_numpy(x, dt, A, B, C, D, h0)
+    np.testing.assert_allclose(y.numpy(), yb, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(fin.numpy(), fb, rtol=1e-12, atol=1e-12)
+
+
+def test_scalar_case_by_hand():
+    # N=P=H=B=1, two steps, written out by hand
+    x = torch.tensor([2.0, -1.0], dtype=torch.float64).reshape(1, 2, 1, 1)
+    dt = torch.tensor([0.5, 0.25], dtype=torch.float64).reshape(1, 2, 1, 1)
+    A = torch.tensor([[-2.0]], dtype=torch.float64)
+    B = torch.tensor([3.0, 4.0], dtype=torch.float64).reshape(1, 2, 1, 1)
+    C = torch.tensor([5.0, 6.0], dtype=torch.float64).reshape(1, 2, 1, 1)
+    h0 = torch.tensor(7.0, dtype=torch.float64).reshape(1, 1, 1, 1)
+    D = torch.tensor([0.5], dtype=torch.float64)
+    h1 = math.exp(-1.0) * 7.0 + 0.5 * 3.0 * 2.0
+    h2 = math.exp(-0.5) * h1 + 0.25 * 4.0 * (-1.0)
+    y, fin = R.issm_scan_sequential(x, dt, A, B, C, D=D, initial_states=h0)
+    assert y.flatten().tolist() == pytest.approx([5.0 * h1 + 1.0, 6.0 * h2 - 0.5], rel=1e-14)
+    assert fin.item() == pytest.approx(h2, rel=1e-14)
+
+
+def test_closed_form_A_zero_is_prefix_sum():
+    x, dt, A, B, C, D, h0 = _rand_problem(G=1)
+    A = torch.zeros_like(A)
+    y, fin = R.issm_scan_sequential(x, dt, A, B, C, initial_states=h0)
+    inj = (dt * B.expand(-1, -1, x.shape[2], -1))[:, :, :, None, :] * x[..., None]   # (B,L,H,P,N)
+    hs = h0[:, None] + torch.cumsum(inj, dim=1)
+    y_ref = torch.einsum("blhpn,bln->blhp", hs, C[:, :, 0])
+    torch.testing.assert_close(y, y_ref, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(fin, hs[:, -1], rtol=1e-12, atol=1e-12)
+
+
+def test_closed_form_dt_zero_and_B_zero():
+    x, dt, A, B, C, D, h0 = _rand_problem(G=1)
+    y, fin = R.issm_scan_sequential(x, torch.zeros_like(dt), A, B, C, D=D, initial_states=h0)
+    y_ref = torch.einsum("bhpn,bln->blhp", h0, C[:, :, 0]) + D[None, None, :, None] * x
+    torch.testing.assert_close(y, y_ref, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(fin, h0, rtol=0, atol=0)
+    # B = 0: pure decay h_t = exp(cumsum(dt*A)) * h0
+    y, fin = R.issm_scan_sequential(x, dt, A, torch.zeros_like(B), C, initial_states=h0)
+    dec = torch.exp(torch.cumsum(dt * A[None, None], dim=1))                      # (B,L,H,N)
+    y_ref = torch.einsum("bhpn,blhn,bln->blhp", h0, dec, C[:, :, 0])
+    torch.testing.assert_close(y, y_ref, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(fin, h0 * dec[:, -1][:, :, None, :], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("chunk", [1, 2, 3, 4, 6, 12])
+def test_chunked_equals_sequential_any_chunk(chunk):
+    x, dt, A, B, C, D, h0 = _rand_problem()
+    y, fin = R.issm_scan_sequential(x, dt, A, B, C, initial_states=h0)
+    yc, fc = R.issm_scan_chunked(x, dt, A, B, C, chunk, initial_states=h0)
+    torch.testing.assert_close(yc, y, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(fc, fin, rtol=1e-10, atol=1e-10)
+
+
+def test_chunked_no_initial_state_and_positive_A():
+    x, dt, A, B, C, D, _ = _rand_problem(h0=False)
+    A = A.clone()
+    A[0] = 0.3            # growing modes are legal for the math
+    y, fin = R.issm_scan_sequential(x, dt, A, B, C)
+    yc, fc = R.issm_scan_chunked(x, dt, A, B, C, 4)
+    torch.testing.assert_close(yc, y, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(fc, fin, rtol=1e-10, atol=1e-10)
+
+
+def test_softplus_and_clamp_semantics():
+    v = torch.tensor([-30.0, -1.0, 0.0, 5.0, 20.0, 20.5, 40.0], dtype=torch.float64)
+    torch.testing.assert_close(R.softplus_ref(v), torch.nn.functional.softplus(v, threshold=20.0), rtol=1e-14, atol=0)
+    assert R.softplus_ref(v)[-1].item() == 40.0
+    dt = torch.tensor([-0.2, 0.05, 0.7], dtype=torch.float64).reshape(1, 3, 1, 1)
+    out = R.dt_transform(dt, dt_bias=torch.tensor([[0.1]], dtype=torch.float64), dt_limit=(0.0, 0.5))
+    assert out.flatten().tolist() == pytest.approx([0.0, 0.15, 0.5])
+    # order is bias -> softplus -> clamp
+    out = R.dt_transform(dt, dt_bias=torch.tensor([[0.1]], dtype=torch.float64), dt_softplus=True, dt_limit=(0.0, 0.72))
+    exp = [min(math.log1p(math.exp(t + 0.1)), 0.72) for t in (-0.2, 0.05, 0.7)]
+    assert out.flatten().tolist() == pytest.approx(exp)
+
+
+def test_D_with_hdim_and_z_gate_order():
+    x, dt, A, B, C, D, h0 = _rand_problem()
+    D2 = torch.randn(x.shape[2], x.shape[3], dtype=torch.float64)
+    z = torch.randn_like(x)
+    y0, _ = R.issm_scan_sequential(x, dt, A, B, C, initial_states=h0)
+    y1, _ = R.issm_scan_sequential(x, dt, A, B, C, D=D2, z=z, initial_states=h0)
+    # gate applies to y + D*x (issm_chunk_scan.py:196-210)
+    torch.testing.assert_close(y1, (y0 + D2[None, None] * x) * torch.nn.functional.silu(z), rtol=1e-12, atol=1e-12)
+
+
+def test_time_reversal_symmetry_of_biscan():
+    x, dt, A, B, C, D, h0 = _rand_problem()
+    xb, Bb, Cb = torch.randn_like(x), torch.randn_like(B), torch.randn_like(C)
+    yf, yb, lf, lb = R.issm_biscan_ref(x, xb, dt, A, B, Bb, C, Cb, D=D, initial_states=h0)
+    y2, l2 = R.issm_scan_sequential(x, dt, A, B, C, D=D, initial_states=h0)
+    torch.testing.assert_close(yf, y2, rtol=0, atol=0)
+    # backward direction by explicit index reversal in a loop
+    yb_np, lb_np = _brute_numpy(xb.flip(1), dt.flip(1), A, Bb.flip(1), Cb.flip(1), D, h0)
+    np.testing.assert_allclose(yb.numpy(), yb_np[:, ::-1], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(lb.numpy(), lb_np, rtol=1e-12, atol=1e-12)
+
+
+def test_gradcheck_sequential_tiny():
+    x, dt, A, B, C, D, h0 = _rand_problem(Bsz=1, L=4, H=2, P=2, N=3, G=1)
+    ins = [t.clone().requires_grad_() for t in (x, dt, A, B, C, D, h0)]
+
+    def f(x, dt, A, B, C, D, h0):
+        return R.issm_scan_sequential(x, dt, A, B, C, D=D, initial_states=h0)
+
+    assert torch.autograd.gradcheck(f, ins, eps=1e-6, atol=1e-7, rtol=1e-5)
+
+
+@pytest.mark.parametrize("L,chunk,softplus", [(12, 4, False), (10, 4, True), (7, 8, True)])
+def test_closed_form_backward_matches_autograd(L, chunk, softplus):
+    x, dt, A, B, C, D, h0 = _rand_problem(L=L, seed=3)
+    if softplus:
+        dt = dt * 8.0 - 3.0                     # pre-softplus values, some negative
+    dt_bias = torch.randn(A.shape, dtype=torch.float64) * 0.1
+    lim = (0.05, 1.5) if softplus else (0.0, R.INF)
+    dy = torch.randn_like(x)
+    dfin = torch.randn_like(h0)
+    ins = [t.clone().requires_grad_() for t in (x, dt, A, B, C, D, dt_bias, h0)]
+    y, fin = R.issm_scan_sequential(ins[0], ins[1], ins[2], ins[3], ins[4], D=ins[5], dt_bias=ins[6],
+                                    initial_states=ins[7], dt_softplus=softplus, dt_limit=lim)
+    (y * dy).sum().add((fin * dfin).sum()).backward()
+    g = R.issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=dfin, D=D, dt_bias=dt_bias,
+                               initial_states=h0, dt_softplus=softplus, dt_limit=lim)
+    names = ["dx", "ddt", "dA", "dB", "dC", "dD", "ddt_bias", "dinitial_states"]
+    for name, t in zip(names, ins):
+        torch.testing.assert_close(g[name], t.grad, rtol=1e-9, atol=1e-9, msg=lambda m: f"{name}: {m}")
+    # invariant: dA = sum_{b,t} da * dt'  is implied by ddt/dA agreeing; also clamp mask zeros exist
+    if softplus:
+        assert (g["ddt"] == 0).any()
+
+
+def test_gated_rmsnorm_closed_form_and_grad():
+    x = torch.randn(3, 5, 8, dtype=torch.float64)
+    z = torch.randn(3, 5, 8, dtype=torch.float64)
+    w = torch.randn(8, dtype=torch.float64)
+    y = R.gated_rmsnorm_ref(x, w, z=z, eps=1e-5, norm_before_gate=False)
+    u = x * z * torch.sigmoid(z)
+    exp = u / torch.sqrt((u * u).mean(-1, keepdim=True) + 1e-5) * w
+    torch.testing.assert_close(y, exp, rtol=1e-13, atol=1e-13)
+    y2 = R.gated_rmsnorm_ref(x, w, z=z, eps=1e-5, norm_before_gate=True)
+    exp2 = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w * z * torch.sigmoid(z)
+    torch.testing.assert_close(y2, exp2, rtol=1e-13, atol=1e-13)
+    # scale invariance of rmsnorm without gate (eps -> 0)
+    y3 = R.gated_rmsnorm_ref(x, w, eps=0.0)
+    torch.testing.assert_close(R.gated_rmsnorm_ref(3.0 * x, w, eps=0.0), y3, rtol=1e-12, atol=1e-12)
+    # each row of y3/w has unit mean square
+    torch.testing.assert_close(((y3 / w) ** 2).mean(-1), torch.ones(3, 5, dtype=torch.float64), rtol=1e-12, atol=1e-12)
+    ins = [t.clone().requires_grad_() for t in (x[:1, :2], w, z[:1, :2])]
+    assert torch.autograd.gradcheck(lambda a, b, c: R.gated_rmsnorm_ref(a, b, z=c), ins, eps=1e-6, atol=1e-7)
+
+
+def test_make_inputs_is_deterministic_and_in_range():
+    a = R.make_inputs(1, 8, 2, 4, 8, seed=7)
+    b = R.make_inputs(1, 8, 2, 4, 8, seed=7)
+    for k in a:
+        assert torch.equal(a[k], b[k])
+    assert a["dt_raw"].min() >= -4 and a["dt_raw"].max() <= -1
+    assert (a["A"] <= -1).all() and (a["A"] >= -16).all()
+    assert (a["A"][:, :1] == a["A"]).all()
