@@ -1,0 +1,154 @@
+"""ctypes binding of libissm_hip.so (the C ABI declared in include/issm.h).
+
+The library is the only compute path of this package: if it is missing, loading fails
+loudly -- there is no PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Sequence
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libissm_hip.so")
+
+ISSM_CHUNK = 64
+ISSM_F32, ISSM_BF16 = 0, 1
+FLAG_DT_SOFTPLUS, FLAG_D_HAS_HDIM, FLAG_SEQ_IDX = 1, 2, 4
+
+EXPORTS = [
+    "issm_abi_version", "issm_last_error", "issm_fwd_workspace_bytes", "issm_bwd_workspace_bytes",
+    "issm_scan_fwd", "issm_scan_bwd", "issm_stage_chunk_local", "issm_stage_state_passing_fwd",
+    "issm_stage_chunk_scan", "issm_stage_bwd_gate", "issm_stage_bwd_dstates",
+    "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_stage_bwd_dx", "issm_stage_bwd_reduce",
+    "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
+]
+
+
+class Dims(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk_size", "ndir")]
+
+
+class Tensor(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("stride", C.c_int64 * 3)]
+
+
+class ScanArgs(C.Structure):
+    _fields_ = [
+        ("dims", Dims),
+        ("io_dtype", C.c_int32), ("dt_dtype", C.c_int32), ("h0_dtype", C.c_int32),
+        ("flags", C.c_uint32),
+        ("dt_min", C.c_float), ("dt_max", C.c_float),
+        ("x", Tensor * 2), ("dt", Tensor), ("Bm", Tensor * 2), ("Cm", Tensor * 2), ("z", Tensor * 2),
+        ("A", C.c_void_p), ("D", C.c_void_p), ("dt_bias", C.c_void_p),
+        ("h0", Tensor),
+        ("out", Tensor * 2),
+        ("final_states", C.c_void_p * 2),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("saved", C.c_void_p),
+        ("dout", Tensor * 2),
+        ("dfinal", C.c_void_p * 2),
+        ("dx", Tensor * 2), ("dB", Tensor * 2), ("dC", Tensor * 2), ("dz", Tensor * 2),
+        ("ddt", Tensor),
+        ("dA", C.c_void_p), ("dD", C.c_void_p), ("ddt_bias", C.c_void_p), ("dh0", C.c_void_p),
+        ("bwd_workspace", C.c_void_p), ("bwd_workspace_bytes", C.c_size_t),
+        ("stream", C.c_void_p),
+    ]
+
+
+class NormArgs(C.Structure):
+    _fields_ = [
+        ("rows", C.c_int64), ("ncols", C.c_int32), ("group_size", C.c_int32),
+        ("dtype", C.c_int32), ("weight_dtype", C.c_int32), ("norm_before_gate", C.c_int32),
+        ("eps", C.c_float),
+        ("x", C.c_void_p), ("z", C.c_void_p), ("w", C.c_void_p),
+        ("x_row_stride", C.c_int64), ("z_row_stride", C.c_int64),
+        ("y", C.c_void_p), ("y_row_stride", C.c_int64),
+        ("rstd", C.c_void_p),
+        ("dy", C.c_void_p), ("dy_row_stride", C.c_int64),
+        ("dx", C.c_void_p), ("dz", C.c_void_p),
+        ("dx_row_stride", C.c_int64), ("dz_row_stride", C.c_int64),
+        ("dw_partial", C.c_void_p), ("dw", C.c_void_p),
+        ("stream", C.c_void_p),
+    ]
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m dest3d_amd.build` "
+            "(hipcc, --offload-arch=gfx950).  This package has no fallback path.")
+    lib = C.CDLL(LIB_PATH)
+    lib.issm_last_error.restype = C.c_char_p
+    P = C.POINTER
+    lib.issm_fwd_workspace_bytes.argtypes = [P(ScanArgs), P(C.c_size_t)]
+    lib.issm_bwd_workspace_bytes.argtypes = [P(ScanArgs), P(C.c_size_t)]
+    lib.issm_scan_fwd.argtypes = [P(ScanArgs)]
+    lib.issm_scan_bwd.argtypes = [P(ScanArgs)]
+    vp = C.c_void_p
+    lib.issm_stage_chunk_local.argtypes = [P(ScanArgs), vp, vp, vp]
+    lib.issm_stage_state_passing_fwd.argtypes = [P(ScanArgs), vp, vp]
+    lib.issm_stage_chunk_scan.argtypes = [P(ScanArgs), vp, vp, vp]
+    lib.issm_stage_bwd_gate.argtypes = [P(ScanArgs), vp, vp]
+    lib.issm_stage_bwd_dstates.argtypes = [P(ScanArgs), vp, vp, vp]
+    lib.issm_stage_state_passing_bwd.argtypes = [P(ScanArgs), vp, vp, vp, vp, vp]
+    lib.issm_stage_bwd_chunk.argtypes = [P(ScanArgs), C.c_int, vp, vp, vp, vp, vp, vp, vp]
+    lib.issm_stage_bwd_dx.argtypes = [P(ScanArgs), vp, vp, vp, vp]
+    lib.issm_stage_bwd_reduce.argtypes = [P(ScanArgs), vp, vp, vp, vp]
+    lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
+    lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
+    lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
+    for name in EXPORTS:
+        if name != "issm_last_error":
+            getattr(lib, name).restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed (status {rc}): {load().issm_last_error().decode()}")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return ISSM_F32
+    if dt == torch.bfloat16:
+        return ISSM_BF16
+    raise TypeError(f"unsupported dtype {dt}: the ISSM kernels take float32 or bfloat16")
+
+
+def tensor_desc(t: Optional[torch.Tensor]) -> Tensor:
+    """Descriptor of a 4-D tensor whose last dim is contiguous (or an absent tensor)."""
+    d = Tensor()
+    if t is None:
+        d.ptr = None
+        return d
+    assert t.dim() == 4 and t.stride(-1) == 1, "innermost dimension must be contiguous"
+    d.ptr = t.data_ptr()
+    for i in range(3):
+        d.stride[i] = t.stride(i)
+    return d
+
+
+def ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def current_stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on a HIP device: the ISSM operator has no CPU path")

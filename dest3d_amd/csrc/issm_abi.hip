@@ -1,0 +1,366 @@
+// C ABI of libissm_hip.so: argument validation, workspace carving and stage sequencing.
+// All device work lives in issm_fwd.hip / issm_bwd.hip / rmsnorm_gated.hip.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/issm.h"
+#include "issm_dev.h"
+
+namespace issm {
+int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, hipStream_t st);
+int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream_t st);
+int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float* out_x, hipStream_t st);
+int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t st);
+int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* dm, hipStream_t st);
+int launch_state_bwd(const KP& p, const float* states, const float* cs_last, float* dstates, float* g_last,
+                     float* dh0_dir, hipStream_t st);
+int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
+                     const float* g_last, float* partA, float* partBias, hipStream_t st);
+int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const float* cabt, float* partD,
+                  hipStream_t st);
+int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, const float* partD,
+                      const float* dh0_dir, float* dA, float* dbias, float* dD, float* dh0, hipStream_t st);
+
+int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
+int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
+}  // namespace issm
+
+using namespace issm;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static TensorD td(const issm_tensor& t) {
+  TensorD r;
+  r.ptr = t.ptr;
+  r.s0 = t.stride[0];
+  r.s1 = t.stride[1];
+  r.s2 = t.stride[2];
+  return r;
+}
+
+static size_t align64(size_t nfloats) { return (nfloats + 63) & ~(size_t)63; }
+
+struct FwdWs {
+  size_t states, cs_last, cabt, out_x, total;  // offsets in floats
+};
+struct BwdWs {
+  size_t dstates, dm, g_last, dh0_dir, partA, partBias, partD, dy_ws, total;
+};
+
+static int nchunks(const issm_dims& d) { return (d.seqlen + ISSM_CHUNK - 1) / ISSM_CHUNK; }
+
+static FwdWs fwd_layout(const issm_dims& d, bool has_z) {
+  const size_t Bt = (size_t)d.batch * d.ndir, nc = nchunks(d), H = d.nheads, P = d.headdim, N = d.dstate;
+  FwdWs w;
+  size_t o = 0;
+  w.states = o; o += align64(Bt * (nc + 1) * H * P * N);
+  w.cs_last = o; o += align64(Bt * nc * H * N);
+  w.cabt = o; o += align64(Bt * nc * H * ISSM_CHUNK * ISSM_CHUNK);
+  w.out_x = o; if (has_z) o += align64(Bt * d.seqlen * H * P);
+  w.total = o;
+  return w;
+}
+
+static BwdWs bwd_layout(const issm_dims& d, bool has_z) {
+  const size_t Bt = (size_t)d.batch * d.ndir, nc = nchunks(d), H = d.nheads, P = d.headdim, N = d.dstate;
+  BwdWs w;
+  size_t o = 0;
+  w.dstates = o; o += align64(Bt * nc * H * P * N);
+  w.dm = o; o += align64(Bt * nc * H * ISSM_CHUNK * ISSM_CHUNK);
+  w.g_last = o; o += align64(Bt * nc * H * N);
+  w.dh0_dir = o; o += align64((size_t)d.ndir * d.batch * H * P * N);
+  w.partA = o; o += align64(Bt * nc * H * N);
+  w.partBias = o; o += align64(Bt * nc * H * N);
+  w.partD = o; o += align64(Bt * nc * H * P);
+  w.dy_ws = o; if (has_z) o += align64(Bt * d.seqlen * H * P);
+  w.total = o;
+  return w;
+}
+
+static int check_dims(const issm_scan_args* a) {
+  if (!a) return fail(ISSM_E_NULL, "args is NULL");
+  const issm_dims& d = a->dims;
+  if (d.batch <= 0 || d.seqlen <= 0 || d.nheads <= 0 || d.headdim <= 0 || d.dstate <= 0 || d.ngroups <= 0)
+    return fail(ISSM_E_SHAPE, "non-positive dimension (B=%d L=%d H=%d P=%d N=%d G=%d)", d.batch, d.seqlen, d.nheads,
+                d.headdim, d.dstate, d.ngroups);
+  if (d.chunk_size <= 0) return fail(ISSM_E_SHAPE, "chunk_size must be positive, got %d", d.chunk_size);
+  if (d.nheads % d.ngroups) return fail(ISSM_E_SHAPE, "nheads %d not divisible by ngroups %d", d.nheads, d.ngroups);
+  if (d.ndir != 1 && d.ndir != 2) return fail(ISSM_E_SHAPE, "ndir must be 1 or 2, got %d", d.ndir);
+  if (d.headdim > MAXP) return fail(ISSM_E_UNSUPPORTED, "headdim %d > %d is not built", d.headdim, MAXP);
+  if ((long)d.batch * d.ndir * nchunks(d) * d.nheads > 0x7fffffffL) return fail(ISSM_E_SHAPE, "too many chunk units");
+  return ISSM_OK;
+}
+
+static int check_common(const issm_scan_args* a) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  if ((unsigned)a->io_dtype > 1u || (unsigned)a->dt_dtype > 1u || (unsigned)a->h0_dtype > 1u)
+    return fail(ISSM_E_DTYPE, "unknown dtype code (io=%d dt=%d h0=%d)", a->io_dtype, a->dt_dtype, a->h0_dtype);
+  if (a->flags & ISSM_FLAG_SEQ_IDX) return fail(ISSM_E_UNSUPPORTED, "seq_idx is not supported");
+  if (!(a->dt_min >= 0.0f)) return fail(ISSM_E_UNSUPPORTED, "dt_limit[0] = %g < 0 is not supported", a->dt_min);
+  if (!(a->dt_max >= a->dt_min)) return fail(ISSM_E_SHAPE, "dt_limit is empty (%g, %g)", a->dt_min, a->dt_max);
+  if (!a->A) return fail(ISSM_E_NULL, "A is NULL");
+  if (!a->dt.ptr) return fail(ISSM_E_NULL, "dt is NULL");
+  for (int dir = 0; dir < a->dims.ndir; ++dir) {
+    if (!a->x[dir].ptr || !a->Bm[dir].ptr || !a->Cm[dir].ptr)
+      return fail(ISSM_E_NULL, "x/B/C of direction %d is NULL", dir);
+    if ((a->z[0].ptr != nullptr) != (a->z[dir].ptr != nullptr))
+      return fail(ISSM_E_NULL, "z must be given for all directions or none");
+  }
+  return ISSM_OK;
+}
+
+static KP make_kp(const issm_scan_args* a) {
+  KP p;
+  memset(&p, 0, sizeof(p));
+  const issm_dims& d = a->dims;
+  p.B = d.batch; p.L = d.seqlen; p.H = d.nheads; p.P = d.headdim; p.N = d.dstate; p.G = d.ngroups;
+  p.ndir = d.ndir; p.nc = nchunks(d); p.hpg = d.nheads / d.ngroups; p.dir0 = 0;
+  p.io_dt = a->io_dtype; p.dt_dt = a->dt_dtype; p.h0_dt = a->h0_dtype;
+  p.flags = ((a->flags & ISSM_FLAG_DT_SOFTPLUS) ? F_SOFTPLUS : 0u) | ((a->flags & ISSM_FLAG_D_HAS_HDIM) ? F_D_HDIM : 0u);
+  p.dt_min = a->dt_min; p.dt_max = a->dt_max;
+  for (int i = 0; i < 2; ++i) {
+    p.x[i] = td(a->x[i]); p.Bm[i] = td(a->Bm[i]); p.Cm[i] = td(a->Cm[i]); p.z[i] = td(a->z[i]);
+    p.out[i] = td(a->out[i]); p.dout[i] = td(a->dout[i]); p.dx[i] = td(a->dx[i]); p.dB[i] = td(a->dB[i]);
+    p.dC[i] = td(a->dC[i]); p.dz[i] = td(a->dz[i]);
+    p.final_states[i] = a->final_states[i];
+    p.dfinal[i] = a->dfinal[i];
+  }
+  p.dt = td(a->dt); p.ddt = td(a->ddt); p.h0 = td(a->h0);
+  p.A = a->A; p.D = a->D; p.dt_bias = a->dt_bias;
+  return p;
+}
+
+static int launched(int hip_err, const char* what) {
+  if (hip_err == 0) return ISSM_OK;
+  return fail(ISSM_E_LAUNCH, "%s: %s", what, hipGetErrorString((hipError_t)hip_err));
+}
+
+extern "C" {
+
+int issm_abi_version(void) { return ISSM_ABI_VERSION; }
+const char* issm_last_error(void) { return g_err; }
+
+int issm_fwd_workspace_bytes(const issm_scan_args* a, size_t* out) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  if (!out) return fail(ISSM_E_NULL, "out is NULL");
+  *out = fwd_layout(a->dims, a->z[0].ptr != nullptr).total * sizeof(float);
+  return ISSM_OK;
+}
+
+int issm_bwd_workspace_bytes(const issm_scan_args* a, size_t* out) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  if (!out) return fail(ISSM_E_NULL, "out is NULL");
+  *out = bwd_layout(a->dims, a->z[0].ptr != nullptr).total * sizeof(float);
+  return ISSM_OK;
+}
+
+int issm_stage_chunk_local(const issm_scan_args* a, float* states, float* cs_last, float* cabt) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!cs_last) return fail(ISSM_E_NULL, "cs_last is NULL");
+  KP p = make_kp(a);
+  return launched(launch_chunk_local(p, states, cs_last, cabt, (hipStream_t)a->stream), "chunk_local");
+}
+
+int issm_stage_state_passing_fwd(const issm_scan_args* a, float* states, const float* cs_last) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  if (!states || !cs_last) return fail(ISSM_E_NULL, "states/cs_last is NULL");
+  KP p = make_kp(a);
+  return launched(launch_state_fwd(p, states, cs_last, (hipStream_t)a->stream), "state_passing_fwd");
+}
+
+int issm_stage_chunk_scan(const issm_scan_args* a, const float* states, const float* cabt, float* out_x) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!states || !cabt) return fail(ISSM_E_NULL, "states/cabt is NULL");
+  for (int dir = 0; dir < a->dims.ndir; ++dir)
+    if (!a->out[dir].ptr) return fail(ISSM_E_NULL, "out of direction %d is NULL", dir);
+  if (a->z[0].ptr && !out_x) return fail(ISSM_E_NULL, "out_x is required when z is given");
+  KP p = make_kp(a);
+  return launched(launch_chunk_scan(p, states, cabt, out_x, (hipStream_t)a->stream), "chunk_scan");
+}
+
+int issm_scan_fwd(const issm_scan_args* a) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  const bool has_z = a->z[0].ptr != nullptr;
+  const FwdWs w = fwd_layout(a->dims, has_z);
+  if (!a->workspace || a->workspace_bytes < w.total * sizeof(float))
+    return fail(ISSM_E_WORKSPACE, "forward workspace: need %zu bytes, got %zu", w.total * sizeof(float),
+                a->workspace ? a->workspace_bytes : (size_t)0);
+  for (int dir = 0; dir < a->dims.ndir; ++dir)
+    if (!a->out[dir].ptr) return fail(ISSM_E_NULL, "out of direction %d is NULL", dir);
+  float* ws = (float*)a->workspace;
+  KP p = make_kp(a);
+  hipStream_t st = (hipStream_t)a->stream;
+  if ((rc = launched(launch_chunk_local(p, ws + w.states, ws + w.cs_last, ws + w.cabt, st), "chunk_local"))) return rc;
+  if ((rc = launched(launch_state_fwd(p, ws + w.states, ws + w.cs_last, st), "state_passing_fwd"))) return rc;
+  return launched(launch_chunk_scan(p, ws + w.states, ws + w.cabt, has_z ? ws + w.out_x : nullptr, st), "chunk_scan");
+}
+
+int issm_stage_bwd_gate(const issm_scan_args* a, const float* out_x, float* dy_gated) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if (!out_x || !dy_gated || !a->z[0].ptr) return fail(ISSM_E_NULL, "out_x/dy_gated/z is NULL");
+  KP p = make_kp(a);
+  return launched(launch_bwd_gate(p, out_x, dy_gated, (hipStream_t)a->stream), "bwd_gate");
+}
+
+static int check_dout(const issm_scan_args* a, const float* dy_gated) {
+  if (dy_gated) return ISSM_OK;
+  for (int dir = 0; dir < a->dims.ndir; ++dir)
+    if (!a->dout[dir].ptr) return fail(ISSM_E_NULL, "dout of direction %d is NULL", dir);
+  return ISSM_OK;
+}
+
+int issm_stage_bwd_dstates(const issm_scan_args* a, const float* dy_gated, float* dstates, float* dm) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if ((rc = check_dout(a, dy_gated))) return rc;
+  KP p = make_kp(a);
+  return launched(launch_bwd_dstates(p, dy_gated, dstates, dm, (hipStream_t)a->stream), "bwd_dstates");
+}
+
+int issm_stage_state_passing_bwd(const issm_scan_args* a, const float* states, const float* cs_last, float* dstates,
+                                 float* g_last, float* dh0_dir) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  if (!states || !cs_last || !dstates || !g_last || !dh0_dir) return fail(ISSM_E_NULL, "state_passing_bwd: NULL buffer");
+  KP p = make_kp(a);
+  return launched(launch_state_bwd(p, states, cs_last, dstates, g_last, dh0_dir, (hipStream_t)a->stream),
+                  "state_passing_bwd");
+}
+
+int issm_stage_bwd_chunk(const issm_scan_args* a, int dir, const float* dy_gated, const float* states,
+                         const float* dstates, const float* dm, const float* g_last, float* part_a,
+                         float* part_bias) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if ((rc = check_dout(a, dy_gated))) return rc;
+  if (dir < 0 || dir >= a->dims.ndir) return fail(ISSM_E_SHAPE, "dir %d out of range", dir);
+  if (!states || !dstates || !dm || !g_last || !part_a || !part_bias) return fail(ISSM_E_NULL, "bwd_chunk: NULL buffer");
+  KP p = make_kp(a);
+  p.dir0 = dir;
+  return launched(launch_bwd_chunk(p, dy_gated, states, dstates, dm, g_last, part_a, part_bias, (hipStream_t)a->stream),
+                  "bwd_chunk");
+}
+
+int issm_stage_bwd_dx(const issm_scan_args* a, const float* dy_gated, const float* dstates, const float* cabt,
+                      float* part_d) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  if ((rc = check_dout(a, dy_gated))) return rc;
+  if (!dstates || !cabt) return fail(ISSM_E_NULL, "bwd_dx: NULL buffer");
+  if (a->D && a->dD && !part_d) return fail(ISSM_E_NULL, "bwd_dx: part_d is NULL");
+  KP p = make_kp(a);
+  return launched(launch_bwd_dx(p, dy_gated, dstates, cabt, part_d, (hipStream_t)a->stream), "bwd_dx");
+}
+
+int issm_stage_bwd_reduce(const issm_scan_args* a, const float* part_a, const float* part_bias, const float* part_d,
+                          const float* dh0_dir) {
+  int rc = check_dims(a);
+  if (rc) return rc;
+  KP p = make_kp(a);
+  return launched(launch_bwd_reduce(p, part_a, part_bias, part_d, dh0_dir, part_a ? a->dA : nullptr,
+                                    (part_bias && a->dt_bias) ? a->ddt_bias : nullptr,
+                                    (part_d && a->D) ? a->dD : nullptr, dh0_dir ? a->dh0 : nullptr,
+                                    (hipStream_t)a->stream),
+                  "bwd_reduce");
+}
+
+int issm_scan_bwd(const issm_scan_args* a) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  const bool has_z = a->z[0].ptr != nullptr;
+  const FwdWs fw = fwd_layout(a->dims, has_z);
+  const BwdWs bw = bwd_layout(a->dims, has_z);
+  if (!a->saved) return fail(ISSM_E_WORKSPACE, "saved forward workspace is NULL");
+  if (!a->bwd_workspace || a->bwd_workspace_bytes < bw.total * sizeof(float))
+    return fail(ISSM_E_WORKSPACE, "backward workspace: need %zu bytes, got %zu", bw.total * sizeof(float),
+                a->bwd_workspace ? a->bwd_workspace_bytes : (size_t)0);
+  for (int dir = 0; dir < a->dims.ndir; ++dir)
+    if (!a->dout[dir].ptr) return fail(ISSM_E_NULL, "dout of direction %d is NULL", dir);
+  const float* sv = (const float*)a->saved;
+  float* ws = (float*)a->bwd_workspace;
+  KP p = make_kp(a);
+  hipStream_t st = (hipStream_t)a->stream;
+  const float* dy = nullptr;
+  if (has_z) {
+    if ((rc = launched(launch_bwd_gate(p, sv + fw.out_x, ws + bw.dy_ws, st), "bwd_gate"))) return rc;
+    dy = ws + bw.dy_ws;
+  }
+  if ((rc = launched(launch_bwd_dstates(p, dy, ws + bw.dstates, ws + bw.dm, st), "bwd_dstates"))) return rc;
+  if ((rc = launched(launch_state_bwd(p, sv + fw.states, sv + fw.cs_last, ws + bw.dstates, ws + bw.g_last,
+                                      ws + bw.dh0_dir, st),
+                     "state_passing_bwd")))
+    return rc;
+  for (int dir = 0; dir < p.ndir; ++dir) {
+    KP pd = p;
+    pd.dir0 = dir;
+    if ((rc = launched(launch_bwd_chunk(pd, dy, sv + fw.states, ws + bw.dstates, ws + bw.dm, ws + bw.g_last,
+                                        ws + bw.partA, ws + bw.partBias, st),
+                       "bwd_chunk")))
+      return rc;
+  }
+  if ((rc = launched(launch_bwd_dx(p, dy, ws + bw.dstates, sv + fw.cabt, ws + bw.partD, st), "bwd_dx"))) return rc;
+  return launched(launch_bwd_reduce(p, ws + bw.partA, ws + bw.partBias, ws + bw.partD, ws + bw.dh0_dir, a->dA,
+                                    a->dt_bias ? a->ddt_bias : nullptr, a->D ? a->dD : nullptr, a->dh0, st),
+                  "bwd_reduce");
+}
+
+// ------------------------------------------------------------------ gated RMSNorm
+int issm_rmsnorm_bwd_blocks(int64_t rows) {
+  if (rows <= 0) return 0;
+  return (int)(rows < 2048 ? rows : 2048);
+}
+
+static int norm_params(const issm_norm_args* a, NormP* p, bool bwd) {
+  if (!a) return fail(ISSM_E_NULL, "args is NULL");
+  if (a->rows <= 0 || a->ncols <= 0) return fail(ISSM_E_SHAPE, "rmsnorm: rows=%lld ncols=%d", (long long)a->rows, a->ncols);
+  const int gs = a->group_size > 0 ? a->group_size : a->ncols;
+  if (a->ncols % gs) return fail(ISSM_E_SHAPE, "rmsnorm: ncols %d not divisible by group_size %d", a->ncols, gs);
+  if ((unsigned)a->dtype > 1u || (unsigned)a->weight_dtype > 1u) return fail(ISSM_E_DTYPE, "rmsnorm: unknown dtype");
+  if (!a->x || !a->w || !a->rstd) return fail(ISSM_E_NULL, "rmsnorm: x/w/rstd is NULL");
+  if (a->ncols > 16384) return fail(ISSM_E_UNSUPPORTED, "rmsnorm: ncols %d > 16384", a->ncols);
+  if (!bwd && !a->y) return fail(ISSM_E_NULL, "rmsnorm: y is NULL");
+  if (bwd && (!a->dy || !a->dx || !a->dw_partial || !a->dw)) return fail(ISSM_E_NULL, "rmsnorm bwd: NULL buffer");
+  if (bwd && a->z && !a->dz) return fail(ISSM_E_NULL, "rmsnorm bwd: dz is NULL");
+  p->rows = a->rows; p->ncols = a->ncols; p->gs = gs; p->ngroups = a->ncols / gs;
+  p->dt = a->dtype; p->wdt = a->weight_dtype; p->nbg = a->norm_before_gate; p->eps = a->eps;
+  p->x = a->x; p->z = a->z; p->w = a->w; p->xs = a->x_row_stride; p->zs = a->z_row_stride;
+  p->y = a->y; p->ys = a->y_row_stride; p->rstd = a->rstd;
+  p->dy = a->dy; p->dys = a->dy_row_stride; p->dx = a->dx; p->dz = a->dz; p->dxs = a->dx_row_stride;
+  p->dzs = a->dz_row_stride; p->dw_partial = a->dw_partial; p->dw = a->dw;
+  p->nblocks = issm_rmsnorm_bwd_blocks(a->rows);
+  return ISSM_OK;
+}
+
+int issm_gated_rmsnorm_fwd(const issm_norm_args* a) {
+  NormP p;
+  int rc = norm_params(a, &p, false);
+  if (rc) return rc;
+  return launched(launch_rmsnorm_fwd(p, (hipStream_t)a->stream), "rmsnorm_fwd");
+}
+
+int issm_gated_rmsnorm_bwd(const issm_norm_args* a) {
+  NormP p;
+  int rc = norm_params(a, &p, true);
+  if (rc) return rc;
+  return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd");
+}
+
+}  // extern "C"

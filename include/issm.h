@@ -1,0 +1,231 @@
+/*
+ * issm.h -- C ABI of libissm_hip.so: the interactive-SSM (ISSM) chunked scan of DEST,
+ * forward and backward, plus the gated RMSNorm epilogue, as hand-written gfx950 HIP
+ * kernels.
+ *
+ * The reference has no native code on this path (it launches Triton kernels from
+ * Python); the entry points below are what a ctypes/cffi binding inside the
+ * reference's issm_triton/ package would call instead of those launchers.  Each
+ * declaration cites the reference function it replaces (paths relative to the
+ * reference checkout).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller.  The library never
+ *    allocates, frees or retains memory; all work is enqueued on `stream` and is
+ *    asynchronous with respect to the host.
+ *  - Every function returns ISSM_OK (0) or a negative issm_status; the message for
+ *    the calling thread's last failure is returned by issm_last_error().  Nothing
+ *    throws and nothing calls exit().
+ *  - Tensors with an issm_tensor descriptor may be strided in their first three
+ *    dimensions (element strides); the innermost dimension must be contiguous.
+ *  - Layouts: x,z,out,dout,dx,dz (B,L,H,P); dt,ddt (B,L,H,N); Bm,Cm,dB,dC (B,L,G,N);
+ *    A,dt_bias,dA,ddt_bias (H,N) fp32 contiguous; D,dD (H) or (H,P) fp32 contiguous;
+ *    h0 (B,H,P,N); final_states,dfinal,dh0 (B,H,P,N) fp32 contiguous.
+ *  - Time is split into chunks of ISSM_CHUNK tokens inside the library whatever
+ *    `chunk_size` the caller names: the result of the scan does not depend on the
+ *    chunk length.  nc = ceil(L / ISSM_CHUNK); tail rows behave as dt' = 0
+ *    (issm_triton/issm_chunk_state.py:81-100).
+ *  - ndir = 2 runs the module's bidirectional pair (models/dest_module.py:565-575) in
+ *    one call: direction 1 walks the same dt / A / D / h0 backwards in time with its
+ *    own x / Bm / Cm and writes its outputs back in natural (un-flipped) time order.
+ */
+#ifndef ISSM_H
+#define ISSM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ISSM_ABI_VERSION 1
+#define ISSM_CHUNK 64 /* tokens per internal chunk */
+
+typedef enum issm_status {
+  ISSM_OK = 0,
+  ISSM_E_NULL = -1,        /* a required pointer is NULL */
+  ISSM_E_SHAPE = -2,       /* a dimension is non-positive / inconsistent (issm_combined.py:58-83) */
+  ISSM_E_STRIDE = -3,      /* a stride is unusable */
+  ISSM_E_DTYPE = -4,       /* unknown dtype code */
+  ISSM_E_UNSUPPORTED = -5, /* legal in the reference but not built (seq_idx, dt_min < 0) */
+  ISSM_E_WORKSPACE = -6,   /* workspace missing or too small */
+  ISSM_E_LAUNCH = -7       /* hipGetLastError() != hipSuccess after a launch */
+} issm_status;
+
+typedef enum issm_dtype { ISSM_F32 = 0, ISSM_BF16 = 1 } issm_dtype;
+
+enum {
+  ISSM_FLAG_DT_SOFTPLUS = 1u << 0, /* apply softplus to dt + dt_bias (softplus.py:7-16) */
+  ISSM_FLAG_D_HAS_HDIM = 1u << 1,  /* D is (H,P) instead of (H) */
+  ISSM_FLAG_SEQ_IDX = 1u << 2      /* caller had a seq_idx: rejected with ISSM_E_UNSUPPORTED */
+};
+
+typedef struct issm_dims {
+  int32_t batch, seqlen, nheads, headdim, dstate, ngroups;
+  int32_t chunk_size; /* the caller's chunk_size, validated (> 0) and otherwise unused */
+  int32_t ndir;       /* 1 = one scan, 2 = forward + time-reversed scan */
+} issm_dims;
+
+typedef struct issm_tensor {
+  void* ptr;         /* NULL = absent */
+  int64_t stride[3]; /* element strides of dims 0,1,2 */
+} issm_tensor;
+
+/* One argument block for the forward, the backward and the stage entry points.
+ * Fields that an entry point does not use may be zero. */
+typedef struct issm_scan_args {
+  issm_dims dims;
+  int32_t io_dtype; /* issm_dtype of x, Bm, Cm, z, out, dout, dx, dB, dC, dz */
+  int32_t dt_dtype; /* issm_dtype of dt, ddt */
+  int32_t h0_dtype; /* issm_dtype of h0 */
+  uint32_t flags;
+  float dt_min, dt_max; /* dt_limit; dt_min >= 0 required */
+  /* inputs ([dir]) */
+  issm_tensor x[2];
+  issm_tensor dt;
+  issm_tensor Bm[2], Cm[2];
+  issm_tensor z[2]; /* optional gate */
+  const float* A;
+  const float* D;       /* optional */
+  const float* dt_bias; /* optional */
+  issm_tensor h0;       /* optional; strides of dims B,H,P */
+  /* forward outputs */
+  issm_tensor out[2];
+  float* final_states[2]; /* optional */
+  /* Forward workspace, issm_fwd_workspace_bytes() bytes, 256-byte aligned.  After
+   * issm_scan_fwd it holds what issm_scan_bwd needs (per-chunk entry states, the
+   * intra-chunk C.A.B^T blocks, chunk decay totals, the pre-gate output if z is given)
+   * and is passed unchanged to issm_scan_bwd as `saved`. */
+  void* workspace;
+  size_t workspace_bytes;
+  /* backward inputs */
+  const void* saved;
+  issm_tensor dout[2];
+  const float* dfinal[2]; /* optional */
+  /* backward outputs (NULL pointer = not wanted, where the math allows skipping) */
+  issm_tensor dx[2], dB[2], dC[2], dz[2];
+  issm_tensor ddt;
+  float* dA;
+  float* dD;
+  float* ddt_bias;
+  float* dh0;
+  /* backward scratch, issm_bwd_workspace_bytes() bytes, 256-byte aligned */
+  void* bwd_workspace;
+  size_t bwd_workspace_bytes;
+  void* stream; /* hipStream_t */
+} issm_scan_args;
+
+/* Version of this header the library was built against. */
+int issm_abi_version(void);
+/* Message of the calling thread's most recent failure ("" if none). */
+const char* issm_last_error(void);
+
+/* Workspace sizes for a problem (only args->dims and args->z[0].ptr are read). */
+int issm_fwd_workspace_bytes(const issm_scan_args* args, size_t* out);
+int issm_bwd_workspace_bytes(const issm_scan_args* args, size_t* out);
+
+/* Whole operator.
+ * issm_scan_fwd  replaces _issm_chunk_scan_combined_fwd (issm_triton/issm_combined.py:57-92),
+ *                called from ISSMChunkScanCombinedFn.forward (issm_combined.py:38-47).
+ * issm_scan_bwd  replaces _issm_chunk_scan_combined_bwd (issm_combined.py:95-179),
+ *                called from ISSMChunkScanCombinedFn.backward (issm_combined.py:49-54).
+ *                Unlike the reference it does not recompute the forward: it reads `saved`. */
+int issm_scan_fwd(const issm_scan_args* args);
+int issm_scan_bwd(const issm_scan_args* args);
+
+/* Stage entry points (used by the operator above; exported for tests and profiling).
+ * Intermediates, all fp32 contiguous, Bt = batch*ndir with index b*ndir+dir:
+ *   states  (Bt, nc+1, H, P, N) chunk-local end states, then (in place) slot c = state entering
+ *                               chunk c and slot nc = final state
+ *   cs_last (Bt, nc, H, N)      per-chunk total of dt'*A
+ *   cabt    (Bt, nc, H, 64, 64) intra-chunk matrix M[l][s], valid for l >= s
+ *
+ * issm_stage_chunk_local: dt transform + cumsum, chunk states and C.A.B^T in one pass
+ *   over dt.  Replaces _chunk_cumsum_fwd (issm_chunk_state.py:11-104), _chunk_state_fwd
+ *   (issm_chunk_state.py:234-356) and _bmm_CABT_chunk_fwd (issm_cabt_bmm.py:7-153).
+ *   states / cabt may be NULL to skip that product. */
+int issm_stage_chunk_local(const issm_scan_args* args, float* states, float* cs_last, float* cabt);
+/* issm_stage_state_passing_fwd: H_0 = h0, H_{c+1} = exp(cs_last_c) * H_c + S_c, in place
+ *   (states[c] becomes H_c); final = H_nc.  Replaces _state_passing_fwd
+ *   (issm_state_passing.py:5-107). */
+int issm_stage_state_passing_fwd(const issm_scan_args* args, float* states, const float* cs_last);
+/* issm_stage_chunk_scan: out = (C*exp(cs)) . H^T + tril(M) . x + D*x, optional silu(z) gate.
+ *   Replaces _chunk_scan_fwd (issm_chunk_scan.py:10-214).  out_x (optional, fp32
+ *   (Bt,L,H,P) contiguous) receives the pre-gate value when z is given. */
+int issm_stage_chunk_scan(const issm_scan_args* args, const float* states, const float* cabt,
+                          float* out_x);
+/* issm_stage_bwd_gate: z-gate backward: dz and dy = dout*silu(z) (fp32 (Bt,L,H,P) contiguous,
+ *   physical time order) from the saved pre-gate output.  Replaces _chunk_scan_bwd_dz
+ *   (issm_chunk_scan.py:217-377); its dD part is produced by issm_stage_bwd_dx. */
+int issm_stage_bwd_gate(const issm_scan_args* args, const float* out_x, float* dy_gated);
+/* issm_stage_bwd_dstates: dH_c = dy^T . (C*exp(cs)) into dstates (Bt,nc,H,P,N) and
+ *   dM = tril(dy . x^T) into dm (Bt,nc,H,64,64); either output may be NULL.  `dy` is args->dout
+ *   unless dy_gated is given.  Replaces _chunk_scan_bwd_dstates (issm_chunk_scan.py:380-512) and
+ *   _chunk_scan_bwd_dcb (issm_chunk_scan.py:790-900). */
+int issm_stage_bwd_dstates(const issm_scan_args* args, const float* dy_gated, float* dstates, float* dm);
+/* issm_stage_state_passing_bwd: reverse recurrence in place (dstates[c] becomes dS_c, the gradient
+ *   of the chunk-local end state), g_last (Bt,nc,H,N) = sum_p dS_c * H_{c+1} (the total gradient
+ *   reaching the chunk's last cumulative sum through the states), and dh0_dir (ndir,B,H,P,N).
+ *   `states` is (Bt,nc+1,H,P,N) as left by issm_stage_state_passing_fwd.  Replaces
+ *   _state_passing_bwd (issm_state_passing.py:110-278) and the sum over P at issm_combined.py:159. */
+int issm_stage_state_passing_bwd(const issm_scan_args* args, const float* states,
+                                 const float* cs_last, float* dstates, float* g_last,
+                                 float* dh0_dir);
+/* issm_stage_bwd_chunk: ddt, dB, dC of direction `dir` and the per-unit partial sums
+ *   part_a / part_bias (Bt*nc,H,N) of dA / ddt_bias.  ddt accumulates into args->ddt when
+ *   dir > 0.  Replaces _chunk_state_bwd_db (issm_chunk_state.py:493-652), _chunk_scan_bwd_dc
+ *   (issm_chunk_scan.py:515-657), _chunk_scan_chunk_state_bwd_dt (issm_combined.py:398-557),
+ *   _bmm_CABT_dbc_chunk_bwd (issm_cabt_bmm.py:454-673), _chunk_scan_bwd_ddAcs_stable
+ *   (issm_chunk_scan.py:903-1031) and the elementwise part of _chunk_cumsum_bwd
+ *   (issm_chunk_state.py:107-231). */
+int issm_stage_bwd_chunk(const issm_scan_args* args, int dir, const float* dy_gated,
+                         const float* states, const float* dstates, const float* dm,
+                         const float* g_last, float* part_a, float* part_bias);
+/* issm_stage_bwd_dx: dx and the per-unit partial sums part_d (Bt*nc*H,P) of dD.  Replaces
+ *   _chunk_scan_chunk_state_bwd_dx (issm_combined.py:183-395). */
+int issm_stage_bwd_dx(const issm_scan_args* args, const float* dy_gated, const float* dstates,
+                      const float* cabt, float* part_d);
+/* issm_stage_bwd_reduce: fixed-order sums of the partials into args->dA, ddt_bias, dD and of
+ *   dh0_dir over directions into args->dh0.  Replaces the atomics of _chunk_cumsum_bwd
+ *   (issm_chunk_state.py:224-231) and the host-side sums at issm_combined.py:236-240. */
+int issm_stage_bwd_reduce(const issm_scan_args* args, const float* part_a, const float* part_bias,
+                          const float* part_d, const float* dh0_dir);
+
+/* Gated RMSNorm epilogue: y = rmsnorm(x * silu(z)) * w  (norm_before_gate = 0, what DEST
+ * uses) or rmsnorm(x) * w * silu(z) (norm_before_gate = 1); z may be NULL.
+ * Replaces _layer_norm_fwd / _layer_norm_bwd with is_rms_norm=True, bias=None
+ * (issm_triton/layernorm_gated.py:98-137, 261-325).  x,z,y,dy,dx,dz are (rows, ncols) with
+ * a row stride in elements; ncols is split into groups of group_size (0 = one group);
+ * rstd (ngroups*rows) fp32; dw_partial (nblocks, ncols) fp32 scratch where
+ * nblocks = issm_rmsnorm_bwd_blocks(rows); dw (ncols) fp32. */
+typedef struct issm_norm_args {
+  int64_t rows;
+  int32_t ncols, group_size;
+  int32_t dtype;        /* issm_dtype of x, z, y, dy, dx, dz */
+  int32_t weight_dtype; /* issm_dtype of w */
+  int32_t norm_before_gate;
+  float eps;
+  const void *x, *z, *w;
+  int64_t x_row_stride, z_row_stride;
+  void* y;
+  int64_t y_row_stride;
+  float* rstd;
+  /* backward */
+  const void* dy;
+  int64_t dy_row_stride;
+  void *dx, *dz;
+  int64_t dx_row_stride, dz_row_stride;
+  float* dw_partial;
+  float* dw;
+  void* stream;
+} issm_norm_args;
+
+int issm_rmsnorm_bwd_blocks(int64_t rows);
+int issm_gated_rmsnorm_fwd(const issm_norm_args* args);
+int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ISSM_H */

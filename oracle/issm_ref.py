@@ -197,7 +197,7 @@ def issm_biscan_ref(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D=None, initial_states=
 # ------------------------------------------------------- closed-form backward
 def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias=None,
                          initial_states=None, dt_softplus=False, dt_limit=(0.0, INF),
-                         dtype=torch.float64):
+                         dtype=torch.float64, intermediates=False):
     """Gradients of the chunked algorithm written out as explicit sums (no autograd).
 
     Mirrors what issm_combined.py:95-179 assembles from its kernels: dM (chunk_scan.py:
@@ -206,7 +206,11 @@ def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias
     (chunk_state.py:493-652, cabt_bmm.py:454-673, combined.py:398-557), R/F based dC
     (chunk_scan.py:515-657) and the dt/A reductions (chunk_state.py:107-231).
     L need not be a multiple of chunk (tail rows have dt'=0, chunk_state.py:99).
-    z is not handled here (gate it outside).  Returns a dict of gradients in ``dtype``.
+    z is not handled here (gate it outside).  Returns a dict of gradients in ``dtype``;
+    with ``intermediates=True`` also the per-chunk tensors the stage kernels exchange:
+    S (B,nc,H,P,N) chunk-local end states, states (B,nc+1,H,P,N) entry states + final,
+    cs_last (B,nc,H,N), M / dM (B,nc,H,cs,cs) lower-triangular, dH, dS (B,nc,H,P,N),
+    g_next (B,nc,H,N) = sum_p dS_c * H_{c+1}, y (B,L,H,P) without the D term.
     """
     Bsz, L, H, P = x.shape
     N = dt.shape[-1]
@@ -296,6 +300,11 @@ def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias
                dinitial_states=dh0)
     if dt_bias is not None:
         out["ddt_bias"] = ddt.sum(dim=(0, 1))
+    if intermediates:
+        Hall = torch.stack(Hs, dim=1)
+        y = torch.einsum("bclhn,bchpn->bclhp", Ct, Hprev) + torch.einsum("bchls,bcshp->bclhp", M, xc)
+        out.update(S=S, states=Hall, cs_last=last, M=M, dM=dM, dH=dH, dS=dS,
+                   g_next=torch.einsum("bchpn,bchpn->bchn", dS, Hall[:, 1:]), y=unchunk(y))
     return out
 
 
