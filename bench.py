@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the ISSM chunked scan on one MI355X.
+
+Workload (BASELINE.json configs[1]): B=8, L=1024, H=8, P=32, N=256, G=1, chunk=64, forward +
+backward of the bidirectional pair of scans (second direction = reversed token order, same dt /
+A / D / initial states), fp32 inputs, synthetic seeded data already resident in HBM.
+One "step" = one forward + backward call of the operator.  `value` is microseconds per step.
+
+Besides the driver's JSON contract the line carries
+  roofline      the dominant kernel's achieved fraction of its bound (live HIP-event timing)
+  cpu_baseline  the oracle's chunked pure-PyTorch formulation timed on the host cores
+  stages_us     average duration of every kernel of the step
+  variants_us   fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+SHAPE = dict(B=8, L=1024, H=8, P=32, N=256, G=1, cs=64)
+
+
+def make_problem(torch, ndir, dtype, seed=1235):
+    from oracle.issm_ref import make_inputs   # data generator only (shared with the tests)
+    I = make_inputs(SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    dev = "cuda"
+    t = dict(x=[I["x"]], B=[I["B"]], C=[I["C"]], dy=[I["dy"]], dfinal=[I["dfinal"]])
+    if ndir == 2:
+        t["x"].append(torch.randn(I["x"].shape, generator=g))
+        t["B"].append(torch.randn(I["B"].shape, generator=g) / math.sqrt(SHAPE["N"]))
+        t["C"].append(torch.randn(I["C"].shape, generator=g) / math.sqrt(SHAPE["N"]))
+        t["dy"].append(torch.randn(I["x"].shape, generator=g))
+        t["dfinal"].append(torch.randn(I["dfinal"].shape, generator=g))
+    out = {k: [v.to(dev, dtype if k in ("x", "B", "C", "dy") else torch.float32) for v in vs] for k, vs in t.items()}
+    out["dt"] = torch.nn.functional.softplus(I["dt_raw"]).to(dev, dtype)   # module call pattern: dt already softplus'ed
+    out["A"] = I["A"].to(dev)
+    out["D"] = I["D"].to(dev)
+    out["h0"] = torch.zeros(SHAPE["B"], SHAPE["H"], SHAPE["P"], SHAPE["N"], device=dev)
+    return out
+
+
+class Runner:
+    """Forward + backward through the C ABI with preallocated buffers (no autograd, no allocation
+    in the timed region): exactly the kernels ISSMChunkScanCombinedFn launches."""
+
+    def __init__(self, torch, ndir, dtype):
+        from dest3d_amd import _lib as L
+        from dest3d_amd.issm_combined import _Problem
+        self.torch, self.L, self.lib = torch, L, L.load()
+        self.ndir = ndir
+        t = self.t = make_problem(torch, ndir, dtype)
+        self.prob = _Problem(t["x"], t["dt"], t["A"], t["B"], t["C"], SHAPE["cs"], t["D"], [None] * ndir, None,
+                             t["h0"], None, False, (0.0, float("inf")))
+        a = self.a = self.prob.args()
+        dev = "cuda"
+        B_, L_, H, P, N, G = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "G"))
+        e = lambda *s, dt=torch.float32: torch.empty(*s, dtype=dt, device=dev)
+        self.out = [e(B_, L_, H, P, dt=dtype) for _ in range(ndir)]
+        self.fin = [e(B_, H, P, N) for _ in range(ndir)]
+        self.dx = [e(B_, L_, H, P, dt=dtype) for _ in range(ndir)]
+        self.dB = [e(B_, L_, G, N, dt=dtype) for _ in range(ndir)]
+        self.dC = [e(B_, L_, G, N, dt=dtype) for _ in range(ndir)]
+        self.ddt = e(B_, L_, H, N, dt=dtype)
+        self.dA, self.dD, self.dh0 = e(H, N), e(H), e(B_, H, P, N)
+        self.ws = self.prob.workspace(a, bwd=False)
+        self.bws = self.prob.workspace(a, bwd=True)
+        for i in range(ndir):
+            a.out[i] = L.tensor_desc(self.out[i])
+            a.final_states[i] = self.fin[i].data_ptr()
+            a.dout[i] = L.tensor_desc(t["dy"][i])
+            a.dfinal[i] = t["dfinal"][i].data_ptr()
+            a.dx[i], a.dB[i], a.dC[i] = (L.tensor_desc(v[i]) for v in (self.dx, self.dB, self.dC))
+        a.ddt = L.tensor_desc(self.ddt)
+        a.dA, a.dD, a.dh0 = self.dA.data_ptr(), self.dD.data_ptr(), self.dh0.data_ptr()
+        a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
+        a.saved = self.ws.data_ptr()
+        a.bwd_workspace, a.bwd_workspace_bytes = self.bws.data_ptr(), self.bws.numel()
+        a.stream = L.current_stream_ptr(torch.device("cuda"))
+
+    def step(self):
+        self.L.check(self.lib.issm_scan_fwd(C.byref(self.a)), "fwd")
+        self.L.check(self.lib.issm_scan_bwd(C.byref(self.a)), "bwd")
+
+    def time_steps(self, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e6
+
+    def stage_times(self, reps=20):
+        """Average duration of each kernel, HIP events on the launch stream around `reps`
+        back-to-back launches of that kernel."""
+        torch, lib, a = self.torch, self.lib, self.a
+        nd = self.ndir
+        B_, L_, H, P, N = (SHAPE[k] for k in ("B", "L", "H", "P", "N"))
+        nc = math.ceil(L_ / 64)
+        Bt = B_ * nd
+        f = lambda *s: torch.zeros(*s, device="cuda")
+        st, csl, cabt = f(Bt, nc + 1, H, P, N), f(Bt, nc, H, N), f(Bt, nc, H, 64, 64)
+        dst, dm, gn, dh0d = f(Bt, nc, H, P, N), f(Bt, nc, H, 64, 64), f(Bt, nc, H, N), f(nd, B_, H, P, N)
+        pa, pb, pd = f(Bt * nc, H, N), f(Bt * nc, H, N), f(Bt * nc * H, P)
+        p = lambda t: t.data_ptr()
+        stages = [
+            ("chunk_local", lambda: lib.issm_stage_chunk_local(C.byref(a), p(st), p(csl), p(cabt))),
+            ("state_passing_fwd", lambda: lib.issm_stage_state_passing_fwd(C.byref(a), p(st), p(csl))),
+            ("chunk_scan", lambda: lib.issm_stage_chunk_scan(C.byref(a), p(st), p(cabt), None)),
+            ("bwd_dstates", lambda: lib.issm_stage_bwd_dstates(C.byref(a), None, p(dst), p(dm))),
+            ("state_passing_bwd", lambda: lib.issm_stage_state_passing_bwd(C.byref(a), p(st), p(csl), p(dst), p(gn), p(dh0d))),
+            ("bwd_chunk", lambda: [lib.issm_stage_bwd_chunk(C.byref(a), d, None, p(st), p(dst), p(dm), p(gn), p(pa), p(pb))
+                                   for d in range(nd)][-1]),
+            ("bwd_dx", lambda: lib.issm_stage_bwd_dx(C.byref(a), None, p(dst), p(cabt), p(pd))),
+            ("bwd_reduce", lambda: lib.issm_stage_bwd_reduce(C.byref(a), p(pa), p(pb), p(pd), p(dh0d))),
+        ]
+        res = {}
+        for name, fn in stages:
+            for _ in range(3):
+                self.L.check(fn(), name)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            e1.synchronize()
+            res[name] = e0.elapsed_time(e1) / reps * 1e3
+        return res
+
+
+def stage_work(ndir):
+    """Algorithmic FLOPs (2*MAC; exps not counted) and bytes per launch of each kernel."""
+    B_, L_, H, P, N, cs = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "cs"))
+    U = B_ * ndir * H * math.ceil(L_ / cs)
+    tri = cs * (cs + 1) // 2
+    E_cs, E_st = U * P * N, B_ * ndir * H * P * N
+    return {
+        "chunk_local": ("mfma", 2 * U * (cs * P * N + tri * N)),
+        "chunk_scan": ("mfma", 2 * U * (cs * P * N + tri * P)),
+        "bwd_dstates": ("mfma", 2 * U * (cs * P * N + tri * P)),
+        "bwd_chunk": ("mfma", 2 * U * (2 * cs * P * N + 2 * tri * N)),
+        "bwd_dx": ("mfma", 2 * U * (cs * P * N + tri * P)),
+        "state_passing_fwd": ("hbm", 4 * (2 * E_cs + U * N + 2 * E_st)),
+        "state_passing_bwd": ("hbm", 4 * (3 * E_cs + 2 * U * N + 2 * E_st)),
+    }
+
+
+def cpu_baseline(torch):
+    """Chunked pure-PyTorch formulation (oracle.issm_scan_chunked, fp32, autograd backward) on
+    the host cores, on a bounded sample: 2 of the 8 batch elements, one direction, 2 repetitions
+    (about 15-30 s); scaled by 8 (= 4 x batch, 2 x directions) to the workload's unit."""
+    from oracle import issm_ref as R
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    torch.set_num_threads(cores)
+    I = R.make_inputs(2, SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=1235)
+    ins = [I["x"].clone().requires_grad_(), torch.nn.functional.softplus(I["dt_raw"]).requires_grad_(),
+           I["A"].clone().requires_grad_(), I["B"].clone().requires_grad_(), I["C"].clone().requires_grad_()]
+    best = float("inf")
+    for _ in range(2):
+        for t in ins:
+            t.grad = None
+        t0 = time.perf_counter()
+        y, fin = R.issm_scan_chunked(*ins, SHAPE["cs"])
+        ((y * I["dy"]).sum() + (fin * I["dfinal"]).sum()).backward()
+        best = min(best, time.perf_counter() - t0)
+    return {"value": best * 8 * 1e6, "unit": "us/call", "cores": cores, "kind": "port",
+            "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    run = Runner(torch, 2, torch.float32)
+    us = run.time_steps(args.steps, args.warmup)
+    stages = run.stage_times()
+    work = stage_work(2)
+    dom = max((k for k in stages if k in work), key=lambda k: stages[k])
+    bound, amount = work[dom]
+    if bound == "mfma":
+        achieved = amount / (stages[dom] * 1e-6) / 1e12
+        roof = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None, "kernel": dom}
+    else:
+        achieved = amount / (stages[dom] * 1e-6) / 1e9
+        roof = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": achieved / PEAK_HBM_GBS, "traffic": None, "kernel": dom}
+    per_stage = {}
+    for k, (b, amt) in work.items():
+        rate = amt / (stages[k] * 1e-6)
+        per_stage[k] = {"us": round(stages[k], 2), "bound": b,
+                        "frac": round(rate / (PEAK_FP32_MFMA_TFLOPS * 1e12 if b == "mfma" else PEAK_HBM_GBS * 1e9), 4)}
+    variants = {}
+    if not args.no_variants:
+        for name, nd, dt in (("uni_fp32", 1, torch.float32), ("uni_bf16", 1, torch.bfloat16),
+                             ("bidir_bf16", 2, torch.bfloat16)):
+            r = Runner(torch, nd, dt)
+            variants[name] = round(r.time_steps(max(args.steps // 2, 5), 5), 2)
+            del r
+    line = {
+        "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: B=8 L=1024 H=8 P=32 N=256 G=1 chunk=64, fwd+bwd, bidirectional pair "
+                               "(fused), fp32 I/O, fp32 MFMA accumulate"},
+        "roofline": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in roof.items()},
+        "stages_us": {k: round(v, 2) for k, v in stages.items()},
+        "stage_roofline": per_stage,
+        "variants_us": variants,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(torch)
+        line["cpu_baseline"]["value"] = round(line["cpu_baseline"]["value"], 1)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
