@@ -3,10 +3,10 @@
 //   k_bwd_gate      z-gate backward (elementwise)
 //   k_bwd_dstates   dH_c = dy^T (C*exp(cs))  and  dM = tril(dy x^T)
 //   k_state_bwd     reverse inter-chunk recurrence (HBM streaming)
-//   k_bwd_chunk     per (chunk, group, 32-column slice), looping over the heads of the
+//   k_bwd_chunk     per (chunk, group, 64-column slice), looping over the heads of the
 //                   group: ddt, dB, dC and the per-unit partial sums of dA / ddt_bias
 //   k_bwd_dx        dx and the per-unit partial sums of dD
-//   k_bwd_reduce    fixed-order sums of the partials (bit-reproducible, no atomics)
+//   k_colsum ...    fixed-order sums of the partials (bit-reproducible, no atomics)
 //
 // With Bd = B dt', E(l,s) = exp(cs[l]-cs[s]) and per state column n
 //   Q[m] = sum_p x[m,p] dS[p],  R[l] = sum_p dy[l,p] H[p],
@@ -52,12 +52,12 @@ struct BwdStSmem {
   static constexpr int LDPT = PT * 16 + 4;
   float dys[CS * LDPT];
   float xs[CS * LDPT];
-  float cs[CS * LDN];
-  float ct[CS * LDN];
-  float tot[4 * NS];
 };
 
-template <int PT>
+// dH[p][n] = sum_l dy[l][p] * C[l][n] exp2(cs[l][n]): contraction over rows, so the B operand
+// comes straight from the registers of the column-lane layout; each wave walks its own 16
+// columns of every 64-column slice without any barrier after the dy / x tiles are staged.
+template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __restrict__ dy_ws,
                                                           float* __restrict__ dstates, float* __restrict__ dm) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -65,25 +65,36 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
   SM& s = *reinterpret_cast<SM*>(smem_raw);
   constexpr int LDPT = SM::LDPT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rg = tid >> 6, col = tid & 63;
+  const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
-  const int ppad = PT * 16;
 
-  if (dy_ws) load_lp_tile_ws(p, u, dy_ws, s.dys, ppad, LDPT);
-  else load_lp_tile(p, u, p.dout[u.dir], p.io_dt, s.dys, ppad, LDPT);
-  load_lp_tile(p, u, p.x[u.dir], p.io_dt, s.xs, ppad, LDPT);
+  int n = wave * 16 + cm;
+  bool vn = n < p.N;
+  int prow[16];
+  float raw[16], cv[16];
+  if (dstates) {
+    lane_rows(p, u, g4, vn, prow);
+    lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+    lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+  }
+  {
+    float dv[CS * PT * 16 / NTHREADS], xv[CS * PT * 16 / NTHREADS];
+    dy_load<IOB, PT>(p, u, dy_ws, dv);
+    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    lp_store<PT>(dv, s.dys, LDPT);
+    lp_store<PT>(xv, s.xs, LDPT);
+  }
   __syncthreads();
 
   if (dm) {
     float* m = dm + sq_off(p, u.bt, u.c, u.h);
-    const int cm = lane & 15, g = lane >> 4;
     for (int j = 0; j <= wave; ++j) {
       f4 acc = {0, 0, 0, 0};
 #pragma unroll
-      for (int kb = 0; kb < ppad; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
+      for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int l = wave * 16 + 4 * g + r, sc = j * 16 + cm;
+        const int l = wave * 16 + 4 * g4 + r, sc = j * 16 + cm;
         m[l * CS + sc] = sc <= l ? acc[r] : 0.0f;
       }
     }
@@ -91,38 +102,39 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
   if (!dstates) return;
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
-    float pre[16];
-    prep_slice<NS>(p, u, n0, s.cs, s.ct, s.tot, pre);
+    float ct[16];
     {
-      const int n = n0 + col;
-      const TensorD& tc = p.Cm[u.dir];
-      const long cb = (long)u.b * tc.s0 + (long)u.g * tc.s2 + n;
+      float dtp[16], cs[16], dummy[16];
+      lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int l = rg * 16 + i, tt = u.c * CS + l;
-        const bool v = (n < p.N) && (tt < p.L);
-        const float cv = v ? ldv(tc.ptr, cb + (long)phys_row(p, u.dir, tt) * tc.s1, p.io_dt) : 0.0f;
-        s.ct[l * LDN + col] = cv * ex2(s.cs[l * LDN + col]);
-      }
+      for (int k = 0; k < 16; ++k) ct[k] = cv[k] * ex2(cs[k]);
     }
-    __syncthreads();
+    const int n_cur = n;
+    const bool vn_cur = vn;
+    if (n0 + NS < p.N) {
+      n = n0 + NS + wave * 16 + cm;
+      vn = n < p.N;
+      lane_rows(p, u, g4, vn, prow);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+    }
     f4 acc[PT];
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
 #pragma unroll
-    for (int kb = 0; kb < CS; kb += 16)
+    for (int k = 0; k < 16; ++k) {
+      const float* yr = s.dys + lane_row(k, g4) * LDPT + cm;
 #pragma unroll
-      for (int pt = 0; pt < PT; ++pt) mma16_kk(acc[pt], s.dys, LDPT, pt * 16, s.ct, LDN, wave * 16, kb, lane);
-    const int n = n0 + wave * 16 + (lane & 15);
+      for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(yr[pt * 16], ct[k], acc[pt]);
+    }
     float* dst = dstates + dst_off(p, u.bt, u.c, u.h);
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int pp = pt * 16 + 4 * (lane >> 4) + r;
-        if (pp < p.P && n < p.N) dst[(long)pp * p.N + n] = acc[pt][r];
+        const int pp = pt * 16 + 4 * g4 + r;
+        if (pp < p.P && vn_cur) dst[(long)pp * p.N + n_cur] = acc[pt][r];
       }
-    __syncthreads();
   }
 }
 
@@ -144,6 +156,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
   const int b = bt / p.ndir, dir = bt % p.ndir;
   const int tid = threadIdx.x, pg = tid >> 4, nq = tid & 15;
   const int n = ns * 64 + nq * 4;
+  const bool vec = ((p.N & 3) == 0) && (n + 3 < p.N);
   float carry[4][4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
@@ -156,22 +169,45 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
   }
   for (int c = p.nc - 1; c >= 0; --c) {
     float gp[4] = {0, 0, 0, 0};
-    float dec[4];
+    float dec[4], hn[4][4], dh[4][4];
+    // issue every load of this chunk before the dependent arithmetic
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dec[j] = n + j < p.N ? __expf(cs_last[vec_off(p, bt, c, h) + n + j]) : 0.0f;
+    for (int j = 0; j < 4; ++j) dec[j] = n + j < p.N ? cs_last[vec_off(p, bt, c, h) + n + j] : 0.0f;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int pp = pg + 16 * k;
-      if (pp >= p.P) continue;
-      const float* hn = states + st_off(p, bt, c + 1, h) + (long)pp * p.N + n;
+      const float* hp = states + st_off(p, bt, c + 1, h) + (long)pp * p.N + n;
+      const float* dd = dstates + dst_off(p, bt, c, h) + (long)pp * p.N + n;
+      if (vec && pp < p.P) {
+        const f4 a = *(const f4*)hp, d = *(const f4*)dd;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { hn[k][j] = a[j]; dh[k][j] = d[j]; }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool v = pp < p.P && n + j < p.N;
+          hn[k][j] = v ? hp[j] : 0.0f;
+          dh[k][j] = v ? dd[j] : 0.0f;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dec[j] = __expf(dec[j]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int pp = pg + 16 * k;
       float* dd = dstates + dst_off(p, bt, c, h) + (long)pp * p.N + n;
+      if (vec && pp < p.P) {
+        *(f4*)dd = (f4){carry[k][0], carry[k][1], carry[k][2], carry[k][3]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (pp < p.P && n + j < p.N) dd[j] = carry[k][j];
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (n + j >= p.N) continue;
-        const float dh = dd[j];
-        dd[j] = carry[k][j];
-        gp[j] += hn[j] * carry[k][j];
-        carry[k][j] = dec[j] * carry[k][j] + dh;
+        gp[j] += hn[k][j] * carry[k][j];
+        carry[k][j] = dec[j] * carry[k][j] + dh[k][j];
       }
     }
 #pragma unroll
@@ -196,26 +232,112 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 }
 
 // -------------------------------------------------------------- chunk backward
+// Workgroup = (batch, chunk, group, 64 state columns) of one direction, looping over the heads of
+// the group.  Column-lane layout: cumulative sums, decays, level operands, E1, X2 and the suffix
+// sums live in registers of one lane; only x, dy and dM (shared by the four waves) go through LDS.
 template <int PT>
 struct BwdChunkSmem {
   static constexpr int LDPT = PT * 16 + 4;
-  float cs[CS * LDNB];
-  float dts[CS * LDNB];
-  float bs[CS * LDNB];
-  float ccs[CS * LDNB];
-  float opa[CS * LDNB];  // level operand Bw, later E1
-  float opb[CS * LDNB];  // level operand Cw, later X2
   float xs[CS * LDPT];
   float dys[CS * LDPT];
   float dms[CS * LDC];
-  float dss[PT * 16 * LDNB];
-  float hs[PT * 16 * LDNB];
-  float tot[8 * NSB];
-  float red[2 * 8 * NSB];
 };
 
-// partials: partA (Bt*nc, H, N) then partBias (Bt*nc, H, N)
-template <int PT>
+// One level (w = 2^LV) of the row hierarchy for F and G.  op[k] = Bd * exp2(ref - cs) on lower
+// rows (right factor of the decay), C * exp2(cs - ref) on upper rows (left factor); ref = cs of
+// the last row of the lower half of the row's 2w-block, fetched from the lane that owns it.  Rows
+// that are upper at this level receive their F contribution (x2), lower rows their G
+// contribution (e1).
+template <int LV>
+__device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
+                                          const float* __restrict__ dms, f4 (&e1)[4], f4 (&x2)[4], int cm, int g4) {
+  constexpr int w = 1 << LV;
+  float op[16], ee[16];
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    float r01, r23;
+    if (LV == 0) { r01 = cs[4 * J]; r23 = cs[4 * J + 2]; }
+    else if (LV == 1) r01 = r23 = cs[4 * J + 1];
+    else if (LV == 2) r01 = r23 = __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64);
+    else if (LV == 3) r01 = r23 = __shfl(cs[4 * J + 3], cm + 16, 64);
+    else if (LV == 4) r01 = r23 = __shfl(cs[4 * (J & 2) + 3], cm + 48, 64);
+    else r01 = r23 = __shfl(cs[7], cm + 48, 64);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * J + j;
+      const bool upper = LV == 0 ? (j & 1) : LV == 1 ? (j & 2) : LV == 2 ? (g4 & 1) : LV == 3 ? (g4 & 2)
+                                                                            : LV == 4 ? (J & 1) : (J & 2);
+      const float ref = j < 2 ? r01 : r23;
+      const float e = ex2(upper ? cs[k] - ref : ref - cs[k]);
+      ee[k] = e;
+      op[k] = (upper ? Cv[k] : Bd[k]) * e;
+    }
+  }
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    f4 acc = {0, 0, 0, 0};
+    if (LV == 5) {
+      if (I >= 2) {  // F: rows of tiles 2,3 gather from the lower rows s in tiles 0,1
+#pragma unroll
+        for (int J = 0; J < 2; ++J) {
+          const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + J * 16 + 4 * g4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc = mfma4(av[j], op[4 * J + j], acc);
+        }
+      } else {  // G: rows of tiles 0,1 gather from the upper rows l in tiles 2,3
+#pragma unroll
+        for (int J = 2; J < 4; ++J) {
+          const float* ap = dms + (J * 16 + 4 * g4) * LDC + I * 16 + cm;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc = mfma4(ap[j * LDC], op[4 * J + j], acc);
+        }
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        if (I >= 2) x2[I][rr] += ee[4 * I + rr] * acc[rr];
+        else e1[I][rr] += ee[4 * I + rr] * acc[rr];
+      }
+    } else if (LV == 4) {
+      if (I & 1) {
+        const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + (I - 1) * 16 + 4 * g4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mfma4(av[j], op[4 * (I - 1) + j], acc);
+      } else {
+        const float* ap = dms + ((I + 1) * 16 + 4 * g4) * LDC + I * 16 + cm;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mfma4(ap[j * LDC], op[4 * (I + 1) + j], acc);
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        if (I & 1) x2[I][rr] += ee[4 * I + rr] * acc[rr];
+        else e1[I][rr] += ee[4 * I + rr] * acc[rr];
+      }
+    } else {
+      // inside the diagonal tile: contraction rows kr = 4 g4 + j, restricted to the 2w-block of the
+      // output row (lane cm); lower rows feed F, upper rows feed G
+      f4 gw = {0, 0, 0, 0};
+      const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + I * 16 + 4 * g4);
+      const float* ap = dms + (I * 16 + 4 * g4) * LDC + I * 16 + cm;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kr = 4 * g4 + j;
+        const bool same = LV == 3 || ((cm ^ kr) < 2 * w);
+        const bool kup = (kr >> LV) & 1;
+        acc = mfma4((same && !kup) ? av[j] : 0.0f, op[4 * I + j], acc);
+        gw = mfma4((same && kup) ? ap[j * LDC] : 0.0f, op[4 * I + j], gw);
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const bool upper = ((4 * g4 + rr) >> LV) & 1;
+        if (upper) x2[I][rr] += ee[4 * I + rr] * acc[rr];
+        else e1[I][rr] += ee[4 * I + rr] * gw[rr];
+      }
+    }
+  }
+}
+
+// partA, partBias: (Bt*nc, H, N) per-unit partial sums of dA and ddt_bias
+template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws,
                                                         const float* __restrict__ states,
                                                         const float* __restrict__ dstates,
@@ -226,226 +348,170 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __res
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
   constexpr int LDPT = SM::LDPT;
+  constexpr int KP_ = PT * 4;  // dS / H values per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rg = tid >> 5, col = tid & 31;  // column-thread layout: rows 8rg..8rg+7
   const int cm = lane & 15, g4 = lane >> 4;
-  const int ppad = PT * 16;
-  const int nsl = (p.N + NSB - 1) / NSB;
+  const int nsl = (p.N + NS - 1) / NS;
   Unit u;
-  {
-    int id = xcd_remap(blockIdx.x, gridDim.x);
-    const int ns = id % nsl;
-    id /= nsl;
-    u.g = id % p.G;
-    id /= p.G;
-    u.c = id % p.nc;
-    u.b = id / p.nc;
-    u.dir = p.dir0;
-    u.bt = u.b * p.ndir + u.dir;
-    u.h = 0;
-    const int n0 = ns * NSB;
-    const int n = n0 + col;
-    const bool vn = n < p.N;
+  int id = xcd_remap(blockIdx.x, gridDim.x);
+  const int ns = id % nsl;
+  id /= nsl;
+  u.g = id % p.G;
+  id /= p.G;
+  u.c = id % p.nc;
+  u.b = id / p.nc;
+  u.dir = p.dir0;
+  u.bt = u.b * p.ndir + u.dir;
+  u.h = u.g * p.hpg;
+  const int n = ns * NS + wave * 16 + cm;
+  const bool vn = n < p.N;
 
-    load_ln_tile<NSB>(p, u, p.Bm[u.dir], p.io_dt, u.g, n0, s.bs);
-    load_ln_tile<NSB>(p, u, p.Cm[u.dir], p.io_dt, u.g, n0, s.ccs);
-    float dBacc[8], dCacc[8];
+  int prow[16];
+  lane_rows(p, u, g4, vn, prow);
+  float Bv[16], Cv[16];
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, Bv);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, Cv);
+  float dBacc[16], dCacc[16];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dBacc[i] = dCacc[i] = 0.0f;
+  for (int k = 0; k < 16; ++k) dBacc[k] = dCacc[k] = 0.0f;
+  int oddt[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) oddt[k] = (prow[k] < 0 || !p.ddt.ptr) ? -1 : prow[k] * (int)p.ddt.s1 + n;
 
-    for (int hh = 0; hh < p.hpg; ++hh) {
-      u.h = u.g * p.hpg + hh;
-      float pre[8];
-      prep_slice<NSB>(p, u, n0, s.cs, s.dts, s.tot, pre);
-      if (dy_ws) load_lp_tile_ws(p, u, dy_ws, s.dys, ppad, LDPT);
-      else load_lp_tile(p, u, p.dout[u.dir], p.io_dt, s.dys, ppad, LDPT);
-      load_lp_tile(p, u, p.x[u.dir], p.io_dt, s.xs, ppad, LDPT);
-      {
-        const float* m = dm + sq_off(p, u.bt, u.c, u.h);
-        for (int e = tid; e < CS * CS; e += NTHREADS) {
-          const int l = e >> 6, sc = e & 63;
-          s.dms[l * LDC + sc] = sc <= l ? m[e] : 0.0f;
-        }
-        const float* ds = dstates + dst_off(p, u.bt, u.c, u.h);
-        const float* hp = states + st_off(p, u.bt, u.c, u.h);
-        for (int e = tid; e < ppad * NSB; e += NTHREADS) {
-          const int pp = e >> 5, c2 = e & 31;
-          const bool v = pp < p.P && n0 + c2 < p.N;
-          s.dss[pp * LDNB + c2] = v ? ds[(long)pp * p.N + n0 + c2] : 0.0f;
-          s.hs[pp * LDNB + c2] = v ? hp[(long)pp * p.N + n0 + c2] : 0.0f;
-        }
+  for (int hh = 0; hh < p.hpg; ++hh) {
+    u.h = u.g * p.hpg + hh;
+    // ---- global loads of this head
+    float raw[16], dsv[KP_], hv[KP_], old[16];
+    lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+    {
+      int os[KP_];
+#pragma unroll
+      for (int q = 0; q < KP_; ++q) {
+        const int pp = 16 * (q >> 2) + 4 * g4 + (q & 3);
+        os[q] = (vn && pp < p.P) ? pp * p.N + n : -1;
       }
-      __syncthreads();
+      gload<false, KP_>(dstates, dst_off(p, u.bt, u.c, u.h), os, dsv);
+      gload<false, KP_>(states, st_off(p, u.bt, u.c, u.h), os, hv);
+    }
+    const long ddt_base = (long)u.b * p.ddt.s0 + (long)u.h * p.ddt.s2;
+    if (p.dir0 > 0) gload<DTB, 16>(p.ddt.ptr, ddt_base, oddt, old);
+    {
+      float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
+      f4 mv[4];
+      dy_load<IOB, PT>(p, u, dy_ws, dv);
+      lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+      tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv);
+      __syncthreads();  // the previous head no longer reads the LDS tiles
+      lp_store<PT>(dv, s.dys, LDPT);
+      lp_store<PT>(xv, s.xs, LDPT);
+      tril_store(mv, s.dms);
+    }
+    __syncthreads();
 
-      // Q, R and the diagonal (l == s) terms, in accumulator layout: wave owns rows 16*wave..+15
-      f4 e1[2], x2[2];
+    // ---- dt transform and running sum down the chunk (log2 domain)
+    const float An = vn ? p.A[u.h * p.N + n] : 0.0f;
+    float dtp[16], cs[16], dfac[16];
+    const float last = lane_prep<true>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dfac);
+    float Bd[16];
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
-#pragma unroll
-        for (int kb = 0; kb < ppad; kb += 16) {
-          mma16_mk(q, s.xs, LDPT, wave * 16, s.dss, LDNB, nt * 16, kb, lane);
-          mma16_mk(r, s.dys, LDPT, wave * 16, s.hs, LDNB, nt * 16, kb, lane);
-        }
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int row = wave * 16 + 4 * g4 + rr, cx = nt * 16 + cm;
-          const float cl = s.cs[row * LDNB + cx], last = s.cs[63 * LDNB + cx];
-          const float dd = s.dms[row * LDC + row];
-          e1[nt][rr] = ex2(last - cl) * q[rr] + dd * s.ccs[row * LDNB + cx];
-          x2[nt][rr] = ex2(cl) * r[rr] + dd * s.bs[row * LDNB + cx] * s.dts[row * LDNB + cx];
-        }
-      }
+    for (int k = 0; k < 16; ++k) Bd[k] = Bv[k] * dtp[k];
 
-      // hierarchy levels of F and G
+    // ---- Q, R, diagonal terms.  e1 / x2 [I][r] <-> row 16I + 4 g4 + r <-> index k = 4I + r
+    f4 e1[4], x2[4];
 #pragma unroll
-      for (int lv = 5; lv >= 0; --lv) {
-        const int w = 1 << lv;
-        __syncthreads();
+    for (int I = 0; I < 4; ++I) {
+      f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int l = rg * 8 + i;
-          const int ref = (l & ~(2 * w - 1)) + w - 1;
-          const float cr = s.cs[ref * LDNB + col], cl = s.cs[l * LDNB + col];
-          const bool upper = (l & w) != 0;
-          const float e = ex2(upper ? cl - cr : cr - cl);
-          s.opa[l * LDNB + col] = upper ? 0.0f : s.bs[l * LDNB + col] * s.dts[l * LDNB + col] * e;
-          s.opb[l * LDNB + col] = upper ? s.ccs[l * LDNB + col] * e : 0.0f;
-        }
-        __syncthreads();
-        const int I = wave;
-        // F: rows of this tile that are "upper" at this level; K runs over s
-        int fk0 = 0, fk1 = 0, gk0 = 0, gk1 = 0;
-        if (lv == 5) {
-          if (I >= 2) { fk0 = 0; fk1 = 32; } else { gk0 = 32; gk1 = 64; }
-        } else if (lv == 4) {
-          if (I & 1) { fk0 = 16 * (I - 1); fk1 = 16 * I; } else { gk0 = 16 * (I + 1); gk1 = 16 * (I + 2); }
-        } else {
-          fk0 = gk0 = 16 * I;
-          fk1 = gk1 = 16 * I + 16;
-        }
+      for (int kb = 0; kb < PT; ++kb) {
+        const f4 ax = *(const f4*)(s.xs + (I * 16 + cm) * LDPT + kb * 16 + 4 * g4);
+        const f4 ay = *(const f4*)(s.dys + (I * 16 + cm) * LDPT + kb * 16 + 4 * g4);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          f4 fw = {0, 0, 0, 0}, gw = {0, 0, 0, 0};
-          for (int kb = fk0; kb < fk1; kb += 16) {
-            // A = dM[l][s] (M-major), B = Bw[s][n] (K-major)
-            f4 av = *(const f4*)(s.dms + (I * 16 + cm) * LDC + kb + 4 * g4);
-            if (lv < 3) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if (((cm ^ (4 * g4 + j)) >= 2 * w)) av[j] = 0.0f;
-            }
-            const float* bp = s.opa + (kb + 4 * g4) * LDNB + nt * 16 + cm;
-            fw = mfma4(av.x, bp[0], fw);
-            fw = mfma4(av.y, bp[LDNB], fw);
-            fw = mfma4(av.z, bp[2 * LDNB], fw);
-            fw = mfma4(av.w, bp[3 * LDNB], fw);
-          }
-          for (int kb = gk0; kb < gk1; kb += 16) {
-            // A[m][k=l] = dM[l][m] (K-major), B = Cw[l][n] (K-major)
-            const float* ap = s.dms + (kb + 4 * g4) * LDC + I * 16 + cm;
-            const float* bp = s.opb + (kb + 4 * g4) * LDNB + nt * 16 + cm;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              float a = ap[j * LDC];
-              if (lv < 3 && ((cm ^ (4 * g4 + j)) >= 2 * w)) a = 0.0f;
-              gw = mfma4(a, bp[j * LDNB], gw);
-            }
-          }
-#pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            const int row = wave * 16 + 4 * g4 + rr, cx = nt * 16 + cm;
-            const int ref = (row & ~(2 * w - 1)) + w - 1;
-            const float cr = s.cs[ref * LDNB + cx], cl = s.cs[row * LDNB + cx];
-            if (row & w) x2[nt][rr] += ex2(cl - cr) * fw[rr];
-            else e1[nt][rr] += ex2(cr - cl) * gw[rr];
-          }
+        for (int j = 0; j < 4; ++j) {
+          q = mfma4(ax[j], dsv[4 * kb + j], q);
+          r = mfma4(ay[j], hv[4 * kb + j], r);
         }
       }
-      __syncthreads();
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int row = wave * 16 + 4 * g4 + rr, cx = nt * 16 + cm;
-          s.opa[row * LDNB + cx] = e1[nt][rr];
-          s.opb[row * LDNB + cx] = x2[nt][rr];
-        }
-      __syncthreads();
-
-      // column phase: thread owns rows 8rg..8rg+7 of column col
-      float ddtp[8], dcs[8], dv[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int l = rg * 8 + i;
-        const float E1 = s.opa[l * LDNB + col], X2 = s.opb[l * LDNB + col];
-        const float b = s.bs[l * LDNB + col], c = s.ccs[l * LDNB + col], d = s.dts[l * LDNB + col];
-        dv[i] = d;
-        dBacc[i] += d * E1;
-        dCacc[i] += X2;
-        ddtp[i] = b * E1;
-        dcs[i] = c * X2 - b * d * E1;
+      for (int rr = 0; rr < 4; ++rr) {
+        const int k = 4 * I + rr, row = 16 * I + 4 * g4 + rr;
+        const float dd = s.dms[row * LDC + row];
+        e1[I][rr] = ex2(last - cs[k]) * q[rr] + dd * Cv[k];
+        x2[I][rr] = ex2(cs[k]) * r[rr] + dd * Bd[k];
       }
-      if (rg == 7 && vn) dcs[7] += g_last[vec_off(p, u.bt, u.c, u.h) + n];
-      float run = 0.0f;
-#pragma unroll
-      for (int i = 7; i >= 0; --i) {
-        run += dcs[i];
-        dcs[i] = run;
-      }
-      s.tot[rg * NSB + col] = run;
-      __syncthreads();
-      float off = 0.0f;
-      for (int g = rg + 1; g < 8; ++g) off += s.tot[g * NSB + col];
-      const float An = vn ? p.A[u.h * p.N + n] : 0.0f;
-      float sumA = 0.0f, sumB = 0.0f;
-      const TensorD& tdd = p.ddt;
-      const long dbase = (long)u.b * tdd.s0 + (long)u.h * tdd.s2 + n;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int l = rg * 8 + i, tt = u.c * CS + l;
-        const float da = dcs[i] + off;
-        sumA += da * dv[i];
-        float val = ddtp[i] + da * An;
-        float sp = pre[i];
-        if (p.flags & F_SOFTPLUS) sp = (pre[i] <= 20.0f) ? log1pf(__expf(pre[i])) : pre[i];
-        if (sp < p.dt_min || sp > p.dt_max) val = 0.0f;
-        if ((p.flags & F_SOFTPLUS) && pre[i] <= 20.0f) val *= sigmoidf_(pre[i]);
-        if (vn && tt < p.L) {
-          sumB += val;
-          if (tdd.ptr) {
-            const long o = dbase + (long)phys_row(p, u.dir, tt) * tdd.s1;
-            if (p.dir0 > 0) val += ldv(tdd.ptr, o, p.dt_dt);
-            stv(const_cast<void*>(tdd.ptr), o, p.dt_dt, val);
-          }
-        }
-      }
-      s.red[rg * NSB + col] = sumA;
-      s.red[8 * NSB + rg * NSB + col] = sumB;
-      __syncthreads();
-      if (rg == 0 && vn) {
-        float a = 0.0f, bsum = 0.0f;
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-          a += s.red[g * NSB + col];
-          bsum += s.red[8 * NSB + g * NSB + col];
-        }
-        partA[vec_off(p, u.bt, u.c, u.h) + n] = a;
-        partBias[vec_off(p, u.bt, u.c, u.h) + n] = bsum;
-      }
-      __syncthreads();
     }
 
+    // ---- hierarchy levels of F and G; scheduling barriers keep one level's operands live at a time
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<5>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<4>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<3>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<2>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<1>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_level<0>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- column phase: everything below is local to the lane except the scans over rows
+    float dcs[16], val[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float E1 = e1[k >> 2][k & 3], X2 = x2[k >> 2][k & 3];
+      dBacc[k] += dtp[k] * E1;
+      dCacc[k] += X2;
+      val[k] = Bv[k] * E1;
+      dcs[k] = Cv[k] * X2 - Bd[k] * E1;
+    }
+    if (g4 == 3 && vn) dcs[15] += g_last[vec_off(p, u.bt, u.c, u.h) + n];
+    {
+      float carry = 0.0f;  // sum over all rows after the current tile
+#pragma unroll
+      for (int J = 3; J >= 0; --J) {
+        float c = 0.0f;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          c += dcs[4 * J + j];
+          dcs[4 * J + j] = c;
+        }
+        const float incl = scan_g_incl_rev(c, g4);
+        const float add = carry + (incl - c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dcs[4 * J + j] += add;
+        carry += __shfl(incl, cm, 64);
+      }
+    }
+    float sumA = 0.0f, sumB = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float da = dcs[k];
+      sumA += da * dtp[k];
+      val[k] = (val[k] + da * An) * dfac[k];
+      if (prow[k] >= 0) sumB += val[k];
+      if (p.dir0 > 0) val[k] += old[k];
+    }
+    gstore<DTB, 16>(const_cast<void*>(p.ddt.ptr), ddt_base, oddt, val);
+    sumA = scan_g_incl(sumA, g4);
+    sumB = scan_g_incl(sumB, g4);
+    if (g4 == 3 && vn) {
+      partA[vec_off(p, u.bt, u.c, u.h) + n] = sumA;
+      partBias[vec_off(p, u.bt, u.c, u.h) + n] = sumB;
+    }
+  }
+
+  {
     const TensorD& tB = p.dB[u.dir];
     const TensorD& tC = p.dC[u.dir];
+    int ob[16], oc[16];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int tt = u.c * CS + rg * 8 + i;
-      if (!vn || tt >= p.L) continue;
-      const int pr = phys_row(p, u.dir, tt);
-      if (tB.ptr) stv(const_cast<void*>(tB.ptr), (long)u.b * tB.s0 + (long)pr * tB.s1 + (long)u.g * tB.s2 + n, p.io_dt, dBacc[i]);
-      if (tC.ptr) stv(const_cast<void*>(tC.ptr), (long)u.b * tC.s0 + (long)pr * tC.s1 + (long)u.g * tC.s2 + n, p.io_dt, dCacc[i]);
+    for (int k = 0; k < 16; ++k) {
+      ob[k] = (prow[k] < 0 || !tB.ptr) ? -1 : prow[k] * (int)tB.s1 + n;
+      oc[k] = (prow[k] < 0 || !tC.ptr) ? -1 : prow[k] * (int)tC.s1 + n;
     }
+    gstore<IOB, 16>(const_cast<void*>(tB.ptr), (long)u.b * tB.s0 + (long)u.g * tB.s2, ob, dBacc);
+    gstore<IOB, 16>(const_cast<void*>(tC.ptr), (long)u.b * tC.s0 + (long)u.g * tC.s2, oc, dCacc);
   }
 }
 
@@ -455,14 +521,12 @@ struct BwdDxSmem {
   static constexpr int LDPT = PT * 16 + 4;
   float dys[CS * LDPT];
   float ms[CS * LDC];
-  float cs[CS * LDN];
-  float bt[CS * LDN];
-  float dss[PT * 16 * LDN];
-  float tot[4 * NS];
+  float bt[CS * LDN];       // B dt' exp2(last - cs) [m][n]; later dy*x products
+  float dss[PT * 16 * LDN]; // dS [p][n]
 };
 
 // partD: (Bt*nc*H, P) per-unit sums over rows of dy*x
-template <int PT>
+template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restrict__ dy_ws,
                                                      const float* __restrict__ dstates,
                                                      const float* __restrict__ cabt, float* __restrict__ partD) {
@@ -471,44 +535,47 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   SM& s = *reinterpret_cast<SM*>(smem_raw);
   constexpr int LDPT = SM::LDPT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rg = tid >> 6, col = tid & 63;
+  const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
-  const int ppad = PT * 16;
+  const float* ds = dstates + dst_off(p, u.bt, u.c, u.h);
 
-  if (dy_ws) load_lp_tile_ws(p, u, dy_ws, s.dys, ppad, LDPT);
-  else load_lp_tile(p, u, p.dout[u.dir], p.io_dt, s.dys, ppad, LDPT);
+  int n = wave * 16 + cm;
+  bool vn = n < p.N;
+  int prow[16];
+  lane_rows(p, u, g4, vn, prow);
+  float raw[16], bv[16];
+  PnRegs<PT> sv;
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+  pn_load<PT>(p, ds, 0, sv);
   {
-    const float* m = cabt + sq_off(p, u.bt, u.c, u.h);
-    for (int e = tid; e < CS * CS; e += NTHREADS) {
-      const int l = e >> 6, sc = e & 63;
-      s.ms[l * LDC + sc] = sc <= l ? m[e] : 0.0f;
-    }
+    float dv[CS * PT * 16 / NTHREADS];
+    f4 mv[4];
+    dy_load<IOB, PT>(p, u, dy_ws, dv);
+    tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
+    lp_store<PT>(dv, s.dys, LDPT);
+    tril_store(mv, s.ms);
   }
   f4 acc[PT];
 #pragma unroll
   for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-  const float* ds = dstates + dst_off(p, u.bt, u.c, u.h);
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
-    float pre[16];
-    prep_slice<NS>(p, u, n0, s.cs, s.bt, s.tot, pre);
     {
-      const int n = n0 + col;
-      const TensorD& tb = p.Bm[u.dir];
-      const long bb = (long)u.b * tb.s0 + (long)u.g * tb.s2 + n;
-      const float last = s.cs[63 * LDN + col];
+      float dtp[16], cs[16], dummy[16];
+      const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int l = rg * 16 + i, tt = u.c * CS + l;
-        const bool v = (n < p.N) && (tt < p.L);
-        const float bv = v ? ldv(tb.ptr, bb + (long)phys_row(p, u.dir, tt) * tb.s1, p.io_dt) : 0.0f;
-        s.bt[l * LDN + col] = bv * s.bt[l * LDN + col] * ex2(last - s.cs[l * LDN + col]);
-      }
-      for (int e = tid; e < ppad * NS; e += NTHREADS) {
-        const int pp = e >> 6, c2 = e & 63;
-        const bool v = pp < p.P && n0 + c2 < p.N;
-        s.dss[pp * LDN + c2] = v ? ds[(long)pp * p.N + n0 + c2] : 0.0f;
-      }
+      for (int k = 0; k < 16; ++k)
+        s.bt[lane_row(k, g4) * LDN + wave * 16 + cm] = bv[k] * dtp[k] * ex2(last - cs[k]);
+    }
+    pn_store<PT>(sv, s.dss);
+    if (n0 + NS < p.N) {
+      n = n0 + NS + wave * 16 + cm;
+      vn = n < p.N;
+      lane_rows(p, u, g4, vn, prow);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+      pn_load<PT>(p, ds, n0 + NS, sv);
     }
     __syncthreads();
 #pragma unroll
@@ -524,30 +591,33 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
 
   const TensorD& tx = p.x[u.dir];
   const TensorD& tdx = p.dx[u.dir];
-  float* prod = s.cs;  // reuse: [64][LDN] is at least [64][ppad]
+  float* prod = s.bt;  // [64][LDN] holds at least [64][16 PT]
 #pragma unroll
-  for (int pt = 0; pt < PT; ++pt)
+  for (int pt = 0; pt < PT; ++pt) {
+    int ox[4], odx[4];
+    float xv[4], v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int l = wave * 16 + 4 * (lane >> 4) + r, pp = pt * 16 + (lane & 15);
-      const int tt = u.c * CS + l;
-      float pv = 0.0f;
-      if (tt < p.L && pp < p.P) {
-        const int pr = phys_row(p, u.dir, tt);
-        const float dyv = s.dys[l * LDPT + pp];
-        float v = acc[pt][r];
-        if (p.D) {
-          v += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + pp] : p.D[u.h]) * dyv;
-          pv = dyv * ldv(tx.ptr, (long)u.b * tx.s0 + (long)pr * tx.s1 + (long)u.h * tx.s2 + pp, p.io_dt);
-        }
-        if (tdx.ptr)
-          stv(const_cast<void*>(tdx.ptr), (long)u.b * tdx.s0 + (long)pr * tdx.s1 + (long)u.h * tdx.s2 + pp, p.io_dt, v);
-      }
-      prod[l * LDN + pp] = pv;
+      const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm, tt = u.c * CS + l;
+      const bool ok = tt < p.L && pp < p.P;
+      const int pr = ok ? phys_row(p, u.dir, tt) : 0;
+      ox[r] = (ok && p.D) ? pr * (int)tx.s1 + pp : -1;
+      odx[r] = (ok && tdx.ptr) ? pr * (int)tdx.s1 + pp : -1;
     }
+    gload<IOB, 4>(tx.ptr, (long)u.b * tx.s0 + (long)u.h * tx.s2, ox, xv);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm;
+      const float dyv = s.dys[l * LDPT + pp];
+      v[r] = acc[pt][r];
+      if (p.D) v[r] += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + (pp < p.P ? pp : 0)] : p.D[u.h]) * dyv;
+      prod[l * LDN + pp] = dyv * xv[r];
+    }
+    gstore<IOB, 4>(const_cast<void*>(tdx.ptr), (long)u.b * tdx.s0 + (long)u.h * tdx.s2, odx, v);
+  }
   if (p.D && partD) {
     __syncthreads();
-    if (tid < ppad) {
+    if (tid < PT * 16) {
       float sum = 0.0f;
       for (int l = 0; l < CS; ++l) sum += prod[l * LDN + tid];
       if (tid < p.P) partD[(((long)u.bt * p.nc + u.c) * p.H + u.h) * p.P + tid] = sum;
@@ -556,56 +626,65 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
 }
 
 // ------------------------------------------------------------------- reductions
-// dA[h,n] = sum_j partA[j,h,n];  ddt_bias likewise;  dD[h(,p)] = sum_j partD[j,h,p];
-// dh0 = sum over directions.  One thread per output element, fixed summation order.
-__global__ __launch_bounds__(NTHREADS) void k_bwd_reduce(KP p, const float* __restrict__ partA,
-                                                         const float* __restrict__ partBias,
-                                                         const float* __restrict__ partD,
-                                                         const float* __restrict__ dh0_dir, float* __restrict__ dA,
-                                                         float* __restrict__ dbias, float* __restrict__ dD,
-                                                         float* __restrict__ dh0) {
-  const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
-  const long nHN = (long)p.H * p.N;
-  const int J = p.B * p.ndir * p.nc;
-  const long nD = (p.flags & F_D_HDIM) ? (long)p.H * p.P : p.H;
-  const long nS = (long)p.B * p.H * p.P * p.N;
-  if (id < nHN) {
-    if (dA) {
-      float a = 0.0f;
-      for (int j = 0; j < J; ++j) a += partA[(long)j * nHN + id];
-      dA[id] = a;
+// Column sums of a (J, ncols) fp32 matrix in a fixed order (bit-reproducible, no atomics):
+// block = 32 columns x 8 row groups; row group g adds rows g, g+8, ... and the 8 group sums are
+// combined in order.
+__global__ __launch_bounds__(NTHREADS) void k_colsum(const float* __restrict__ src, int J, int ncols,
+                                                     float* __restrict__ dst) {
+  __shared__ float red[8 * 32];
+  const int c = blockIdx.x * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  if (c < ncols) {
+    int j = g;
+    for (; j + 24 < J; j += 32) {
+      a0 += src[(long)j * ncols + c];
+      a1 += src[(long)(j + 8) * ncols + c];
+      a2 += src[(long)(j + 16) * ncols + c];
+      a3 += src[(long)(j + 24) * ncols + c];
     }
-    if (dbias) {
-      float a = 0.0f;
-      for (int j = 0; j < J; ++j) a += partBias[(long)j * nHN + id];
-      dbias[id] = a;
-    }
+    for (; j < J; j += 8) a0 += src[(long)j * ncols + c];
   }
-  if (id < nD && dD) {
-    float a = 0.0f;
-    if (p.flags & F_D_HDIM) {
-      for (int j = 0; j < J; ++j) a += partD[(long)j * p.H * p.P + id];
-    } else {
-      for (int j = 0; j < J; ++j)
-        for (int pp = 0; pp < p.P; ++pp) a += partD[((long)j * p.H + id) * p.P + pp];
-    }
-    dD[id] = a;
-  }
-  if (id < nS && dh0) {
-    float a = dh0_dir[id];
-    if (p.ndir > 1) a += dh0_dir[nS + id];
-    dh0[id] = a;
+  red[threadIdx.x] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (g == 0 && c < ncols) {
+    float t = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += red[k * 32 + (threadIdx.x & 31)];
+    dst[c] = t;
   }
 }
 
-// -------------------------------------------------------------------- launchers
-#define ISSM_PT_SWITCH(pt, STMT) \
-  switch (pt) {                  \
-    case 1: { constexpr int PT_ = 1; STMT; } break; \
-    case 2: { constexpr int PT_ = 2; STMT; } break; \
-    case 3: { constexpr int PT_ = 3; STMT; } break; \
-    default: { constexpr int PT_ = 4; STMT; } break; \
+// dD[h] = sum over units and p of partD[(j*H + h)*P + p]: one block per head.
+__global__ __launch_bounds__(NTHREADS) void k_dd_scalar(const float* __restrict__ partD, int J, int H, int P,
+                                                        float* __restrict__ dD) {
+  __shared__ float red[NTHREADS];
+  const int h = blockIdx.x;
+  float a = 0.0f;
+  for (int e = threadIdx.x; e < J * P; e += NTHREADS) a += partD[((long)(e / P) * H + h) * P + (e % P)];
+  red[threadIdx.x] = a;
+  __syncthreads();
+  for (int o = NTHREADS / 2; o > 0; o >>= 1) {
+    if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+    __syncthreads();
   }
+  if (threadIdx.x == 0) dD[h] = red[0];
+}
+
+// dh0 = sum over directions of dh0_dir
+__global__ __launch_bounds__(NTHREADS) void k_dh0(const float* __restrict__ dh0_dir, long n, int ndir,
+                                                  float* __restrict__ dh0) {
+  const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (id >= n) return;
+  float a = dh0_dir[id];
+  if (ndir > 1) a += dh0_dir[n + id];
+  dh0[id] = a;
+}
+
+// -------------------------------------------------------------------- launchers
+template <typename K>
+static int set_lds(K kernel, size_t bytes) {
+  return (int)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
 
 int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t st) {
   const long total = (long)p.B * p.ndir * p.L * p.H * p.P;
@@ -616,11 +695,10 @@ int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t s
 
 int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* dm, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  const int pt = (p.P + 15) / 16;
-  ISSM_PT_SWITCH(pt, {
+  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
     const size_t sm = sizeof(BwdStSmem<PT_>);
-    { hipError_t e_ = hipFuncSetAttribute((const void*)k_bwd_dstates<PT_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm); if (e_ != hipSuccess) return (int)e_; }
-    hipLaunchKernelGGL(k_bwd_dstates<PT_>, dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
+    if (int e = set_lds(k_bwd_dstates<PT_, IOB_, DTB_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_dstates<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
   });
   return (int)hipGetLastError();
 }
@@ -634,13 +712,12 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
 
 int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
                      const float* g_last, float* partA, float* partBias, hipStream_t st) {
-  const int blocks = p.B * p.nc * p.G * ((p.N + NSB - 1) / NSB);
-  const int pt = (p.P + 15) / 16;
-  ISSM_PT_SWITCH(pt, {
+  const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
+  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
     const size_t sm = sizeof(BwdChunkSmem<PT_>);
-    { hipError_t e_ = hipFuncSetAttribute((const void*)k_bwd_chunk<PT_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm); if (e_ != hipSuccess) return (int)e_; }
-    hipLaunchKernelGGL(k_bwd_chunk<PT_>, dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last,
-                       partA, partBias);
+    if (int e = set_lds(k_bwd_chunk<PT_, IOB_, DTB_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk<PT_, IOB_, DTB_>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
+                       dm, g_last, partA, partBias);
   });
   return (int)hipGetLastError();
 }
@@ -648,24 +725,31 @@ int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const
 int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const float* cabt, float* partD,
                   hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  const int pt = (p.P + 15) / 16;
-  ISSM_PT_SWITCH(pt, {
+  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
     const size_t sm = sizeof(BwdDxSmem<PT_>);
-    { hipError_t e_ = hipFuncSetAttribute((const void*)k_bwd_dx<PT_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm); if (e_ != hipSuccess) return (int)e_; }
-    hipLaunchKernelGGL(k_bwd_dx<PT_>, dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
+    if (int e = set_lds(k_bwd_dx<PT_, IOB_, DTB_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_dx<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
   });
   return (int)hipGetLastError();
 }
 
 int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, const float* partD,
                       const float* dh0_dir, float* dA, float* dbias, float* dD, float* dh0, hipStream_t st) {
-  long n = (long)p.H * p.N;
-  const long nS = (long)p.B * p.H * p.P * p.N;
-  if (dh0 && nS > n) n = nS;
-  const long nD = (long)p.H * p.P;
-  if (nD > n) n = nD;
-  hipLaunchKernelGGL(k_bwd_reduce, dim3((unsigned)((n + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st, p, partA,
-                     partBias, partD, dh0_dir, dA, dbias, dD, dh0);
+  const int J = p.B * p.ndir * p.nc;
+  const int nHN = p.H * p.N;
+  if (dA) hipLaunchKernelGGL(k_colsum, dim3((nHN + 31) / 32), dim3(NTHREADS), 0, st, partA, J, nHN, dA);
+  if (dbias) hipLaunchKernelGGL(k_colsum, dim3((nHN + 31) / 32), dim3(NTHREADS), 0, st, partBias, J, nHN, dbias);
+  if (dD) {
+    if (p.flags & F_D_HDIM)
+      hipLaunchKernelGGL(k_colsum, dim3((p.H * p.P + 31) / 32), dim3(NTHREADS), 0, st, partD, J, p.H * p.P, dD);
+    else
+      hipLaunchKernelGGL(k_dd_scalar, dim3(p.H), dim3(NTHREADS), 0, st, partD, J, p.H, p.P, dD);
+  }
+  if (dh0) {
+    const long n = (long)p.B * p.H * p.P * p.N;
+    hipLaunchKernelGGL(k_dh0, dim3((unsigned)((n + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st, dh0_dir, n, p.ndir,
+                       dh0);
+  }
   return (int)hipGetLastError();
 }
 

@@ -2,17 +2,21 @@
 //
 // Tiling conventions used by every kernel in this directory
 //  * one workgroup = 256 threads = 4 wavefronts of 64 lanes;
-//  * time is cut into chunks of CS = 64 tokens, the state dimension into slices of
-//    NS = 64 columns; a "unit" is one (batch*direction, chunk, head);
-//  * every LDS tile is a row-major float array whose leading dimension is
-//    (width + 4): with ld = 4 (mod 8) both fragment access patterns below are free
-//    of bank conflicts;
-//  * matrix products run on v_mfma_f32_16x16x4_f32.  Lane (m = lane & 15,
-//    g = lane >> 4) feeds the j-th of four back-to-back MFMAs with k = kb + 4g + j,
-//    so that an operand stored with k contiguous ("M-major", tile[m][k]) is fetched
-//    with one 128-bit LDS read and an operand stored with m contiguous ("K-major",
-//    tile[k][m]) with four 32-bit reads.  The accumulator register r of that lane
-//    holds element (row = 4g + r, col = m) of the 16x16 result.
+//  * time is cut into chunks of CS = 64 tokens, the state dimension into slices of NS = 64
+//    columns; a "unit" is one (batch*direction, chunk, head);
+//  * every LDS tile is a row-major float array whose leading dimension is (width + 4): with
+//    ld = 4 (mod 8) both fragment access patterns below are free of bank conflicts;
+//  * matrix products run on v_mfma_f32_16x16x4_f32.  Lane (cm = lane & 15, g4 = lane >> 4)
+//    feeds the j-th of four back-to-back MFMAs with k = kb + 4 g4 + j, so that an operand
+//    stored with k contiguous ("M-major", tile[m][k]) is fetched with one 128-bit LDS read and
+//    an operand stored with m contiguous ("K-major", tile[k][m]) with four 32-bit reads.  The
+//    accumulator register r of that lane holds element (row = 4 g4 + r, col = cm) of the
+//    16x16 result;
+//  * "column-lane layout": a wave owns 16 state columns, lane (cm, g4) owns column cm and the
+//    16 chunk rows {16J + 4 g4 + j : J, j = 0..3}, array index k = 4J + j.  A lane then holds
+//    exactly the elements it feeds as the K-major B operand of a product that contracts over
+//    rows, and exactly the accumulator rows it gets back from a product whose output rows are
+//    chunk rows, so cumulative sums, decays and all elementwise work stay in registers.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -20,13 +24,10 @@
 namespace issm {
 
 constexpr int CS = 64;         // tokens per chunk
-constexpr int NS = 64;         // state columns per slice (forward kernels)
+constexpr int NS = 64;         // state columns per slice
 constexpr int LDN = NS + 4;    // leading dimension of [*][NS] tiles
-constexpr int NSB = 32;        // state columns per slice (backward chunk kernel)
-constexpr int LDNB = NSB + 4;
 constexpr int LDC = CS + 4;    // leading dimension of [*][CS] tiles
 constexpr int MAXP = 64;       // largest head dimension built
-constexpr int LDP = MAXP + 4;  // leading dimension of [*][P] tiles
 constexpr int NTHREADS = 256;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
@@ -41,7 +42,7 @@ struct TensorD {
 // Kernel parameter block (passed by value).
 struct KP {
   int B, L, H, P, N, G, ndir, nc, hpg;
-  int dir0;  // first direction handled by this launch (kernels launched per direction)
+  int dir0;  // direction handled by this launch (kernels launched per direction)
   int io_dt, dt_dt, h0_dt;  // 0 = f32, 1 = bf16
   unsigned flags;
   float dt_min, dt_max;
@@ -76,7 +77,6 @@ struct NormP {
   int nblocks;
 };
 
-
 __device__ __forceinline__ float bf16_to_f(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float f) {
   uint32_t u = __float_as_uint(f);
@@ -84,6 +84,7 @@ __device__ __forceinline__ uint16_t f_to_bf16(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
   return (uint16_t)(u >> 16);
 }
+// runtime-dtype element access (used only outside hot loops)
 __device__ __forceinline__ float ldv(const void* p, long i, int dt) {
   return dt ? bf16_to_f(((const uint16_t*)p)[i]) : ((const float*)p)[i];
 }
@@ -92,9 +93,48 @@ __device__ __forceinline__ void stv(void* p, long i, int dt, float v) {
 }
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// softplus as the reference evaluates it: log(exp(x) + 1) for x <= 20, identity above
+__device__ __forceinline__ float softplus_(float x) { return x <= 20.0f ? __logf(1.0f + __expf(x)) : x; }
 
-// Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range
-// of logical ids so that units sharing B/C tiles (the heads of one chunk) share an L2.
+// Batched global loads / stores of one element type: all CNT accesses are issued before any
+// value is consumed.  The address is (uniform element offset ubase) + (per-lane 32-bit element
+// offset off[i]), which lets the compiler keep the base in scalar registers; off[i] < 0 marks an
+// absent element (load: reads as 0, the access itself goes to offset 0; store: skipped).
+template <bool BF, int CNT>
+__device__ __forceinline__ void gload(const void* p, long ubase, const int (&off)[CNT], float (&out)[CNT]) {
+  if (BF) {
+    const uint16_t* q = (const uint16_t*)p + ubase;
+    uint16_t r[CNT];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) r[i] = q[off[i] < 0 ? 0 : off[i]];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) out[i] = off[i] < 0 ? 0.0f : bf16_to_f(r[i]);
+  } else {
+    const float* q = (const float*)p + ubase;
+    float r[CNT];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) r[i] = q[off[i] < 0 ? 0 : off[i]];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) out[i] = off[i] < 0 ? 0.0f : r[i];
+  }
+}
+template <bool BF, int CNT>
+__device__ __forceinline__ void gstore(void* p, long ubase, const int (&off)[CNT], const float (&v)[CNT]) {
+  if (BF) {
+    uint16_t* q = (uint16_t*)p + ubase;
+#pragma unroll
+    for (int i = 0; i < CNT; ++i)
+      if (off[i] >= 0) q[off[i]] = f_to_bf16(v[i]);
+  } else {
+    float* q = (float*)p + ubase;
+#pragma unroll
+    for (int i = 0; i < CNT; ++i)
+      if (off[i] >= 0) q[off[i]] = v[i];
+  }
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
+// ids so that units sharing B/C tiles (the heads of one chunk) share an L2.
 __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
   if (nblocks & 7) return bid;
   return (bid & 7) * (nblocks >> 3) + (bid >> 3);
@@ -136,20 +176,9 @@ __device__ __forceinline__ void mma16_mk(f4& acc, const float* a, int lda, int m
   acc = mfma4(av.z, bp[2 * ldb], acc);
   acc = mfma4(av.w, bp[3 * ldb], acc);
 }
-// A K-major, B M-major
-__device__ __forceinline__ void mma16_km(f4& acc, const float* a, int lda, int m0, const float* b, int ldb,
-                                         int n0, int kb, int lane) {
-  const int m = lane & 15, g = lane >> 4;
-  const float* ap = a + (kb + 4 * g) * lda + m0 + m;
-  f4 bv = *(const f4*)(b + (n0 + m) * ldb + kb + 4 * g);
-  acc = mfma4(ap[0], bv.x, acc);
-  acc = mfma4(ap[lda], bv.y, acc);
-  acc = mfma4(ap[2 * lda], bv.z, acc);
-  acc = mfma4(ap[3 * lda], bv.w, acc);
-}
 
-// Decode a unit id -> (b, dir, c, h); h is fastest so that the heads of one chunk run
-// back to back and share the B/C tiles in cache.
+// Decode a unit id -> (b, dir, c, h); h is fastest so that the heads of one chunk run back to
+// back and share the B/C tiles in cache.
 struct Unit {
   int b, dir, bt, c, h, g;
 };
@@ -167,97 +196,181 @@ __device__ __forceinline__ Unit decode_unit(const KP& p, int u) {
 // physical row of logical time t for a direction
 __device__ __forceinline__ int phys_row(const KP& p, int dir, int t) { return dir ? p.L - 1 - t : t; }
 
-// dt transform of one element (bias -> softplus -> clamp), also returns the
-// pre-activation for the backward masks.
-__device__ __forceinline__ float dt_act(const KP& p, float pre) {
-  float v = pre;
-  if (p.flags & F_SOFTPLUS) v = (pre <= 20.0f) ? log1pf(__expf(pre)) : pre;
-  return fminf(fmaxf(v, p.dt_min), p.dt_max);
+// ---------------------------------------------------------------- column-lane layout helpers
+// chunk row of array index k for lane group g4
+__device__ __forceinline__ int lane_row(int k, int g4) { return 16 * (k >> 2) + 4 * g4 + (k & 3); }
+
+// inclusive prefix / suffix over the four lane groups g4 = 0..3 (lanes cm, cm+16, cm+32, cm+48)
+__device__ __forceinline__ float scan_g_incl(float v, int g4) {
+  float t = __shfl_up(v, 16, 64);
+  if (g4 >= 1) v += t;
+  t = __shfl_up(v, 32, 64);
+  if (g4 >= 2) v += t;
+  return v;
+}
+__device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
+  float t = __shfl_down(v, 16, 64);
+  if (g4 <= 2) v += t;
+  t = __shfl_down(v, 32, 64);
+  if (g4 <= 1) v += t;
+  return v;
 }
 
-// Slice prologue for a slice of NSL (64 or 32) state columns.  Thread (rg = tid / NSL,
-// col = tid % NSL) owns RPT = 64*NSL/256 consecutive rows of column n0+col of one unit.
-// Loads dt, applies the transform, forms the inclusive running sum of dt' * A * log2(e)
-// down the chunk (so decays are exp2 of differences) and leaves
-//   csS[l][col] = running sum (log2 domain),  dtS[l][col] = dt'
-// in LDS (leading dimension NSL+4).  `tot` is a [256/NSL][NSL] scratch.  pre[i] receives
-// dt + bias of the owned rows.  Rows past the end of the sequence and columns past N read
-// as dt' = 0.  Ends with a barrier.
-template <int NSL>
-__device__ __forceinline__ void prep_slice(const KP& p, const Unit& u, int n0, float* csS, float* dtS,
-                                           float* tot, float* pre) {
-  constexpr int RPT = CS * NSL / NTHREADS, LD = NSL + 4;
-  const int tid = threadIdx.x, rg = tid / NSL, col = tid % NSL;
-  const int n = n0 + col;
-  const bool vn = n < p.N;
-  const float A2 = vn ? p.A[u.h * p.N + n] * LOG2E : 0.0f;
-  const float bias = (vn && p.dt_bias) ? p.dt_bias[u.h * p.N + n] : 0.0f;
-  const long base = (long)u.b * p.dt.s0 + (long)u.h * p.dt.s2 + n;
-  float dtp[RPT], cs[RPT], raw[RPT];
+// Physical rows of the lane's 16 chunk rows (or -1 past the end of the sequence / invalid column).
+__device__ __forceinline__ void lane_rows(const KP& p, const Unit& u, int g4, bool vn, int (&prow)[16]) {
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    const int t = u.c * CS + rg * RPT + i;
-    const bool v = vn && t < p.L;
-    raw[i] = v ? ldv(p.dt.ptr, base + (long)phys_row(p, u.dir, t) * p.dt.s1, p.dt_dt) : 0.0f;
+  for (int k = 0; k < 16; ++k) {
+    const int tt = u.c * CS + lane_row(k, g4);
+    prow[k] = (vn && tt < p.L) ? phys_row(p, u.dir, tt) : -1;
   }
-  float run = 0.0f;
+}
+// Lane's 16 values of column n of a (B,L,G|H,N)-shaped tensor.
+template <bool BF>
+__device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third, int n, const int (&prow)[16],
+                                             float (&out)[16]) {
+  int off[16];
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    const int t = u.c * CS + rg * RPT + i;
-    const bool v = vn && t < p.L;
-    pre[i] = raw[i] + bias;
-    dtp[i] = v ? dt_act(p, pre[i]) : 0.0f;
-    run += dtp[i] * A2;
-    cs[i] = run;
-  }
-  tot[rg * NSL + col] = run;
-  __syncthreads();
-  float off = 0.0f;
-  for (int g = 0; g < rg; ++g) off += tot[g * NSL + col];
+  for (int k = 0; k < 16; ++k) off[k] = prow[k] < 0 ? -1 : prow[k] * (int)t.s1 + n;
+  gload<BF, 16>(t.ptr, (long)b * t.s0 + (long)third * t.s2, off, out);
+}
+// dt transform (bias -> softplus -> clamp) of the lane's rows and the inclusive running sum of
+// dt' * A * log2(e) down the chunk (so decays are exp2 of differences).  `raw` holds the loaded
+// dt values.  dfac (if WANT_DFAC) receives d dt' / d dt: the softplus derivative times the clamp
+// mask.  Returns the chunk total (running sum at row 63), the same on all lanes of the column.
+template <bool WANT_DFAC>
+__device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, int cm, int g4,
+                                           const int (&prow)[16], const float (&raw)[16], float (&dtp)[16],
+                                           float (&cs)[16], float (&dfac)[16]) {
+  const float A2 = vn ? p.A[h * p.N + n] * LOG2E : 0.0f;
+  const float bias = (vn && p.dt_bias) ? p.dt_bias[h * p.N + n] : 0.0f;
+  if (p.flags & F_SOFTPLUS) {
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    csS[(rg * RPT + i) * LD + col] = cs[i] + off;
-    dtS[(rg * RPT + i) * LD + col] = dtp[i];
+    for (int k = 0; k < 16; ++k) {
+      const float pre = raw[k] + bias;
+      const float sp = softplus_(pre);
+      dtp[k] = prow[k] < 0 ? 0.0f : fminf(fmaxf(sp, p.dt_min), p.dt_max);
+      if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : (pre <= 20.0f ? sigmoidf_(pre) : 1.0f);
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float sp = raw[k] + bias;
+      dtp[k] = prow[k] < 0 ? 0.0f : fminf(fmaxf(sp, p.dt_min), p.dt_max);
+      if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : 1.0f;
+    }
   }
-  __syncthreads();
+  float carry = 0.0f;
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    float c = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      c += dtp[4 * J + j] * A2;
+      cs[4 * J + j] = c;
+    }
+    const float incl = scan_g_incl(c, g4);
+    const float add = carry + (incl - c);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cs[4 * J + j] += add;
+    carry += __shfl(incl, cm + 48, 64);
+  }
+  return carry;
 }
 
-// Rows of a (B,L,G|H,N)-shaped operand into LDS: dst[l][col] for the 64 rows of the unit's
-// chunk, columns n0..n0+NSL-1 (zero outside the sequence / past N).
-template <int NSL>
-__device__ __forceinline__ void load_ln_tile(const KP& p, const Unit& u, const TensorD& t, int dtype, int third,
-                                             int n0, float* dst) {
-  constexpr int RPT = CS * NSL / NTHREADS, LD = NSL + 4;
-  const int tid = threadIdx.x, rg = tid / NSL, col = tid % NSL;
-  const int n = n0 + col;
-  const long base = (long)u.b * t.s0 + (long)third * t.s2 + n;
+// ------------------------------------------------------------------ cooperative tile loaders
+// The unit's (64 x P) tile of a (B,L,H,P) tensor, zero padded to 16*PT columns: registers, then
+// LDS dst[l][p] (leading dimension ld).  Element e = tid + 256 i is (l, p) = (e / 16PT, e % 16PT).
+template <bool BF, int PT>
+__device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const TensorD& t,
+                                        float (&v)[CS * PT * 16 / NTHREADS]) {
+  constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
+  int off[CNT];
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    const int l = rg * RPT + i, tt = u.c * CS + l;
-    const bool v = (n < p.N) && (tt < p.L);
-    dst[l * LD + col] = v ? ldv(t.ptr, base + (long)phys_row(p, u.dir, tt) * t.s1, dtype) : 0.0f;
+  for (int i = 0; i < CNT; ++i) {
+    const int e = threadIdx.x + i * NTHREADS;
+    const int l = e / PPAD, pp = e % PPAD, tt = u.c * CS + l;
+    off[i] = ((pp < p.P) && (tt < p.L)) ? phys_row(p, u.dir, tt) * (int)t.s1 + pp : -1;
+  }
+  gload<BF, CNT>(t.ptr, (long)u.b * t.s0 + (long)u.h * t.s2, off, v);
+}
+template <int PT>
+__device__ __forceinline__ void lp_store(const float (&v)[CS * PT * 16 / NTHREADS], float* dst, int ld) {
+  constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
+#pragma unroll
+  for (int i = 0; i < CNT; ++i) {
+    const int e = threadIdx.x + i * NTHREADS;
+    dst[(e / PPAD) * ld + (e % PPAD)] = v[i];
+  }
+}
+// dy tile: from the caller's dout (io dtype) or from the gated fp32 (Bt,L,H,P) workspace copy.
+template <bool BF, int PT>
+__device__ __forceinline__ void dy_load(const KP& p, const Unit& u, const float* dy_ws,
+                                        float (&v)[CS * PT * 16 / NTHREADS]) {
+  if (dy_ws) {
+    TensorD t;
+    t.ptr = dy_ws + (long)(u.bt - u.b) * p.L * p.H * p.P;  // so that b * s0 lands on row block bt
+    t.s0 = (long)p.L * p.H * p.P;
+    t.s1 = (long)p.H * p.P;
+    t.s2 = p.P;
+    lp_load<false, PT>(p, u, t, v);
+  } else {
+    lp_load<BF, PT>(p, u, p.dout[u.dir], v);
   }
 }
 
-// The unit's (64 x P) tile of a (B,L,H,P) tensor into LDS dst[l][p] (leading dimension ld),
-// zero padded to ppad columns.
-__device__ __forceinline__ void load_lp_tile(const KP& p, const Unit& u, const TensorD& t, int dtype, float* dst,
-                                             int ppad, int ld) {
-  const long base = (long)u.b * t.s0 + (long)u.h * t.s2;
-  for (int e = threadIdx.x; e < CS * ppad; e += NTHREADS) {
-    const int l = e / ppad, pp = e - l * ppad, tt = u.c * CS + l;
-    const bool v = (pp < p.P) && (tt < p.L);
-    dst[l * ld + pp] = v ? ldv(t.ptr, base + (long)phys_row(p, u.dir, tt) * t.s1 + pp, dtype) : 0.0f;
+// Lower triangle (s <= l, rest zero) of a 64x64 fp32 block: registers, then LDS dst[l][s] (ld = LDC).
+__device__ __forceinline__ void tril_load(const float* __restrict__ src, f4 (&v)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = threadIdx.x + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
+    v[i] = (s4 <= l) ? *(const f4*)(src + l * CS + s4) : (f4){0, 0, 0, 0};
   }
 }
-// Same for an fp32 contiguous (Bt,L,H,P) workspace tensor stored in physical time order.
-__device__ __forceinline__ void load_lp_tile_ws(const KP& p, const Unit& u, const float* src, float* dst, int ppad,
-                                                int ld) {
-  const long base = ((long)u.bt * p.L) * p.H * p.P + (long)u.h * p.P;
-  for (int e = threadIdx.x; e < CS * ppad; e += NTHREADS) {
-    const int l = e / ppad, pp = e - l * ppad, tt = u.c * CS + l;
-    const bool v = (pp < p.P) && (tt < p.L);
-    dst[l * ld + pp] = v ? src[base + (long)phys_row(p, u.dir, tt) * p.H * p.P + pp] : 0.0f;
+__device__ __forceinline__ void tril_store(const f4 (&v)[4], float* dst) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = threadIdx.x + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
+    f4 w = v[i];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s4 + j > l) w[j] = 0.0f;
+    *(f4*)(dst + l * LDC + s4) = w;
+  }
+}
+
+// Columns n0..n0+63 of a (P x N) fp32 slab, zero padded to 16*PT rows and past N: registers, then
+// LDS dst[p][col] (leading dimension LDN).
+template <int PT>
+struct PnRegs {
+  static constexpr int Q = NS / 4, TOT = PT * 16 * Q, CNT = (TOT + NTHREADS - 1) / NTHREADS;
+  f4 v[CNT];
+};
+template <int PT>
+__device__ __forceinline__ void pn_load(const KP& p, const float* __restrict__ src, int n0, PnRegs<PT>& r) {
+  typedef PnRegs<PT> R;
+  const bool vec = (p.N & 3) == 0;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = threadIdx.x + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    const bool ok = e < R::TOT && pp < p.P;
+    const float* q = src + (long)pp * p.N + n0 + c4;
+    if (vec) {
+      r.v[i] = (ok && n0 + c4 < p.N) ? *(const f4*)q : (f4){0, 0, 0, 0};
+    } else {
+      f4 w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = (ok && n0 + c4 + j < p.N) ? q[j] : 0.0f;
+      r.v[i] = w;
+    }
+  }
+}
+template <int PT>
+__device__ __forceinline__ void pn_store(const PnRegs<PT>& r, float* dst) {
+  typedef PnRegs<PT> R;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = threadIdx.x + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    if (e < R::TOT) *(f4*)(dst + pp * LDN + c4) = r.v[i];
   }
 }
 
@@ -277,5 +390,23 @@ __device__ __forceinline__ long vec_off(const KP& p, int bt, int c, int h) {
 __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   return (((long)bt * p.nc + c) * p.H + h) * CS * CS;
 }
+
+// Kernel dispatch on (P tiles, io dtype, dt dtype): the statement sees PT_, IOB_, DTB_ as constants.
+#define ISSM_DISPATCH_DT(iob, dtb, ...)                                \
+  if (iob) {                                                           \
+    constexpr bool IOB_ = true;                                        \
+    if (dtb) { constexpr bool DTB_ = true; __VA_ARGS__ }               \
+    else { constexpr bool DTB_ = false; __VA_ARGS__ }                  \
+  } else {                                                             \
+    constexpr bool IOB_ = false;                                       \
+    if (dtb) { constexpr bool DTB_ = true; __VA_ARGS__ }               \
+    else { constexpr bool DTB_ = false; __VA_ARGS__ }                  \
+  }
+#define ISSM_DISPATCH(pt, iob, dtb, ...)                                                   \
+  do {                                                                                     \
+    if ((pt) <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) }      \
+    else if ((pt) == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) } \
+    else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) }                \
+  } while (0)
 
 }  // namespace issm

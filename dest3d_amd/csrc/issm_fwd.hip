@@ -20,144 +20,195 @@
 
 namespace issm {
 
+template <int PT>
 struct FwdLocalSmem {
-  float xs[CS * LDP];    // x tile [l][p]
-  float cs[CS * LDN];    // running sum of dt'*A*log2e [l][n]
-  float bd[CS * LDN];    // B*dt' [l][n]
-  float cc[CS * LDN];    // C [l][n]
-  float opa[CS * LDN];   // level operand Cw / decayed B
-  float opb[CS * LDN];   // level operand Bw
-  float tot[4 * NS];
+  static constexpr int LDPT = PT * 16 + 4;
+  float xs[CS * LDPT];  // x tile [l][p]
+  float cs[CS * LDN];   // running sum of dt'*A*log2e [l][n] of the current slice
+  float bd[CS * LDN];   // B*dt' [l][n]
+  float cc[CS * LDN];   // C [l][n]
 };
 
-template <int PT>
+// Row-lane fragments of 16 rows x 64 columns: lane (cm, g4) holds row cm, columns 16kb + 4g4 + j.
+struct Frag {
+  f4 v[4];
+};
+__device__ __forceinline__ Frag frag_rows(const float* tile, int row0, int cm, int g4) {
+  Frag f;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) f.v[kb] = *(const f4*)(tile + (row0 + cm) * LDN + kb * 16 + 4 * g4);
+  return f;
+}
+__device__ __forceinline__ Frag frag_row_bcast(const float* tile, int row, int g4) {
+  Frag f;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) f.v[kb] = *(const f4*)(tile + row * LDN + kb * 16 + 4 * g4);
+  return f;
+}
+
+// Off-diagonal 16x16 block (I, J) of M at the level whose reference row is R:
+//   acc += (C_I * exp2(cs_I - cs_R)) . (Bd_J * exp2(cs_R - cs_J))^T   over the slice's 64 columns.
+__device__ __forceinline__ void m_offdiag(f4& acc, const float* csL, const float* ccL, const float* bdL, int I,
+                                          int J, int R, int cm, int g4) {
+  const Frag ci = frag_rows(csL, I * 16, cm, g4), cc = frag_rows(ccL, I * 16, cm, g4);
+  const Frag cj = frag_rows(csL, J * 16, cm, g4), bd = frag_rows(bdL, J * 16, cm, g4);
+  const Frag cr = frag_row_bcast(csL, R, g4);
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = cc.v[kb][j] * ex2(ci.v[kb][j] - cr.v[kb][j]);
+      const float b = bd.v[kb][j] * ex2(cr.v[kb][j] - cj.v[kb][j]);
+      acc = mfma4(a, b, acc);
+    }
+}
+
+// One sub-16 level (w = 2^LV) of the wave's diagonal block, operands built in registers from the
+// wave's own row fragments; the reference row of lane row cm is another row of the same block.
+template <int LV>
+__device__ __forceinline__ void m_diag_level(f4& acc, const Frag& cs, const Frag& cc, const Frag& bd, int cm,
+                                             int g4) {
+  constexpr int w = 1 << LV;
+  const int src = ((cm & ~(2 * w - 1)) + w - 1) + 16 * g4;
+  const bool upper = (cm & w) != 0;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float c = cs.v[kb][j];
+      const float ref = __shfl(c, src, 64);
+      const float e = ex2(upper ? c - ref : ref - c);
+      acc = mfma4(upper ? cc.v[kb][j] * e : 0.0f, upper ? 0.0f : bd.v[kb][j] * e, acc);
+    }
+}
+
+template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS) void k_chunk_local(KP p, float* __restrict__ states,
                                                           float* __restrict__ cs_last, float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  FwdLocalSmem& s = *reinterpret_cast<FwdLocalSmem*>(smem_raw);
+  typedef FwdLocalSmem<PT> SM;
+  SM& s = *reinterpret_cast<SM*>(smem_raw);
+  constexpr int LDPT = SM::LDPT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rg = tid >> 6, col = tid & 63;
+  const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
-  const int ppad = PT * 16;
+  const bool want_m = cabt != nullptr, want_s = states != nullptr;
 
-  load_lp_tile(p, u, p.x[u.dir], p.io_dt, s.xs, ppad, LDP);
-
-  // accumulators of M: level 32, 16 and the four sub-16 levels + diagonal of the wave's diagonal tile
-  f4 a32 = {0, 0, 0, 0}, a16 = {0, 0, 0, 0}, a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0}, a2 = {0, 0, 0, 0},
+  // column-lane operands of the first slice and the x tile are in flight together
+  int n = wave * 16 + cm;
+  bool vn = n < p.N;
+  int prow[16];
+  lane_rows(p, u, g4, vn, prow);
+  float raw[16], bv[16], cv[16];
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+  {
+    float xv[CS * PT * 16 / NTHREADS];
+    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    lp_store<PT>(xv, s.xs, LDPT);
+  }
+  // accumulators of M: up to two off-diagonal blocks, the four sub-16 levels and the diagonal
+  f4 o1 = {0, 0, 0, 0}, o2 = {0, 0, 0, 0}, a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0}, a2 = {0, 0, 0, 0},
      a1 = {0, 0, 0, 0}, a0 = {0, 0, 0, 0};
-  const bool want_m = cabt != nullptr;
-  const bool want_s = states != nullptr;
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
-    float pre[16];
-    prep_slice<NS>(p, u, n0, s.cs, s.opa /* dt' parked here */, s.tot, pre);
-    // bd = B*dt', cc = C
-    {
-      const int n = n0 + col;
-      const TensorD& tb = p.Bm[u.dir];
-      const TensorD& tc = p.Cm[u.dir];
-      const long bb = (long)u.b * tb.s0 + (long)u.g * tb.s2 + n;
-      const long cb = (long)u.b * tc.s0 + (long)u.g * tc.s2 + n;
+    float dtp[16], cs[16], dummy[16];
+    const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
+    float bd[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int l = rg * 16 + i, tt = u.c * CS + l;
-        const bool v = (n < p.N) && (tt < p.L);
-        const int pr = phys_row(p, u.dir, tt);
-        const float bv = v ? ldv(tb.ptr, bb + (long)pr * tb.s1, p.io_dt) : 0.0f;
-        const float cv = v ? ldv(tc.ptr, cb + (long)pr * tc.s1, p.io_dt) : 0.0f;
-        s.bd[l * LDN + col] = bv * s.opa[l * LDN + col];
-        s.cc[l * LDN + col] = cv;
+    for (int k = 0; k < 16; ++k) bd[k] = bv[k] * dtp[k];
+    if (want_m) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int o = lane_row(k, g4) * LDN + wave * 16 + cm;
+        s.cs[o] = cs[k];
+        s.bd[o] = bd[k];
+        s.cc[o] = cv[k];
       }
     }
-    if (rg == 3 && n0 + col < p.N)
-      cs_last[vec_off(p, u.bt, u.c, u.h) + n0 + col] = s.cs[63 * LDN + col] * LN2;
-    __syncthreads();
+    if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
+    const int n_cur = n;
+    const bool vn_cur = vn;
+    if (n0 + NS < p.N) {  // prefetch the next slice
+      n = n0 + NS + wave * 16 + cm;
+      vn = n < p.N;
+      lane_rows(p, u, g4, vn, prow);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+    }
+    __syncthreads();  // x tile (first slice) and the slice's LDS tiles are complete
 
     if (want_s) {
-      // decayed B: B*dt'*exp(cs_last - cs[l])
-      const float last = s.cs[63 * LDN + col];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int l = rg * 16 + i;
-        s.opa[l * LDN + col] = s.bd[l * LDN + col] * ex2(last - s.cs[l * LDN + col]);
-      }
-      __syncthreads();
-      // S[p][n] = sum_l x[l][p] * Bdec[l][n]; wave owns 16 columns
+      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
 #pragma unroll
-      for (int kb = 0; kb < CS; kb += 16)
+      for (int J = 0; J < 4; ++J)
 #pragma unroll
-        for (int pt = 0; pt < PT; ++pt) mma16_kk(acc[pt], s.xs, LDP, pt * 16, s.opa, LDN, wave * 16, kb, lane);
-      const int n = n0 + wave * 16 + (lane & 15);
+        for (int j = 0; j < 4; ++j) {
+          const int k = 4 * J + j;
+          const float b = bd[k] * ex2(last - cs[k]);
+          const float* xr = s.xs + lane_row(k, g4) * LDPT + cm;
+#pragma unroll
+          for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(xr[pt * 16], b, acc[pt]);
+        }
       float* dst = states + st_off(p, u.bt, u.c, u.h);
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int pp = pt * 16 + 4 * (lane >> 4) + r;
-          if (pp < p.P && n < p.N) dst[(long)pp * p.N + n] = acc[pt][r];
+          const int pp = pt * 16 + 4 * g4 + r;
+          if (pp < p.P && vn_cur) dst[(long)pp * p.N + n_cur] = acc[pt][r];
         }
     }
 
     if (want_m) {
-      // diagonal level: C . (B dt')^T on the wave's diagonal tile
+      // row-lane phase: this wave's diagonal block from its own row fragments
+      {
+        const Frag fc = frag_rows(s.cs, wave * 16, cm, g4);
+        const Frag fcc = frag_rows(s.cc, wave * 16, cm, g4);
+        const Frag fbd = frag_rows(s.bd, wave * 16, cm, g4);
 #pragma unroll
-      for (int kb = 0; kb < NS; kb += 16) mma16_mm(a0, s.cc, LDN, wave * 16, s.bd, LDN, wave * 16, kb, lane);
+        for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-      for (int lv = 5; lv >= 0; --lv) {
-        const int w = 1 << lv;
-        __syncthreads();  // previous users of opa/opb are done
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int l = rg * 16 + i;
-          const int ref = (l & ~(2 * w - 1)) + w - 1;
-          const float cr = s.cs[ref * LDN + col], cl = s.cs[l * LDN + col];
-          const bool upper = (l & w) != 0;
-          // upper rows act as l (left factor), lower rows as s (right factor)
-          const float e = ex2(upper ? cl - cr : cr - cl);
-          s.opa[l * LDN + col] = upper ? s.cc[l * LDN + col] * e : 0.0f;
-          s.opb[l * LDN + col] = upper ? 0.0f : s.bd[l * LDN + col] * e;
-        }
-        __syncthreads();
-        if (lv == 5) {
-          const int ti = 2 + (wave >> 1), tj = wave & 1;
-#pragma unroll
-          for (int kb = 0; kb < NS; kb += 16) mma16_mm(a32, s.opa, LDN, ti * 16, s.opb, LDN, tj * 16, kb, lane);
-        } else if (lv == 4) {
-          if (wave < 2) {
-            const int ti = wave ? 3 : 1, tj = wave ? 2 : 0;
-#pragma unroll
-            for (int kb = 0; kb < NS; kb += 16) mma16_mm(a16, s.opa, LDN, ti * 16, s.opb, LDN, tj * 16, kb, lane);
-          }
-        } else {
-          f4& acc = lv == 3 ? a8 : lv == 2 ? a4 : lv == 1 ? a2 : a1;
-#pragma unroll
-          for (int kb = 0; kb < NS; kb += 16) mma16_mm(acc, s.opa, LDN, wave * 16, s.opb, LDN, wave * 16, kb, lane);
-        }
+          for (int j = 0; j < 4; ++j) a0 = mfma4(fcc.v[kb][j], fbd.v[kb][j], a0);
+        m_diag_level<3>(a8, fc, fcc, fbd, cm, g4);
+        m_diag_level<2>(a4, fc, fcc, fbd, cm, g4);
+        m_diag_level<1>(a2, fc, fcc, fbd, cm, g4);
+        m_diag_level<0>(a1, fc, fcc, fbd, cm, g4);
       }
+      // off-diagonal blocks: level 16 -> (1,0) ref row 15, (3,2) ref row 47; level 32 -> ref row 31
+      if (wave == 0) {
+        m_offdiag(o1, s.cs, s.cc, s.bd, 1, 0, 15, cm, g4);
+        m_offdiag(o2, s.cs, s.cc, s.bd, 2, 0, 31, cm, g4);
+      } else if (wave == 1) {
+        m_offdiag(o1, s.cs, s.cc, s.bd, 2, 1, 31, cm, g4);
+      } else if (wave == 2) {
+        m_offdiag(o1, s.cs, s.cc, s.bd, 3, 2, 47, cm, g4);
+      } else {
+        m_offdiag(o1, s.cs, s.cc, s.bd, 3, 0, 31, cm, g4);
+        m_offdiag(o2, s.cs, s.cc, s.bd, 3, 1, 31, cm, g4);
+      }
+      __syncthreads();  // before the next slice overwrites the LDS tiles
     }
-    __syncthreads();
   }
 
   if (want_m) {
     float* m = cabt + sq_off(p, u.bt, u.c, u.h);
-    const int cm = lane & 15, g = lane >> 4;
-    // level 32 tile
-    {
-      const int ti = 2 + (wave >> 1), tj = wave & 1;
+    auto put = [&](const f4& a, int I, int J) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) m[(ti * 16 + 4 * g + r) * CS + tj * 16 + cm] = a32[r];
-    }
-    if (wave < 2) {
-      const int ti = wave ? 3 : 1, tj = wave ? 2 : 0;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) m[(ti * 16 + 4 * g + r) * CS + tj * 16 + cm] = a16[r];
-    }
+      for (int r = 0; r < 4; ++r) m[(I * 16 + 4 * g4 + r) * CS + J * 16 + cm] = a[r];
+    };
+    if (wave == 0) { put(o1, 1, 0); put(o2, 2, 0); }
+    else if (wave == 1) put(o1, 2, 1);
+    else if (wave == 2) put(o1, 3, 2);
+    else { put(o1, 3, 0); put(o2, 3, 1); }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int l = 4 * g + r, sc = cm;  // within the diagonal tile
+      const int l = 4 * g4 + r, sc = cm;  // within the diagonal block
       const int d = l ^ sc;
       float v = d == 0 ? a0[r] : d >= 8 ? a8[r] : d >= 4 ? a4[r] : d >= 2 ? a2[r] : a1[r];
       if (sc > l) v = 0.0f;
@@ -226,57 +277,63 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
 }
 
 // ------------------------------------------------------------------ chunk scan
+template <int PT>
 struct FwdScanSmem {
-  float xs[CS * LDP];   // x [s][p]
-  float ms[CS * LDC];   // tril(M) [l][s]
-  float cs[CS * LDN];
-  float ct[CS * LDN];   // C * exp2(cs) [l][n]
-  float hs[MAXP * LDN]; // H [p][n]
-  float tot[4 * NS];
+  static constexpr int LDPT = PT * 16 + 4;
+  float xs[CS * LDPT];      // x [s][p]
+  float ms[CS * LDC];       // tril(M) [l][s]
+  float ct[CS * LDN];       // C * exp2(cs) [l][n]
+  float hs[PT * 16 * LDN];  // H [p][n]
 };
 
-template <int PT>
+template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states,
                                                          const float* __restrict__ cabt, float* __restrict__ out_x) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  FwdScanSmem& s = *reinterpret_cast<FwdScanSmem*>(smem_raw);
+  typedef FwdScanSmem<PT> SM;
+  SM& s = *reinterpret_cast<SM*>(smem_raw);
+  constexpr int LDPT = SM::LDPT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rg = tid >> 6, col = tid & 63;
+  const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
-  const int ppad = PT * 16;
+  const float* hsrc = states + st_off(p, u.bt, u.c, u.h);
 
-  load_lp_tile(p, u, p.x[u.dir], p.io_dt, s.xs, ppad, LDP);
+  int n = wave * 16 + cm;
+  bool vn = n < p.N;
+  int prow[16];
+  lane_rows(p, u, g4, vn, prow);
+  float raw[16], cv[16];
+  PnRegs<PT> hv;
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+  pn_load<PT>(p, hsrc, 0, hv);
   {
-    const float* m = cabt + sq_off(p, u.bt, u.c, u.h);
-    for (int e = tid; e < CS * CS; e += NTHREADS) {
-      const int l = e >> 6, sc = e & 63;
-      s.ms[l * LDC + sc] = sc <= l ? m[e] : 0.0f;
-    }
+    float xv[CS * PT * 16 / NTHREADS];
+    f4 mv[4];
+    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
+    lp_store<PT>(xv, s.xs, LDPT);
+    tril_store(mv, s.ms);
   }
   f4 acc[PT];
 #pragma unroll
   for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
 
-  const float* hsrc = states + st_off(p, u.bt, u.c, u.h);
   for (int n0 = 0; n0 < p.N; n0 += NS) {
-    float pre[16];
-    prep_slice<NS>(p, u, n0, s.cs, s.ct /* dt' unused */, s.tot, pre);
     {
-      const int n = n0 + col;
-      const TensorD& tc = p.Cm[u.dir];
-      const long cb = (long)u.b * tc.s0 + (long)u.g * tc.s2 + n;
+      float dtp[16], cs[16], dummy[16];
+      lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int l = rg * 16 + i, tt = u.c * CS + l;
-        const bool v = (n < p.N) && (tt < p.L);
-        const float cv = v ? ldv(tc.ptr, cb + (long)phys_row(p, u.dir, tt) * tc.s1, p.io_dt) : 0.0f;
-        s.ct[l * LDN + col] = cv * ex2(s.cs[l * LDN + col]);
-      }
-      for (int e = tid; e < ppad * NS; e += NTHREADS) {
-        const int pp = e >> 6, c2 = e & 63;
-        const bool v = pp < p.P && n0 + c2 < p.N;
-        s.hs[pp * LDN + c2] = v ? hsrc[(long)pp * p.N + n0 + c2] : 0.0f;
-      }
+      for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
+    }
+    pn_store<PT>(hv, s.hs);
+    if (n0 + NS < p.N) {
+      n = n0 + NS + wave * 16 + cm;
+      vn = n < p.N;
+      lane_rows(p, u, g4, vn, prow);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+      pn_load<PT>(p, hsrc, n0 + NS, hv);
     }
     __syncthreads();
     // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows
@@ -289,44 +346,46 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   // y[l][p] += sum_{s<=l} M[l][s] x[s][p]; rows of this wave only need s < 16(wave+1)
   for (int kb = 0; kb < (wave + 1) * 16; kb += 16)
 #pragma unroll
-    for (int pt = 0; pt < PT; ++pt) mma16_mk(acc[pt], s.ms, LDC, wave * 16, s.xs, LDP, pt * 16, kb, lane);
+    for (int pt = 0; pt < PT; ++pt) mma16_mk(acc[pt], s.ms, LDC, wave * 16, s.xs, LDPT, pt * 16, kb, lane);
 
   const TensorD& to = p.out[u.dir];
   const TensorD& tz = p.z[u.dir];
 #pragma unroll
-  for (int pt = 0; pt < PT; ++pt)
+  for (int pt = 0; pt < PT; ++pt) {
+    int off[4];
+    float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int l = wave * 16 + 4 * (lane >> 4) + r, pp = pt * 16 + (lane & 15);
+      const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm;
       const int tt = u.c * CS + l;
-      if (tt >= p.L || pp >= p.P) continue;
-      const int pr = phys_row(p, u.dir, tt);
-      float v = acc[pt][r];
-      if (p.D) v += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + pp] : p.D[u.h]) * s.xs[l * LDP + pp];
-      if (tz.ptr) {
-        if (out_x) out_x[(((long)u.bt * p.L + pr) * p.H + u.h) * p.P + pp] = v;
+      const bool ok = tt < p.L && pp < p.P;
+      const int pr = ok ? phys_row(p, u.dir, tt) : 0;
+      v[r] = acc[pt][r];
+      if (p.D && ok) v[r] += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + pp] : p.D[u.h]) * s.xs[l * LDPT + pp];
+      if (tz.ptr && ok) {
+        if (out_x) out_x[(((long)u.bt * p.L + pr) * p.H + u.h) * p.P + pp] = v[r];
         const float zz = ldv(tz.ptr, (long)u.b * tz.s0 + (long)pr * tz.s1 + (long)u.h * tz.s2 + pp, p.io_dt);
-        v *= zz * sigmoidf_(zz);
+        v[r] *= zz * sigmoidf_(zz);
       }
-      stv(const_cast<void*>(to.ptr), (long)u.b * to.s0 + (long)pr * to.s1 + (long)u.h * to.s2 + pp, p.io_dt, v);
+      off[r] = ok ? pr * (int)to.s1 + pp : -1;
     }
+    gstore<IOB, 4>(const_cast<void*>(to.ptr), (long)u.b * to.s0 + (long)u.h * to.s2, off, v);
+  }
 }
 
 // ------------------------------------------------------------------- launchers
+template <typename K>
+static int set_lds(K kernel, size_t bytes) {
+  return (int)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
 int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  const int pt = (p.P + 15) / 16;
-  const size_t sm = sizeof(FwdLocalSmem);
-#define LAUNCH(PT_)                                                                                        \
-  { hipError_t e_ = hipFuncSetAttribute((const void*)k_chunk_local<PT_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm); if (e_ != hipSuccess) return (int)e_; } \
-  hipLaunchKernelGGL(k_chunk_local<PT_>, dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt)
-  switch (pt) {
-    case 1: LAUNCH(1); break;
-    case 2: LAUNCH(2); break;
-    case 3: LAUNCH(3); break;
-    default: LAUNCH(4); break;
-  }
-#undef LAUNCH
+  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+    const size_t sm = sizeof(FwdLocalSmem<PT_>);
+    if (int e = set_lds(k_chunk_local<PT_, IOB_, DTB_>, sm)) return e;
+    hipLaunchKernelGGL((k_chunk_local<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
+  });
   return (int)hipGetLastError();
 }
 
@@ -339,18 +398,11 @@ int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream
 
 int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float* out_x, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  const int pt = (p.P + 15) / 16;
-  const size_t sm = sizeof(FwdScanSmem);
-#define LAUNCH(PT_)                                                                                       \
-  { hipError_t e_ = hipFuncSetAttribute((const void*)k_chunk_scan<PT_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm); if (e_ != hipSuccess) return (int)e_; } \
-  hipLaunchKernelGGL(k_chunk_scan<PT_>, dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x)
-  switch (pt) {
-    case 1: LAUNCH(1); break;
-    case 2: LAUNCH(2); break;
-    case 3: LAUNCH(3); break;
-    default: LAUNCH(4); break;
-  }
-#undef LAUNCH
+  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+    const size_t sm = sizeof(FwdScanSmem<PT_>);
+    if (int e = set_lds(k_chunk_scan<PT_, IOB_, DTB_>, sm)) return e;
+    hipLaunchKernelGGL((k_chunk_scan<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
+  });
   return (int)hipGetLastError();
 }
 
