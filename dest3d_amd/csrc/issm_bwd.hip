@@ -241,6 +241,7 @@ struct BwdChunkSmem {
   float xs[CS * LDPT];
   float dys[CS * LDPT];
   float dms[CS * LDC];
+  float dbc[32 * NTHREADS];  // per-lane dB / dC accumulators [k][tid]
 };
 
 // One level (w = 2^LV) of the row hierarchy for F and G.  op[k] = Bd * exp2(ref - cs) on lower
@@ -248,9 +249,18 @@ struct BwdChunkSmem {
 // the last row of the lower half of the row's 2w-block, fetched from the lane that owns it.  Rows
 // that are upper at this level receive their F contribution (x2), lower rows their G
 // contribution (e1).
+
+// Opaque pass-through of 16 registers: everything that depends on the array is ordered after this
+// point and everything that produces it before, which keeps the phases of a long straight-line
+// kernel from being interleaved (and their temporaries from being live at the same time).
+__device__ __forceinline__ void pin16(float (&a)[16]) {
+  asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+               "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+
 template <int LV>
 __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
-                                          const float* __restrict__ dms, f4 (&e1)[4], f4 (&x2)[4], int cm, int g4) {
+                                          const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm, int g4) {
   constexpr int w = 1 << LV;
   float op[16], ee[16];
 #pragma unroll
@@ -294,8 +304,8 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        if (I >= 2) x2[I][rr] += ee[4 * I + rr] * acc[rr];
-        else e1[I][rr] += ee[4 * I + rr] * acc[rr];
+        if (I >= 2) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+        else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
       }
     } else if (LV == 4) {
       if (I & 1) {
@@ -309,8 +319,8 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        if (I & 1) x2[I][rr] += ee[4 * I + rr] * acc[rr];
-        else e1[I][rr] += ee[4 * I + rr] * acc[rr];
+        if (I & 1) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+        else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
       }
     } else {
       // inside the diagonal tile: contraction rows kr = 4 g4 + j, restricted to the 2w-block of the
@@ -329,8 +339,10 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const bool upper = ((4 * g4 + rr) >> LV) & 1;
-        if (upper) x2[I][rr] += ee[4 * I + rr] * acc[rr];
-        else e1[I][rr] += ee[4 * I + rr] * gw[rr];
+        // (value selects, not a branch between the two arrays: a select between their addresses
+        // would force both arrays out of registers)
+        x2[4 * I + rr] += upper ? ee[4 * I + rr] * acc[rr] : 0.0f;
+        e1[4 * I + rr] += upper ? 0.0f : ee[4 * I + rr] * gw[rr];
       }
     }
   }
@@ -338,12 +350,12 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
 
 // partA, partBias: (Bt*nc, H, N) per-unit partial sums of dA and ddt_bias
 template <int PT, bool IOB, bool DTB>
-__global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws,
-                                                        const float* __restrict__ states,
-                                                        const float* __restrict__ dstates,
-                                                        const float* __restrict__ dm,
-                                                        const float* __restrict__ g_last, float* __restrict__ partA,
-                                                        float* __restrict__ partBias) {
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws,
+                                                           const float* __restrict__ states,
+                                                           const float* __restrict__ dstates,
+                                                           const float* __restrict__ dm,
+                                                           const float* __restrict__ g_last,
+                                                           float* __restrict__ partA, float* __restrict__ partBias) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -366,65 +378,96 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __res
   const int n = ns * NS + wave * 16 + cm;
   const bool vn = n < p.N;
 
-  int prow[16];
-  lane_rows(p, u, g4, vn, prow);
+  // The lane's rows are 16J + 4 g4 + j; their physical rows form an arithmetic progression:
+  // row index k -> r0 + sgn * (16J + j), valid while 16J + j < lim (0 valid rows if the column is absent).
+  const int t0 = u.c * CS + 4 * g4;
+  const int r0 = u.dir ? p.L - 1 - t0 : t0, sgn = u.dir ? -1 : 1;
+  const int lim = vn ? p.L - t0 : 0;
+  auto rowk = [&](int k) { return 16 * (k >> 2) + (k & 3); };
+  // nn is re-materialised per head (opaque to the optimiser) so that the 16-element offset arrays are
+  // recomputed where they are used instead of being hoisted out of the head loop into registers
+  int nn = n;
+  auto offk = [&](int k, int stride) { return rowk(k) < lim ? (r0 + sgn * rowk(k)) * stride + nn : -1; };
+
   float Bv[16], Cv[16];
-  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, Bv);
-  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, Cv);
-  float dBacc[16], dCacc[16];
+  {
+    const TensorD& tb = p.Bm[u.dir];
+    const TensorD& tc = p.Cm[u.dir];
+    int ob[16], oc[16];
 #pragma unroll
-  for (int k = 0; k < 16; ++k) dBacc[k] = dCacc[k] = 0.0f;
-  int oddt[16];
+    for (int k = 0; k < 16; ++k) {
+      ob[k] = offk(k, (int)tb.s1);
+      oc[k] = offk(k, (int)tc.s1);
+    }
+    gload<IOB, 16>(tb.ptr, (long)u.b * tb.s0 + (long)u.g * tb.s2, ob, Bv);
+    gload<IOB, 16>(tc.ptr, (long)u.b * tc.s0 + (long)u.g * tc.s2, oc, Cv);
+  }
+  // dB / dC accumulators over the heads of the group: private to the lane, kept in LDS
 #pragma unroll
-  for (int k = 0; k < 16; ++k) oddt[k] = (prow[k] < 0 || !p.ddt.ptr) ? -1 : prow[k] * (int)p.ddt.s1 + n;
+  for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
   for (int hh = 0; hh < p.hpg; ++hh) {
     u.h = u.g * p.hpg + hh;
+    asm volatile("" : "+v"(nn));
     // ---- global loads of this head
-    float raw[16], dsv[KP_], hv[KP_], old[16];
-    lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
+    float raw[16], dsv[KP_], hv[KP_];
     {
+      int od[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) od[k] = offk(k, (int)p.dt.s1);
+      gload<DTB, 16>(p.dt.ptr, (long)u.b * p.dt.s0 + (long)u.h * p.dt.s2, od, raw);
       int os[KP_];
 #pragma unroll
       for (int q = 0; q < KP_; ++q) {
         const int pp = 16 * (q >> 2) + 4 * g4 + (q & 3);
-        os[q] = (vn && pp < p.P) ? pp * p.N + n : -1;
+        os[q] = (vn && pp < p.P) ? pp * p.N + nn : -1;
       }
       gload<false, KP_>(dstates, dst_off(p, u.bt, u.c, u.h), os, dsv);
       gload<false, KP_>(states, st_off(p, u.bt, u.c, u.h), os, hv);
     }
-    const long ddt_base = (long)u.b * p.ddt.s0 + (long)u.h * p.ddt.s2;
-    if (p.dir0 > 0) gload<DTB, 16>(p.ddt.ptr, ddt_base, oddt, old);
     {
       float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
       f4 mv[4];
-      dy_load<IOB, PT>(p, u, dy_ws, dv);
-      lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
-      tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv);
+      int tq = tid;
+      asm volatile("" : "+v"(tq));
+      dy_load<IOB, PT>(p, u, dy_ws, dv, tq);
+      lp_load<IOB, PT>(p, u, p.x[u.dir], xv, tq);
+      tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv, tq);
       __syncthreads();  // the previous head no longer reads the LDS tiles
-      lp_store<PT>(dv, s.dys, LDPT);
-      lp_store<PT>(xv, s.xs, LDPT);
-      tril_store(mv, s.dms);
+      lp_store<PT>(dv, s.dys, LDPT, tq);
+      lp_store<PT>(xv, s.xs, LDPT, tq);
+      tril_store(mv, s.dms, tq);
     }
     __syncthreads();
 
     // ---- dt transform and running sum down the chunk (log2 domain)
     const float An = vn ? p.A[u.h * p.N + n] : 0.0f;
     float dtp[16], cs[16], dfac[16];
-    const float last = lane_prep<true>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dfac);
+    float last;
+    {
+      int prow[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) prow[k] = rowk(k) < lim ? 0 : -1;
+      last = lane_prep<true>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dfac);
+    }
     float Bd[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) Bd[k] = Bv[k] * dtp[k];
+    pin16(cs); pin16(Bd);
 
     // ---- Q, R, diagonal terms.  e1 / x2 [I][r] <-> row 16I + 4 g4 + r <-> index k = 4I + r
-    f4 e1[4], x2[4];
+    // (LDS fragment addresses are derived from per-head opaque copies of the lane coordinates so that
+    // they are recomputed instead of being kept live across the whole head loop)
+    int cq = cm, gq = g4;
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    float e1[16], x2[16];
 #pragma unroll
     for (int I = 0; I < 4; ++I) {
       f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
 #pragma unroll
       for (int kb = 0; kb < PT; ++kb) {
-        const f4 ax = *(const f4*)(s.xs + (I * 16 + cm) * LDPT + kb * 16 + 4 * g4);
-        const f4 ay = *(const f4*)(s.dys + (I * 16 + cm) * LDPT + kb * 16 + 4 * g4);
+        const f4 ax = *(const f4*)(s.xs + (I * 16 + cq) * LDPT + kb * 16 + 4 * gq);
+        const f4 ay = *(const f4*)(s.dys + (I * 16 + cq) * LDPT + kb * 16 + 4 * gq);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           q = mfma4(ax[j], dsv[4 * kb + j], q);
@@ -433,35 +476,55 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __res
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int k = 4 * I + rr, row = 16 * I + 4 * g4 + rr;
+        const int k = 4 * I + rr, row = 16 * I + 4 * gq + rr;
         const float dd = s.dms[row * LDC + row];
-        e1[I][rr] = ex2(last - cs[k]) * q[rr] + dd * Cv[k];
-        x2[I][rr] = ex2(cs[k]) * r[rr] + dd * Bd[k];
+        e1[k] = ex2(last - cs[k]) * q[rr] + dd * Cv[k];
+        x2[k] = ex2(cs[k]) * r[rr] + dd * Bd[k];
       }
     }
 
     // ---- hierarchy levels of F and G; scheduling barriers keep one level's operands live at a time
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<5>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<5>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<4>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<4>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<3>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<3>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<2>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<2>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<1>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<1>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_level<0>(cs, Bd, Cv, s.dms, e1, x2, cm, g4);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_level<0>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase: everything below is local to the lane except the scans over rows
+    pin16(e1); pin16(x2);
+    asm volatile("" : "+v"(nn));
+    int oddt[16];
+    float old[16];
+    const long ddt_base = (long)u.b * p.ddt.s0 + (long)u.h * p.ddt.s2;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) oddt[k] = p.ddt.ptr ? offk(k, (int)p.ddt.s1) : -1;
+    if (p.dir0 > 0) gload<DTB, 16>(p.ddt.ptr, ddt_base, oddt, old);
     float dcs[16], val[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      const float E1 = e1[k >> 2][k & 3], X2 = x2[k >> 2][k & 3];
-      dBacc[k] += dtp[k] * E1;
-      dCacc[k] += X2;
+      const float E1 = e1[k], X2 = x2[k];
+      s.dbc[k * NTHREADS + tid] += dtp[k] * E1;
+      s.dbc[(16 + k) * NTHREADS + tid] += X2;
       val[k] = Bv[k] * E1;
       dcs[k] = Cv[k] * X2 - Bd[k] * E1;
     }
@@ -489,7 +552,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __res
       const float da = dcs[k];
       sumA += da * dtp[k];
       val[k] = (val[k] + da * An) * dfac[k];
-      if (prow[k] >= 0) sumB += val[k];
+      if (rowk(k) < lim) sumB += val[k];
       if (p.dir0 > 0) val[k] += old[k];
     }
     gstore<DTB, 16>(const_cast<void*>(p.ddt.ptr), ddt_base, oddt, val);
@@ -505,13 +568,16 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_chunk(KP p, const float* __res
     const TensorD& tB = p.dB[u.dir];
     const TensorD& tC = p.dC[u.dir];
     int ob[16], oc[16];
+    float vb[16], vc[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      ob[k] = (prow[k] < 0 || !tB.ptr) ? -1 : prow[k] * (int)tB.s1 + n;
-      oc[k] = (prow[k] < 0 || !tC.ptr) ? -1 : prow[k] * (int)tC.s1 + n;
+      ob[k] = tB.ptr ? offk(k, (int)tB.s1) : -1;
+      oc[k] = tC.ptr ? offk(k, (int)tC.s1) : -1;
+      vb[k] = s.dbc[k * NTHREADS + tid];
+      vc[k] = s.dbc[(16 + k) * NTHREADS + tid];
     }
-    gstore<IOB, 16>(const_cast<void*>(tB.ptr), (long)u.b * tB.s0 + (long)u.g * tB.s2, ob, dBacc);
-    gstore<IOB, 16>(const_cast<void*>(tC.ptr), (long)u.b * tC.s0 + (long)u.g * tC.s2, oc, dCacc);
+    gstore<IOB, 16>(const_cast<void*>(tB.ptr), (long)u.b * tB.s0 + (long)u.g * tB.s2, ob, vb);
+    gstore<IOB, 16>(const_cast<void*>(tC.ptr), (long)u.b * tC.s0 + (long)u.g * tC.s2, oc, vc);
   }
 }
 

@@ -282,54 +282,55 @@ __device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, i
 // LDS dst[l][p] (leading dimension ld).  Element e = tid + 256 i is (l, p) = (e / 16PT, e % 16PT).
 template <bool BF, int PT>
 __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const TensorD& t,
-                                        float (&v)[CS * PT * 16 / NTHREADS]) {
+                                        float (&v)[CS * PT * 16 / NTHREADS], int tid = threadIdx.x) {
   constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
   int off[CNT];
 #pragma unroll
   for (int i = 0; i < CNT; ++i) {
-    const int e = threadIdx.x + i * NTHREADS;
+    const int e = tid + i * NTHREADS;
     const int l = e / PPAD, pp = e % PPAD, tt = u.c * CS + l;
     off[i] = ((pp < p.P) && (tt < p.L)) ? phys_row(p, u.dir, tt) * (int)t.s1 + pp : -1;
   }
   gload<BF, CNT>(t.ptr, (long)u.b * t.s0 + (long)u.h * t.s2, off, v);
 }
 template <int PT>
-__device__ __forceinline__ void lp_store(const float (&v)[CS * PT * 16 / NTHREADS], float* dst, int ld) {
+__device__ __forceinline__ void lp_store(const float (&v)[CS * PT * 16 / NTHREADS], float* dst, int ld,
+                                         int tid = threadIdx.x) {
   constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
 #pragma unroll
   for (int i = 0; i < CNT; ++i) {
-    const int e = threadIdx.x + i * NTHREADS;
+    const int e = tid + i * NTHREADS;
     dst[(e / PPAD) * ld + (e % PPAD)] = v[i];
   }
 }
 // dy tile: from the caller's dout (io dtype) or from the gated fp32 (Bt,L,H,P) workspace copy.
 template <bool BF, int PT>
 __device__ __forceinline__ void dy_load(const KP& p, const Unit& u, const float* dy_ws,
-                                        float (&v)[CS * PT * 16 / NTHREADS]) {
+                                        float (&v)[CS * PT * 16 / NTHREADS], int tid = threadIdx.x) {
   if (dy_ws) {
     TensorD t;
     t.ptr = dy_ws + (long)(u.bt - u.b) * p.L * p.H * p.P;  // so that b * s0 lands on row block bt
     t.s0 = (long)p.L * p.H * p.P;
     t.s1 = (long)p.H * p.P;
     t.s2 = p.P;
-    lp_load<false, PT>(p, u, t, v);
+    lp_load<false, PT>(p, u, t, v, tid);
   } else {
-    lp_load<BF, PT>(p, u, p.dout[u.dir], v);
+    lp_load<BF, PT>(p, u, p.dout[u.dir], v, tid);
   }
 }
 
 // Lower triangle (s <= l, rest zero) of a 64x64 fp32 block: registers, then LDS dst[l][s] (ld = LDC).
-__device__ __forceinline__ void tril_load(const float* __restrict__ src, f4 (&v)[4]) {
+__device__ __forceinline__ void tril_load(const float* __restrict__ src, f4 (&v)[4], int tid = threadIdx.x) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int e = threadIdx.x + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
+    const int e = tid + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
     v[i] = (s4 <= l) ? *(const f4*)(src + l * CS + s4) : (f4){0, 0, 0, 0};
   }
 }
-__device__ __forceinline__ void tril_store(const f4 (&v)[4], float* dst) {
+__device__ __forceinline__ void tril_store(const f4 (&v)[4], float* dst, int tid = threadIdx.x) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int e = threadIdx.x + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
+    const int e = tid + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
     f4 w = v[i];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -346,12 +347,13 @@ struct PnRegs {
   f4 v[CNT];
 };
 template <int PT>
-__device__ __forceinline__ void pn_load(const KP& p, const float* __restrict__ src, int n0, PnRegs<PT>& r) {
+__device__ __forceinline__ void pn_load(const KP& p, const float* __restrict__ src, int n0, PnRegs<PT>& r,
+                                        int tid = threadIdx.x) {
   typedef PnRegs<PT> R;
   const bool vec = (p.N & 3) == 0;
 #pragma unroll
   for (int i = 0; i < R::CNT; ++i) {
-    const int e = threadIdx.x + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
     const bool ok = e < R::TOT && pp < p.P;
     const float* q = src + (long)pp * p.N + n0 + c4;
     if (vec) {
@@ -365,11 +367,11 @@ __device__ __forceinline__ void pn_load(const KP& p, const float* __restrict__ s
   }
 }
 template <int PT>
-__device__ __forceinline__ void pn_store(const PnRegs<PT>& r, float* dst) {
+__device__ __forceinline__ void pn_store(const PnRegs<PT>& r, float* dst, int tid = threadIdx.x) {
   typedef PnRegs<PT> R;
 #pragma unroll
   for (int i = 0; i < R::CNT; ++i) {
-    const int e = threadIdx.x + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
     if (e < R::TOT) *(f4*)(dst + pp * LDN + c4) = r.v[i];
   }
 }
