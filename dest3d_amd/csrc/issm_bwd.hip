@@ -250,14 +250,6 @@ struct BwdChunkSmem {
 // that are upper at this level receive their F contribution (x2), lower rows their G
 // contribution (e1).
 
-// Opaque pass-through of 16 registers: everything that depends on the array is ordered after this
-// point and everything that produces it before, which keeps the phases of a long straight-line
-// kernel from being interleaved (and their temporaries from being live at the same time).
-__device__ __forceinline__ void pin16(float (&a)[16]) {
-  asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
-               "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
-}
-
 template <int LV>
 __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
                                           const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm, int g4) {

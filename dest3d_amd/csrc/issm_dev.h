@@ -133,6 +133,15 @@ __device__ __forceinline__ void gstore(void* p, long ubase, const int (&off)[CNT
   }
 }
 
+// Opaque pass-through of registers: everything that depends on the values is ordered after this
+// point and everything that produces them before, which keeps the phases of a long straight-line
+// kernel from being interleaved by the scheduler (and their temporaries from being live together).
+__device__ __forceinline__ void pin16(float (&a)[16]) {
+  asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+               "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+__device__ __forceinline__ void pin4(f4& a) { asm volatile("" : "+v"(a)); }
+
 // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
 // ids so that units sharing B/C tiles (the heads of one chunk) share an L2.
 __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {

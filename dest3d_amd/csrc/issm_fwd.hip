@@ -83,7 +83,7 @@ __device__ __forceinline__ void m_diag_level(f4& acc, const Frag& cs, const Frag
 }
 
 template <int PT, bool IOB, bool DTB>
-__global__ __launch_bounds__(NTHREADS) void k_chunk_local(KP p, float* __restrict__ states,
+__global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __restrict__ states,
                                                           float* __restrict__ cs_last, float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef FwdLocalSmem<PT> SM;
@@ -175,14 +175,20 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_local(KP p, float* __restric
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
           for (int j = 0; j < 4; ++j) a0 = mfma4(fcc.v[kb][j], fbd.v[kb][j], a0);
+        pin4(a0);
         m_diag_level<3>(a8, fc, fcc, fbd, cm, g4);
+        pin4(a8);
         m_diag_level<2>(a4, fc, fcc, fbd, cm, g4);
+        pin4(a4);
         m_diag_level<1>(a2, fc, fcc, fbd, cm, g4);
+        pin4(a2);
         m_diag_level<0>(a1, fc, fcc, fbd, cm, g4);
+        pin4(a1);
       }
       // off-diagonal blocks: level 16 -> (1,0) ref row 15, (3,2) ref row 47; level 32 -> ref row 31
       if (wave == 0) {
         m_offdiag(o1, s.cs, s.cc, s.bd, 1, 0, 15, cm, g4);
+        pin4(o1);
         m_offdiag(o2, s.cs, s.cc, s.bd, 2, 0, 31, cm, g4);
       } else if (wave == 1) {
         m_offdiag(o1, s.cs, s.cc, s.bd, 2, 1, 31, cm, g4);
@@ -190,6 +196,7 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_local(KP p, float* __restric
         m_offdiag(o1, s.cs, s.cc, s.bd, 3, 2, 47, cm, g4);
       } else {
         m_offdiag(o1, s.cs, s.cc, s.bd, 3, 0, 31, cm, g4);
+        pin4(o1);
         m_offdiag(o2, s.cs, s.cc, s.bd, 3, 1, 31, cm, g4);
       }
       __syncthreads();  // before the next slice overwrites the LDS tiles
