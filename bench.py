@@ -186,6 +186,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
+    ap.add_argument("--traffic", type=float, default=None,
+                    help="measured HBM bytes per launch of the dominant kernel (from rocprofv3 --pmc), echoed into roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -195,6 +199,12 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     run = Runner(torch, 2, torch.float32)
     us = run.time_steps(args.steps, args.warmup)
     stages = run.stage_times()
@@ -209,6 +219,7 @@ def main():
         achieved = amount / (stages[dom] * 1e-6) / 1e9
         roof = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": achieved / PEAK_HBM_GBS, "traffic": None, "kernel": dom}
+    roof["traffic"] = args.traffic
     per_stage = {}
     for k, (b, amt) in work.items():
         rate = amt / (stages[k] * 1e-6)
