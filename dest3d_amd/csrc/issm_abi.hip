@@ -101,6 +101,8 @@ static int check_dims(const issm_scan_args* a) {
   return ISSM_OK;
 }
 
+static int check_strides(const issm_scan_args* a);
+
 static int check_common(const issm_scan_args* a) {
   int rc = check_dims(a);
   if (rc) return rc;
@@ -117,6 +119,39 @@ static int check_common(const issm_scan_args* a) {
     if ((a->z[0].ptr != nullptr) != (a->z[dir].ptr != nullptr))
       return fail(ISSM_E_NULL, "z must be given for all directions or none");
   }
+  return check_strides(a);
+}
+
+// The kernels address a row of a caller tensor as a 64-bit (batch, head) base plus a 32-bit
+// (time row * stride[1] + column) offset: that offset must fit, and strides may not be negative.
+static int check_td(const issm_tensor& t, const char* name, int dir, long rows, long inner) {
+  if (!t.ptr) return ISSM_OK;
+  for (int i = 0; i < 3; ++i)
+    if (t.stride[i] < 0) return fail(ISSM_E_STRIDE, "%s[%d]: negative stride %ld", name, dir, (long)t.stride[i]);
+  if ((rows - 1) * (long)t.stride[1] + inner > 0x7fffffffL)
+    return fail(ISSM_E_STRIDE, "%s[%d]: seqlen * stride[1] = %ld * %ld exceeds the 32-bit row offset range", name, dir,
+                rows, (long)t.stride[1]);
+  return ISSM_OK;
+}
+
+static int check_strides(const issm_scan_args* a) {
+  const issm_dims& d = a->dims;
+  int rc;
+  for (int i = 0; i < d.ndir; ++i) {
+    if ((rc = check_td(a->x[i], "x", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->z[i], "z", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->out[i], "out", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->dout[i], "dout", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->dx[i], "dx", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->dz[i], "dz", i, d.seqlen, d.headdim))) return rc;
+    if ((rc = check_td(a->Bm[i], "B", i, d.seqlen, d.dstate))) return rc;
+    if ((rc = check_td(a->Cm[i], "C", i, d.seqlen, d.dstate))) return rc;
+    if ((rc = check_td(a->dB[i], "dB", i, d.seqlen, d.dstate))) return rc;
+    if ((rc = check_td(a->dC[i], "dC", i, d.seqlen, d.dstate))) return rc;
+  }
+  if ((rc = check_td(a->dt, "dt", 0, d.seqlen, d.dstate))) return rc;
+  if ((rc = check_td(a->ddt, "ddt", 0, d.seqlen, d.dstate))) return rc;
+  if ((rc = check_td(a->h0, "initial_states", 0, d.nheads, d.dstate))) return rc;
   return ISSM_OK;
 }
 

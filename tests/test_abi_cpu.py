@@ -78,6 +78,18 @@ def test_status_codes(lib):
     assert lib.issm_fwd_workspace_bytes(C.byref(a), C.byref(n)) == -5
     d.headdim = 32
     assert lib.issm_scan_fwd(C.byref(a)) == -1          # A is NULL: validated before any launch
+    # stride rules are checked on the host before any launch (the pointers are never dereferenced)
+    fake = 0x1000
+    a.A = fake
+    for t in (a.dt, a.x[0], a.Bm[0], a.Cm[0]):
+        t.ptr = fake
+        t.stride[0], t.stride[1], t.stride[2] = 64 * 3 * 64, 3 * 64, 64
+    a.dt.stride[1] = -1
+    assert lib.issm_scan_fwd(C.byref(a)) == -3 and b"negative stride" in lib.issm_last_error()
+    a.dt.stride[1] = 1 << 30
+    assert lib.issm_scan_fwd(C.byref(a)) == -3 and b"32-bit" in lib.issm_last_error()
+    a.dt.stride[1] = 3 * 64
+    assert lib.issm_scan_fwd(C.byref(a)) == -6          # now only the workspace is missing
     na = L.NormArgs()
     assert lib.issm_gated_rmsnorm_fwd(C.byref(na)) == -2
     assert lib.issm_rmsnorm_bwd_blocks(10) == 10 and lib.issm_rmsnorm_bwd_blocks(10 ** 6) == 2048
