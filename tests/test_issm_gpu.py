@@ -101,6 +101,8 @@ CASES = [
     (1, 130, 2, 36, 128, 1, dict(softplus=False, D="h")),
     (1, 96, 2, 64, 64, 2, dict(h0=False, bias=False, D=None)),
     (1, 320, 8, 32, 256, 1, dict(softplus=False)),
+    (1, 70, 2, 20, 30, 1, dict(D="hp", z=True)),         # N not a multiple of 4, P not a multiple of 16
+    (1, 1, 1, 8, 16, 1, dict()),                          # a single token
 ]
 
 
@@ -321,3 +323,116 @@ def test_properties_at_benchmark_shape():
     _check("final[0]", fg, fr, FWD32)
     for k in ins:
         _check("d" + k, gi[k].grad, ins[k].grad, BWD32)
+
+
+def _split_sequence_check(t, dtype, Lh, tol_sum):
+    """scan(whole sequence) must equal scan(first part) followed by scan(rest) started from the first part's
+    final state, forward and backward (the backward chains d(initial_states) of the second call into
+    d(final_states) of the first).  Both runs use the same chunk boundaries, so everything except the
+    outputs agree bit for bit; gradients agree to rounding (the carried state gradient crosses the cut through
+    a different but equivalent sequence of operations)."""
+    from dest3d_amd import ISSM_chunk_scan_combined as op
+    names = ("x", "dt", "A", "B", "C", "D", "h0")
+    leaf = lambda: {k: t[k].detach().clone().requires_grad_() for k in names}
+    kw = dict(dt_softplus=True, return_final_states=True)
+    a = leaf()
+    y, fin = op(a["x"], a["dt"], a["A"], a["B"], a["C"], 64, D=a["D"], initial_states=a["h0"], **kw)
+    ((y.float() * t["dy"]).sum() + (fin * t["dfinal"]).sum()).backward()
+    b = leaf()
+    cut = lambda v, lo, hi: v[:, lo:hi]
+    y1, f1 = op(cut(b["x"], 0, Lh), cut(b["dt"], 0, Lh), b["A"], cut(b["B"], 0, Lh), cut(b["C"], 0, Lh), 64,
+                D=b["D"], initial_states=b["h0"], **kw)
+    y2, f2 = op(cut(b["x"], Lh, None), cut(b["dt"], Lh, None), b["A"], cut(b["B"], Lh, None), cut(b["C"], Lh, None),
+                64, D=b["D"], initial_states=f1, **kw)
+    ((y1.float() * t["dy"][:, :Lh]).sum() + (y2.float() * t["dy"][:, Lh:]).sum() + (f2 * t["dfinal"]).sum()).backward()
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([y1, y2], dim=1), y) and torch.equal(f2, fin)
+    for k in names:
+        _check(f"d{k} (split vs whole)", b[k].grad, a[k].grad, tol_sum)
+    return y, fin, a
+
+
+def test_long_sequence_bf16_shape():
+    """B=2, L=16384 (256 chunks), H=8, P=32, N=256, bf16 inputs with fp32 states: split-sequence composition at
+    full size, and the fp64 oracle on one (batch, head) over the whole length."""
+    from dest3d_amd import ISSM_chunk_scan_combined as op
+    _say("long sequence bf16 B=2 L=16384 H=8 P=32 N=256")
+    dev = "cuda"
+    I = R.make_inputs(2, 16384, 8, 32, 256, seed=1237, h0_std=0.1)
+    bf = lambda v: v.to(dev, torch.bfloat16)
+    t = dict(x=bf(I["x"]), dt=bf(I["dt_raw"]), B=bf(I["B"]), C=bf(I["C"]), A=I["A"].to(dev), D=I["D"].to(dev),
+             h0=I["h0"].to(dev), dy=I["dy"].to(dev), dfinal=I["dfinal"].to(dev))
+    _split_sequence_check(t, torch.bfloat16, 8192, 1e-2)
+    # oracle on (b, h) = (1, 5): strided views of the big tensors go straight into the operator
+    b0, h0 = 1, 5
+    sl = dict(x=t["x"][b0:b0 + 1, :, h0:h0 + 1], dt=t["dt"][b0:b0 + 1, :, h0:h0 + 1], A=t["A"][h0:h0 + 1],
+              B=t["B"][b0:b0 + 1], C=t["C"][b0:b0 + 1], D=t["D"][h0:h0 + 1], h0=t["h0"][b0:b0 + 1, h0:h0 + 1])
+    dy, df = t["dy"][b0:b0 + 1, :, h0:h0 + 1], t["dfinal"][b0:b0 + 1, h0:h0 + 1]
+    ref = {k: v.detach().double().cpu().clone().requires_grad_() for k, v in sl.items()}
+    yr, fr = R.issm_scan_sequential(ref["x"], ref["dt"], ref["A"], ref["B"], ref["C"], D=ref["D"],
+                                    initial_states=ref["h0"], dt_softplus=True)
+    ((yr * dy.double().cpu()).sum() + (fr * df.double().cpu()).sum()).backward()
+    g = {k: v.detach().requires_grad_() for k, v in sl.items()}      # keeps the strides of the views
+    yg, fg = op(g["x"], g["dt"], g["A"], g["B"], g["C"], 64, D=g["D"], initial_states=g["h0"], dt_softplus=True,
+                return_final_states=True)
+    ((yg.float() * dy).sum() + (fg * df).sum()).backward()
+    torch.cuda.synchronize()
+    _check("y", yg, yr, FWD16)
+    _check("final", fg, fr, FWD16)
+    for k in ref:
+        _check("d" + k, g[k].grad, ref[k].grad, BWD16)
+
+
+def test_large_bidirectional_fp32_shape():
+    """B=16, L=2048, H=16, P=64, N=512, fp32, both directions, h0 ~ N(0, 0.1): split-sequence composition of the
+    single-direction operator at full size, the fused bidirectional call against two single-direction calls
+    (bit-equal), and the fp64 oracle on one (batch, head)."""
+    from dest3d_amd import ISSM_biscan_combined, ISSM_chunk_scan_combined as op
+    _say("large bidirectional fp32 B=16 L=2048 H=16 P=64 N=512")
+    dev = "cuda"
+    I = R.make_inputs(16, 2048, 16, 64, 512, seed=1238, h0_std=0.1)
+    t = dict(x=I["x"].to(dev), dt=I["dt_raw"].to(dev), B=I["B"].to(dev), C=I["C"].to(dev), A=I["A"].to(dev),
+             D=I["D"].to(dev), h0=I["h0"].to(dev), dy=I["dy"].to(dev), dfinal=I["dfinal"].to(dev))
+    del I
+    y, fin, a = _split_sequence_check(t, torch.float32, 1024, 1e-5)
+    # fused bidirectional call, direction 2 = same tensors read back to front
+    names = ("x", "dt", "A", "B", "C", "D", "h0")
+    g = {k: t[k].detach().clone().requires_grad_() for k in names}
+    yf, yb, lf, lb = ISSM_biscan_combined(g["x"], g["x"], g["dt"], g["A"], g["B"], g["B"], g["C"], g["C"], 128,
+                                          D=g["D"], initial_states=g["h0"], dt_softplus=True)
+    assert torch.equal(yf, y) and torch.equal(lf, fin)
+    fl = lambda v: torch.flip(v, dims=[1]).contiguous()
+    r = {k: t[k].detach().clone().requires_grad_() for k in names}
+    y2, l2 = op(fl(r["x"]), fl(r["dt"]), r["A"], fl(r["B"]), fl(r["C"]), 128, D=r["D"], initial_states=r["h0"],
+                dt_softplus=True, return_final_states=True)
+    assert torch.equal(torch.flip(y2, dims=[1]), yb) and torch.equal(l2, lb)
+    dyb = torch.flip(t["dy"], dims=[1]) * 0.5
+    ((yf * t["dy"]).sum() + (yb * dyb).sum() + (lf * t["dfinal"]).sum() + (lb * t["dfinal"]).sum()).backward()
+    ((y2 * torch.flip(dyb, dims=[1])).sum() + (l2 * t["dfinal"]).sum()).backward()
+    torch.cuda.synchronize()
+    # d(fused) = d(direction 1 alone) + d(direction 2 alone): float addition of two bit-identical parts
+    for k in ("x", "B", "C"):
+        _check(f"d{k} fused vs sum of parts", g[k].grad, a[k].grad + r[k].grad, 1e-6)
+    for k in ("dt", "A", "D", "h0"):
+        _check(f"d{k} fused vs sum of parts", g[k].grad, a[k].grad + r[k].grad, 1e-5)
+    del g, r, a, y2, yb, yf
+    torch.cuda.empty_cache()
+    # oracle on (b, h) = (3, 7), both directions through the fused call
+    b0, hh = 3, 7
+    sl = dict(x=t["x"][b0:b0 + 1, :, hh:hh + 1], dt=t["dt"][b0:b0 + 1, :, hh:hh + 1], A=t["A"][hh:hh + 1],
+              B=t["B"][b0:b0 + 1], C=t["C"][b0:b0 + 1], D=t["D"][hh:hh + 1], h0=t["h0"][b0:b0 + 1, hh:hh + 1])
+    dy, df = t["dy"][b0:b0 + 1, :, hh:hh + 1], t["dfinal"][b0:b0 + 1, hh:hh + 1]
+    ref = {k: v.detach().double().cpu().clone().requires_grad_() for k, v in sl.items()}
+    o_ref = R.issm_biscan_ref(ref["x"], ref["x"], ref["dt"], ref["A"], ref["B"], ref["B"], ref["C"], ref["C"],
+                              D=ref["D"], initial_states=ref["h0"], dt_softplus=True)
+    w = (dy.double().cpu(), 0.5 * dy.double().cpu(), df.double().cpu(), -df.double().cpu())
+    sum((o * wi).sum() for o, wi in zip(o_ref, w)).backward()
+    gg = {k: v.detach().requires_grad_() for k, v in sl.items()}     # keeps the strides of the views
+    o = ISSM_biscan_combined(gg["x"], gg["x"], gg["dt"], gg["A"], gg["B"], gg["B"], gg["C"], gg["C"], 128,
+                             D=gg["D"], initial_states=gg["h0"], dt_softplus=True)
+    sum((oi * wi.to(dev).float()).sum() for oi, wi in zip(o, w)).backward()
+    torch.cuda.synchronize()
+    for name, ai, bi in zip(("y_f", "y_b", "last_f", "last_b"), o, o_ref):
+        _check(name, ai, bi, FWD32)
+    for k in ref:
+        _check("d" + k, gg[k].grad, ref[k].grad, BWD32)
