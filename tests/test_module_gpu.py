@@ -1,0 +1,143 @@
+"""The host-side mirror of DEST's MultiHeadISSMScan against a pure-PyTorch fp64 evaluation of the
+reference module's forward (models/dest_module.py:515-612) that uses the oracle for the scan and the
+gated RMSNorm, on the same state_dict.  Error measure and tolerances as in test_issm_gpu.py."""
+import sys
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import issm_ref as R
+
+pytestmark = pytest.mark.gpu
+FWD32, BWD32, FWD16 = 1e-4, 1e-3, 2e-2
+
+
+def _err(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    assert torch.isfinite(a).all()
+    return max(((a - b).norm() / b.norm().clamp_min(1e-300)).item(),
+               ((a - b).abs().max() / b.abs().max().clamp_min(1e-300)).item())
+
+
+def _check(name, a, b, tol):
+    e = _err(a, b)
+    print(f"    {name:28s} err={e:.3e} (tol {tol:g})", flush=True)
+    assert e <= tol, f"{name}: {e:.3e} > {tol:g}"
+
+
+def _module_ref(sd, cfg, in_key, in_query, dist, mask):
+    """dest_module.py:528-585 in the reference's own order of operations (transposed views, flipped
+    copies, two scans), in fp64, with the scan and the gated norm taken from the oracle."""
+    H, G, d_inner = cfg["nheads"], cfg["ngroups"], cfg["d_inner"]
+    P, K = d_inner // H, cfg["d_state"]
+
+    def conv(prefix, t):
+        w, b = sd[prefix + ".dwconv.weight"], sd[prefix + ".dwconv.bias"]
+        return F.silu(F.conv1d(t.transpose(1, 2), w, b, padding=3, groups=w.shape[0])).transpose(1, 2)
+
+    zxbcdt = in_key @ sd["key_proj.weight"].T
+    z, xbc, dt_tok = torch.split(zxbcdt, [d_inner, d_inner + 2 * G, H], dim=-1)
+    x, b_bias, c_bias = torch.split(conv("key_conv", xbc), [d_inner, G, G], dim=-1)
+    h0 = (in_query @ sd["query_proj.weight"].T).reshape(in_query.shape[0], K, H, P).permute(0, 2, 3, 1)
+    A = (-torch.exp(sd["A_log"]))[:, None].expand(H, K)
+    bc = dist @ sd["bc_proj.weight"].T
+    b_base, c_base = torch.split(bc, [G, G], dim=-1)
+    Bm = b_base.transpose(-1, -2) + b_bias.unsqueeze(-1)
+    Cm = c_base.transpose(-1, -2) + c_bias.unsqueeze(-1)
+    dt = F.softplus((dist @ sd["dt_proj.weight"].T).transpose(-1, -2) + dt_tok.unsqueeze(-1)
+                    + sd["dt_bias"].reshape(1, 1, -1, 1))
+    if mask is not None:
+        if mask.dtype == torch.bool:
+            dt = dt.masked_fill(mask.unsqueeze(2), 0.0)
+        else:
+            dt = dt * mask.unsqueeze(2).double()
+    hp = lambda t: t.reshape(*t.shape[:2], H, P)
+    scan = lambda x_, dt_, B_, C_: R.issm_scan_sequential(hp(x_), dt_, A, B_, C_, D=sd["D"], initial_states=h0)
+    key, last = scan(x, dt, Bm, Cm)
+    if cfg["use_biscan"]:
+        x_b, bb, cb = torch.split(conv("key_conv_back", xbc), [d_inner, G, G], dim=-1)
+        fl = lambda t: torch.flip(t, dims=[1])
+        key_b, last_b = scan(fl(x_b), fl(dt), fl(b_base.transpose(-1, -2) + bb.unsqueeze(-1)),
+                             fl(c_base.transpose(-1, -2) + cb.unsqueeze(-1)))
+        key = (key + fl(key_b)) / 2
+        last = (last + last_b) / 2
+    key = R.gated_rmsnorm_ref(key.flatten(-2), sd["key_norm.weight"], z=z, eps=1e-5, norm_before_gate=False)
+    out_key = key @ sd["out_key_proj.weight"].T
+    last = last.permute(0, 3, 1, 2).flatten(-2)
+    last = F.layer_norm(last, (d_inner,), sd["query_norm.weight"], sd["query_norm.bias"], 1e-5)
+    return out_key, last @ sd["out_query_proj.weight"].T
+
+
+@pytest.mark.parametrize("biscan,mask_kind", [(True, None), (True, "float"), (False, "bool")])
+def test_module_matches_fp64_evaluation(biscan, mask_kind):
+    from dest3d_amd.dest_module import MultiHeadISSMScan
+    print(f"[case] module mirror biscan={biscan} mask={mask_kind}", flush=True)
+    sys.stdout.flush()
+    torch.manual_seed(7)
+    Bsz, L, K, D, M, H = 2, 130, 48, 72, 16, 2                       # headdim 36 as in the detector
+    m = MultiHeadISSMScan(d_model=D, d_state=K, d_dist=M, chunk_size=256, nheads=H, expand=1, use_biscan=biscan)
+    with torch.no_grad():                                            # make every parameter matter
+        m.D.normal_()
+        m.key_norm.weight.add_(0.1 * torch.randn(D))
+        m.query_norm.bias.normal_(std=0.1)
+    g = torch.Generator().manual_seed(8)
+    ins = dict(in_key=torch.randn(Bsz, L, D, generator=g), in_query=torch.randn(Bsz, K, D, generator=g),
+               dist=0.5 * torch.randn(Bsz, L, K, M, generator=g))
+    mask = None
+    if mask_kind == "float":
+        mask = torch.rand(Bsz, L, K, generator=g)
+    elif mask_kind == "bool":
+        mask = torch.rand(Bsz, L, K, generator=g) < 0.2
+    w_key, w_query = torch.randn(Bsz, L, D, generator=g), torch.randn(Bsz, K, D, generator=g)
+
+    sd = {k: v.detach().double().clone().requires_grad_() for k, v in m.state_dict().items()}
+    rin = {k: v.double().clone().requires_grad_() for k, v in ins.items()}
+    cfg = dict(nheads=H, ngroups=1, d_inner=D, d_state=K, use_biscan=biscan)
+    ok_ref, oq_ref = _module_ref(sd, cfg, rin["in_key"], rin["in_query"], rin["dist"], mask)
+    ((ok_ref * w_key.double()).sum() + (oq_ref * w_query.double()).sum()).backward()
+
+    m = m.cuda()
+    gin = {k: v.cuda().requires_grad_() for k, v in ins.items()}
+    ok, oq = m(gin["in_key"], gin["in_query"], gin["dist"], None, mask=None if mask is None else mask.cuda())
+    ((ok * w_key.cuda()).sum() + (oq * w_query.cuda()).sum()).backward()
+    torch.cuda.synchronize()
+    _check("out_key", ok, ok_ref, FWD32)
+    _check("out_query", oq, oq_ref, FWD32)
+    for k in ins:
+        _check("d" + k, gin[k].grad, rin[k].grad, BWD32)
+    for k, p in m.named_parameters():
+        _check("d" + k, p.grad, sd[k].grad, BWD32)
+
+
+def test_six_layer_stack_bf16_at_detector_shape():
+    """Six mirror layers at the detector's decoder shape (d_model 288, 8 heads of 36, K = 256 queries,
+    L = 1024 keys, batch 8, d_dist 16), bf16 forward + backward, against the same stack in fp32 on the
+    bf16-rounded weights and inputs.  The fp32 stack is pinned by test_module_matches_fp64_evaluation."""
+    from dest3d_amd.dest_module import MultiHeadISSMScan
+    print("[case] six-layer bf16 stack B=8 L=1024 K=256 d_model=288", flush=True)
+    torch.manual_seed(11)
+    layers = torch.nn.ModuleList(MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8,
+                                                   expand=1) for _ in range(6)).cuda().bfloat16()
+    ref = torch.nn.ModuleList(MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8,
+                                                expand=1) for _ in range(6)).cuda()
+    ref.load_state_dict({k: v.float() for k, v in layers.state_dict().items()})
+    g = torch.Generator().manual_seed(12)
+    key = torch.randn(8, 1024, 288, generator=g).bfloat16().cuda()
+    query = torch.randn(8, 256, 288, generator=g).bfloat16().cuda()
+    dist = (0.5 * torch.randn(8, 1024, 256, 16, generator=g)).bfloat16().cuda()
+
+    def run(stack, k, q, d):
+        k, q = k.clone().requires_grad_(), q.clone().requires_grad_()
+        hk, hq = k, q
+        for layer in stack:                                   # residual stack, as the decoder layers chain
+            ok, oq = layer(hk, hq, d, None)
+            hk, hq = hk + ok, hq + oq
+        (hk.float().square().mean() + hq.float().square().mean()).backward()
+        return hk, hq, k.grad, q.grad
+
+    o16 = run(layers, key, query, dist)
+    o32 = run(ref, key.float(), query.float(), dist.float())
+    torch.cuda.synchronize()
+    for name, a, b in zip(("out_key", "out_query", "d in_key", "d in_query"), o16, o32):
+        _check(name, a, b, 5e-2)
