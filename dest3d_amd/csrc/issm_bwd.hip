@@ -70,12 +70,12 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
 
   int n = wave * 16 + cm;
   bool vn = n < p.N;
-  int prow[16];
+  RowMap rm;
   float raw[16], cv[16];
   if (dstates) {
-    lane_rows(p, u, g4, vn, prow);
-    lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-    lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+    rm = make_rowmap(p, u, g4, 0);
+    lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+    lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   }
   {
     float dv[CS * PT * 16 / NTHREADS], xv[CS * PT * 16 / NTHREADS];
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     float ct[16];
     {
       float dtp[16], cs[16], dummy[16];
-      lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
+      lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k) ct[k] = cv[k] * ex2(cs[k]);
     }
@@ -114,9 +114,9 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
       vn = n < p.N;
-      lane_rows(p, u, g4, vn, prow);
-      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+      rm = make_rowmap(p, u, g4, n0 + NS);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
     f4 acc[PT];
 #pragma unroll
@@ -437,10 +437,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     float dtp[16], cs[16], dfac[16];
     float last;
     {
-      int prow[16];
-#pragma unroll
-      for (int k = 0; k < 16; ++k) prow[k] = rowk(k) < lim ? 0 : -1;
-      last = lane_prep<true>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dfac);
+      const RowMap rm = make_rowmap(p, u, g4, ns * NS);
+      last = lane_prep<true>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dfac);
     }
     float Bd[16];
 #pragma unroll
@@ -599,12 +597,12 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
 
   int n = wave * 16 + cm;
   bool vn = n < p.N;
-  int prow[16];
-  lane_rows(p, u, g4, vn, prow);
+  RowMap rm;
+  rm = make_rowmap(p, u, g4, 0);
   float raw[16], bv[16];
   PnRegs<PT> sv;
-  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
   pn_load<PT>(p, ds, 0, sv);
   {
     float dv[CS * PT * 16 / NTHREADS];
@@ -621,7 +619,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     {
       float dtp[16], cs[16], dummy[16];
-      const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
+      const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k)
         s.bt[lane_row(k, g4) * LDN + wave * 16 + cm] = bv[k] * dtp[k] * ex2(last - cs[k]);
@@ -630,9 +628,9 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
       vn = n < p.N;
-      lane_rows(p, u, g4, vn, prow);
-      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
+      rm = make_rowmap(p, u, g4, n0 + NS);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       pn_load<PT>(p, ds, n0 + NS, sv);
     }
     __syncthreads();

@@ -20,6 +20,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace issm {
 
@@ -225,31 +226,58 @@ __device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
   return v;
 }
 
-// Physical rows of the lane's 16 chunk rows (or -1 past the end of the sequence / invalid column).
-__device__ __forceinline__ void lane_rows(const KP& p, const Unit& u, int g4, bool vn, int (&prow)[16]) {
-#pragma unroll
-  for (int k = 0; k < 16; ++k) {
-    const int tt = u.c * CS + lane_row(k, g4);
-    prow[k] = (vn && tt < p.L) ? phys_row(p, u.dir, tt) : -1;
-  }
+// Where the lane's 16 chunk rows live in memory.  Element k = 4J + j is chunk row 16J + 4 g4 + j,
+// i.e. physical row base + step * (16J + j): a per-lane part (base) plus a part that is the same
+// for the whole wave, so that in a full chunk the address of every element is a scalar base
+// plus ONE per-lane offset.  `full` (uniform) says that all 64 rows and all 64 columns of the
+// slice exist; otherwise rows >= nvalid and lanes with !vn read as zero.
+struct RowMap {
+  int base, step, nvalid;
+  bool full;
+};
+__device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4, int n0) {
+  RowMap r;
+  const int t0 = u.c * CS + 4 * g4;
+  r.base = u.dir ? p.L - 1 - t0 : t0;
+  r.step = u.dir ? -1 : 1;
+  r.nvalid = min(CS, p.L - u.c * CS);
+  r.full = (r.nvalid == CS) && (n0 + NS <= p.N);
+  return r;
 }
 // Lane's 16 values of column n of a (B,L,G|H,N)-shaped tensor.
 template <bool BF>
-__device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third, int n, const int (&prow)[16],
-                                             float (&out)[16]) {
-  int off[16];
+__device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third, int n, bool vn, int g4,
+                                             const RowMap& rm, float (&out)[16]) {
+  typedef typename std::conditional<BF, uint16_t, float>::type T;
+  const T* q = (const T*)t.ptr + ((long)b * t.s0 + (long)third * t.s2);
+  const long ss = (long)rm.step * t.s1;  // uniform
+  T r[16];
+  if (rm.full) {
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n);
 #pragma unroll
-  for (int k = 0; k < 16; ++k) off[k] = prow[k] < 0 ? -1 : prow[k] * (int)t.s1 + n;
-  gload<BF, 16>(t.ptr, (long)b * t.s0 + (long)third * t.s2, off, out);
+    for (int k = 0; k < 16; ++k) r[k] = (q + (16 * (k >> 2) + (k & 3)) * ss)[lo];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) out[k] = BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k];
+  } else {
+    bool ok[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      ok[k] = vn && lane_row(k, g4) < rm.nvalid;
+      const long o = ok[k] ? (long)rm.base * t.s1 + n + (16 * (k >> 2) + (k & 3)) * ss : 0;
+      r[k] = q[o];
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) out[k] = ok[k] ? (BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k]) : 0.0f;
+  }
 }
 // dt transform (bias -> softplus -> clamp) of the lane's rows and the inclusive running sum of
 // dt' * A * log2(e) down the chunk (so decays are exp2 of differences).  `raw` holds the loaded
 // dt values.  dfac (if WANT_DFAC) receives d dt' / d dt: the softplus derivative times the clamp
 // mask.  Returns the chunk total (running sum at row 63), the same on all lanes of the column.
 template <bool WANT_DFAC>
-__device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, int cm, int g4,
-                                           const int (&prow)[16], const float (&raw)[16], float (&dtp)[16],
-                                           float (&cs)[16], float (&dfac)[16]) {
+__device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, int cm, int g4, const RowMap& rm,
+                                           const float (&raw)[16], float (&dtp)[16], float (&cs)[16],
+                                           float (&dfac)[16]) {
   const float A2 = vn ? p.A[h * p.N + n] * LOG2E : 0.0f;
   const float bias = (vn && p.dt_bias) ? p.dt_bias[h * p.N + n] : 0.0f;
   if (p.flags & F_SOFTPLUS) {
@@ -257,16 +285,21 @@ __device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, i
     for (int k = 0; k < 16; ++k) {
       const float pre = raw[k] + bias;
       const float sp = softplus_(pre);
-      dtp[k] = prow[k] < 0 ? 0.0f : fminf(fmaxf(sp, p.dt_min), p.dt_max);
+      dtp[k] = fminf(fmaxf(sp, p.dt_min), p.dt_max);
       if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : (pre <= 20.0f ? sigmoidf_(pre) : 1.0f);
     }
   } else {
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       const float sp = raw[k] + bias;
-      dtp[k] = prow[k] < 0 ? 0.0f : fminf(fmaxf(sp, p.dt_min), p.dt_max);
+      dtp[k] = fminf(fmaxf(sp, p.dt_min), p.dt_max);
       if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : 1.0f;
     }
+  }
+  if (!rm.full) {  // rows past the end of the sequence and absent columns behave as dt' = 0
+#pragma unroll
+    for (int k = 0; k < 16; ++k)
+      if (!(vn && lane_row(k, g4) < rm.nvalid)) dtp[k] = 0.0f;
   }
   float carry = 0.0f;
 #pragma unroll

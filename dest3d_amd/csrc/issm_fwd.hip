@@ -97,12 +97,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   // column-lane operands of the first slice and the x tile are in flight together
   int n = wave * 16 + cm;
   bool vn = n < p.N;
-  int prow[16];
-  lane_rows(p, u, g4, vn, prow);
+  RowMap rm;
+  rm = make_rowmap(p, u, g4, 0);
   float raw[16], bv[16], cv[16];
-  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
-  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   {
     float xv[CS * PT * 16 / NTHREADS];
     lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     float dtp[16], cs[16], dummy[16];
-    const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
+    const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
     float bd[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) bd[k] = bv[k] * dtp[k];
@@ -133,10 +133,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
     if (n0 + NS < p.N) {  // prefetch the next slice
       n = n0 + NS + wave * 16 + cm;
       vn = n < p.N;
-      lane_rows(p, u, g4, vn, prow);
-      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, prow, bv);
-      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+      rm = make_rowmap(p, u, g4, n0 + NS);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
     __syncthreads();  // x tile (first slice) and the slice's LDS tiles are complete
 
@@ -307,12 +307,12 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
 
   int n = wave * 16 + cm;
   bool vn = n < p.N;
-  int prow[16];
-  lane_rows(p, u, g4, vn, prow);
+  RowMap rm;
+  rm = make_rowmap(p, u, g4, 0);
   float raw[16], cv[16];
   PnRegs<PT> hv;
-  lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+  lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   pn_load<PT>(p, hsrc, 0, hv);
   {
     float xv[CS * PT * 16 / NTHREADS];
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     {
       float dtp[16], cs[16], dummy[16];
-      lane_prep<false>(p, u.h, n, vn, cm, g4, prow, raw, dtp, cs, dummy);
+      lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
     }
@@ -337,9 +337,9 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
       vn = n < p.N;
-      lane_rows(p, u, g4, vn, prow);
-      lane_load_ln<DTB>(p.dt, u.b, u.h, n, prow, raw);
-      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, prow, cv);
+      rm = make_rowmap(p, u, g4, n0 + NS);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
       pn_load<PT>(p, hsrc, n0 + NS, hv);
     }
     __syncthreads();
