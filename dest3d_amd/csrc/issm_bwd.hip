@@ -244,32 +244,30 @@ struct BwdChunkSmem {
   float dbc[32 * NTHREADS];  // per-lane dB / dC accumulators [k][tid]
 };
 
-// One level (w = 2^LV) of the row hierarchy for F and G.  op[k] = Bd * exp2(ref - cs) on lower
-// rows (right factor of the decay), C * exp2(cs - ref) on upper rows (left factor); ref = cs of
-// the last row of the lower half of the row's 2w-block, fetched from the lane that owns it.  Rows
-// that are upper at this level receive their F contribution (x2), lower rows their G
-// contribution (e1).
+// F[l] = sum_{s<=l} dM[l,s] Bd[s] exp2(cs[l]-cs[s]) and G[s] = sum_{l>=s} dM[l,s] C[l] exp2(cs[l]-cs[s]) per state
+// column, accumulated into x2 (F) and e1 (G).  A pair (l > s) is handled at the level w = highest set
+// bit of (l xor s); the lane's rows are 16J + 4 g4 + j, so
+//   w = 32, 16  ->  the pair lies in different 16-row tiles: role (upper / lower half of the 2w-block)
+//                   is a compile-time function of J;
+//   w = 8, 4    ->  same tile, different lane groups g4: role depends on g4;
+//   w = 2, 1, 0 ->  both rows belong to the same lane: evaluated directly, one exp2 per pair.
+// At the levels >= 4 a row contributes  op = Bd * exp2(ref - cs)  if it is in the lower half of its
+// block and  op = C * exp2(cs - ref)  if it is in the upper half (ref = cs of the last row of the lower
+// half): both factors are <= 1.
 
+// Levels 32 (LV = 5) and 16 (LV = 4): products of 16x16 blocks of dM with the operand rows.
 template <int LV>
-__device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
-                                          const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm, int g4) {
-  constexpr int w = 1 << LV;
+__device__ __forceinline__ void bwd_big_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
+                                              const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm,
+                                              int g4) {
   float op[16], ee[16];
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    float r01, r23;
-    if (LV == 0) { r01 = cs[4 * J]; r23 = cs[4 * J + 2]; }
-    else if (LV == 1) r01 = r23 = cs[4 * J + 1];
-    else if (LV == 2) r01 = r23 = __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64);
-    else if (LV == 3) r01 = r23 = __shfl(cs[4 * J + 3], cm + 16, 64);
-    else if (LV == 4) r01 = r23 = __shfl(cs[4 * (J & 2) + 3], cm + 48, 64);
-    else r01 = r23 = __shfl(cs[7], cm + 48, 64);
+    const float ref = LV == 4 ? __shfl(cs[4 * (J & 2) + 3], cm + 48, 64) : __shfl(cs[7], cm + 48, 64);
+    const bool upper = LV == 4 ? (J & 1) : (J & 2);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const bool upper = LV == 0 ? (j & 1) : LV == 1 ? (j & 2) : LV == 2 ? (g4 & 1) : LV == 3 ? (g4 & 2)
-                                                                            : LV == 4 ? (J & 1) : (J & 2);
-      const float ref = j < 2 ? r01 : r23;
       const float e = ex2(upper ? cs[k] - ref : ref - cs[k]);
       ee[k] = e;
       op[k] = (upper ? Cv[k] : Bd[k]) * e;
@@ -299,7 +297,7 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
         if (I >= 2) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
         else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
       }
-    } else if (LV == 4) {
+    } else {
       if (I & 1) {
         const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + (I - 1) * 16 + 4 * g4);
 #pragma unroll
@@ -314,27 +312,78 @@ __device__ __forceinline__ void bwd_level(const float (&cs)[16], const float (&B
         if (I & 1) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
         else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
       }
-    } else {
-      // inside the diagonal tile: contraction rows kr = 4 g4 + j, restricted to the 2w-block of the
-      // output row (lane cm); lower rows feed F, upper rows feed G
-      f4 gw = {0, 0, 0, 0};
-      const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + I * 16 + 4 * g4);
-      const float* ap = dms + (I * 16 + 4 * g4) * LDC + I * 16 + cm;
+    }
+  }
+}
+
+// Levels 8 (LV = 3) and 4 (LV = 2), inside a diagonal 16x16 tile.  With T_w[i][j] = dM[max(i,j)][min(i,j)] if
+// the pair (i, j) belongs to level w and 0 otherwise (a symmetric matrix), Z = T_w . op holds the F sum on
+// the upper rows and the G sum on the lower rows: one product serves both, and no operand needs masking,
+// because T_w pairs an upper row only with lower rows of its block and vice versa.
+template <int LV>
+__device__ __forceinline__ void bwd_mid_level(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
+                                              const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm,
+                                              int g4) {
+  const bool up = LV == 2 ? (g4 & 1) : (g4 & 2);  // role of the lane's rows 4 g4 + j
+  const float upf = up ? 1.0f : 0.0f, lof = up ? 0.0f : 1.0f;
+  // A operand: row i = cm of T_w, columns kk = 4 g4 + jj.  Non-zero only where (i, kk) is a level-w pair.
+  const int cg = cm >> 2;
+  const bool iup = LV == 2 ? (cg & 1) : (cg & 2);
+  const bool nz = LV == 2 ? (g4 == (cg ^ 1)) : ((g4 >> 1) != (cg >> 1));
+  const int a_base = iup ? cm * LDC + 4 * g4 : 4 * g4 * LDC + cm;  // dM[i][kk] (i upper) or dM[kk][i] (i lower)
+  const int a_step = iup ? 1 : LDC;
+  float op[16], ee[16];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int kr = 4 * g4 + j;
-        const bool same = LV == 3 || ((cm ^ kr) < 2 * w);
-        const bool kup = (kr >> LV) & 1;
-        acc = mfma4((same && !kup) ? av[j] : 0.0f, op[4 * I + j], acc);
-        gw = mfma4((same && kup) ? ap[j * LDC] : 0.0f, op[4 * I + j], gw);
-      }
+  for (int J = 0; J < 4; ++J) {
+    const float ref = LV == 2 ? __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64) : __shfl(cs[4 * J + 3], cm + 16, 64);
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const bool upper = ((4 * g4 + rr) >> LV) & 1;
-        // (value selects, not a branch between the two arrays: a select between their addresses
-        // would force both arrays out of registers)
-        x2[4 * I + rr] += upper ? ee[4 * I + rr] * acc[rr] : 0.0f;
-        e1[4 * I + rr] += upper ? 0.0f : ee[4 * I + rr] * gw[rr];
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * J + j;
+      const float d = cs[k] - ref;
+      const float e = ex2(up ? d : -d);
+      ee[k] = e;
+      op[k] = (up ? Cv[k] : Bd[k]) * e;
+    }
+  }
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    const float* ap = dms + I * (16 * LDC + 16) + a_base;
+    f4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const float a = ap[jj * a_step];
+      acc = mfma4(nz ? a : 0.0f, op[4 * I + jj], acc);
+    }
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const float v = ee[4 * I + rr] * acc[rr];
+      x2[4 * I + rr] = fmaf(v, upf, x2[4 * I + rr]);
+      e1[4 * I + rr] = fmaf(v, lof, e1[4 * I + rr]);
+    }
+  }
+}
+
+// Levels 2, 1 and the diagonal: the pairs inside each group of four consecutive rows owned by the lane.
+__device__ __forceinline__ void bwd_small_levels(const float (&cs)[16], const float (&Bd)[16], const float (&Cv)[16],
+                                                 const float* __restrict__ dms, float (&e1)[16], float (&x2)[16],
+                                                 int g4) {
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    const float* blk = dms + (16 * J + 4 * g4) * LDC + 16 * J + 4 * g4;  // dM[row jl][col js] of the group
+    f4 m[4];
+#pragma unroll
+    for (int jl = 0; jl < 4; ++jl) m[jl] = *(const f4*)(blk + jl * LDC);
+#pragma unroll
+    for (int jl = 0; jl < 4; ++jl) {
+      const int kl = 4 * J + jl;
+      e1[kl] = fmaf(m[jl][jl], Cv[kl], e1[kl]);
+      x2[kl] = fmaf(m[jl][jl], Bd[kl], x2[kl]);
+#pragma unroll
+      for (int js = 0; js < jl; ++js) {
+        const int ks = 4 * J + js;
+        const float wgt = m[jl][js] * ex2(cs[kl] - cs[ks]);
+        e1[ks] = fmaf(wgt, Cv[kl], e1[ks]);
+        x2[kl] = fmaf(wgt, Bd[ks], x2[kl]);
       }
     }
   }
@@ -466,10 +515,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int k = 4 * I + rr, row = 16 * I + 4 * gq + rr;
-        const float dd = s.dms[row * LDC + row];
-        e1[k] = ex2(last - cs[k]) * q[rr] + dd * Cv[k];
-        x2[k] = ex2(cs[k]) * r[rr] + dd * Bd[k];
+        const int k = 4 * I + rr;
+        e1[k] = ex2(last - cs[k]) * q[rr];
+        x2[k] = ex2(cs[k]) * r[rr];
       }
     }
 
@@ -477,27 +525,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<5>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_big_level<5>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<4>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_big_level<4>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<3>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_mid_level<3>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<2>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_mid_level<2>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<1>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_level<0>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_small_levels(cs, Bd, Cv, s.dms, e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase: everything below is local to the lane except the scans over rows
