@@ -57,7 +57,7 @@ struct BwdStSmem {
 // dH[p][n] = sum_l dy[l][p] * C[l][n] exp2(cs[l][n]): contraction over rows, so the B operand
 // comes straight from the registers of the column-lane layout; each wave walks its own 16
 // columns of every 64-column slice without any barrier after the dy / x tiles are staged.
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __restrict__ dy_ws,
                                                           float* __restrict__ dstates, float* __restrict__ dm) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -69,11 +69,11 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
 
   int n = wave * 16 + cm;
-  bool vn = n < p.N;
+  bool vn = FULL || n < p.N;
   RowMap rm;
   float raw[16], cv[16];
   if (dstates) {
-    rm = make_rowmap(p, u, g4, 0);
+    rm = make_rowmap<FULL>(p, u, g4, 0);
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
     lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   }
@@ -113,8 +113,8 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     const bool vn_cur = vn;
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
-      vn = n < p.N;
-      rm = make_rowmap(p, u, g4, n0 + NS);
+      vn = FULL || n < p.N;
+      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
@@ -390,7 +390,7 @@ __device__ __forceinline__ void bwd_small_levels(const float (&cs)[16], const fl
 }
 
 // partA, partBias: (Bt*nc, H, N) per-unit partial sums of dA and ddt_bias
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws,
                                                            const float* __restrict__ states,
                                                            const float* __restrict__ dstates,
@@ -417,55 +417,28 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   u.bt = u.b * p.ndir + u.dir;
   u.h = u.g * p.hpg;
   const int n = ns * NS + wave * 16 + cm;
-  const bool vn = n < p.N;
+  const bool vn = FULL || n < p.N;
 
-  // The lane's rows are 16J + 4 g4 + j; their physical rows form an arithmetic progression:
-  // row index k -> r0 + sgn * (16J + j), valid while 16J + j < lim (0 valid rows if the column is absent).
-  const int t0 = u.c * CS + 4 * g4;
-  const int r0 = u.dir ? p.L - 1 - t0 : t0, sgn = u.dir ? -1 : 1;
-  const int lim = vn ? p.L - t0 : 0;
+  // rows past the end of the sequence and absent columns: lane_row(k) >= lim
+  const RowMap rm = make_rowmap<FULL>(p, u, g4, ns * NS);
+  const int lim = vn ? rm.nvalid - 4 * g4 : 0;
   auto rowk = [&](int k) { return 16 * (k >> 2) + (k & 3); };
-  // nn is re-materialised per head (opaque to the optimiser) so that the 16-element offset arrays are
-  // recomputed where they are used instead of being hoisted out of the head loop into registers
-  int nn = n;
-  auto offk = [&](int k, int stride) { return rowk(k) < lim ? (r0 + sgn * rowk(k)) * stride + nn : -1; };
+  const bool pn_full = rm.full && p.P == PT * 16;
 
   float Bv[16], Cv[16];
-  {
-    const TensorD& tb = p.Bm[u.dir];
-    const TensorD& tc = p.Cm[u.dir];
-    int ob[16], oc[16];
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      ob[k] = offk(k, (int)tb.s1);
-      oc[k] = offk(k, (int)tc.s1);
-    }
-    gload<IOB, 16>(tb.ptr, (long)u.b * tb.s0 + (long)u.g * tb.s2, ob, Bv);
-    gload<IOB, 16>(tc.ptr, (long)u.b * tc.s0 + (long)u.g * tc.s2, oc, Cv);
-  }
+  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);
+  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, Cv);
   // dB / dC accumulators over the heads of the group: private to the lane, kept in LDS
 #pragma unroll
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
   for (int hh = 0; hh < p.hpg; ++hh) {
     u.h = u.g * p.hpg + hh;
-    asm volatile("" : "+v"(nn));
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
-    {
-      int od[16];
-#pragma unroll
-      for (int k = 0; k < 16; ++k) od[k] = offk(k, (int)p.dt.s1);
-      gload<DTB, 16>(p.dt.ptr, (long)u.b * p.dt.s0 + (long)u.h * p.dt.s2, od, raw);
-      int os[KP_];
-#pragma unroll
-      for (int q = 0; q < KP_; ++q) {
-        const int pp = 16 * (q >> 2) + 4 * g4 + (q & 3);
-        os[q] = (vn && pp < p.P) ? pp * p.N + nn : -1;
-      }
-      gload<false, KP_>(dstates, dst_off(p, u.bt, u.c, u.h), os, dsv);
-      gload<false, KP_>(states, st_off(p, u.bt, u.c, u.h), os, hv);
-    }
+    lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+    lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
+    lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
     {
       float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
       f4 mv[4];
@@ -486,7 +459,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     float dtp[16], cs[16], dfac[16];
     float last;
     {
-      const RowMap rm = make_rowmap(p, u, g4, ns * NS);
       last = lane_prep<true>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dfac);
     }
     float Bd[16];
@@ -546,13 +518,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
 
     // ---- column phase: everything below is local to the lane except the scans over rows
     pin16(e1); pin16(x2);
-    asm volatile("" : "+v"(nn));
-    int oddt[16];
     float old[16];
-    const long ddt_base = (long)u.b * p.ddt.s0 + (long)u.h * p.ddt.s2;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) oddt[k] = p.ddt.ptr ? offk(k, (int)p.ddt.s1) : -1;
-    if (p.dir0 > 0) gload<DTB, 16>(p.ddt.ptr, ddt_base, oddt, old);
+    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     float dcs[16], val[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -586,10 +553,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       const float da = dcs[k];
       sumA += da * dtp[k];
       val[k] = (val[k] + da * An) * dfac[k];
-      if (rowk(k) < lim) sumB += val[k];
+      if (rm.full || rowk(k) < lim) sumB += val[k];
       if (p.dir0 > 0) val[k] += old[k];
     }
-    gstore<DTB, 16>(const_cast<void*>(p.ddt.ptr), ddt_base, oddt, val);
+    if (p.ddt.ptr) lane_store_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, val);
     sumA = scan_g_incl(sumA, g4);
     sumB = scan_g_incl(sumB, g4);
     if (g4 == 3 && vn) {
@@ -599,19 +566,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   }
 
   {
-    const TensorD& tB = p.dB[u.dir];
-    const TensorD& tC = p.dC[u.dir];
-    int ob[16], oc[16];
     float vb[16], vc[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      ob[k] = tB.ptr ? offk(k, (int)tB.s1) : -1;
-      oc[k] = tC.ptr ? offk(k, (int)tC.s1) : -1;
       vb[k] = s.dbc[k * NTHREADS + tid];
       vc[k] = s.dbc[(16 + k) * NTHREADS + tid];
     }
-    gstore<IOB, 16>(const_cast<void*>(tB.ptr), (long)u.b * tB.s0 + (long)u.g * tB.s2, ob, vb);
-    gstore<IOB, 16>(const_cast<void*>(tC.ptr), (long)u.b * tC.s0 + (long)u.g * tC.s2, oc, vc);
+    if (p.dB[u.dir].ptr) lane_store_ln<IOB>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, vb);
+    if (p.dC[u.dir].ptr) lane_store_ln<IOB>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
   }
 }
 
@@ -626,7 +588,7 @@ struct BwdDxSmem {
 };
 
 // partD: (Bt*nc*H, P) per-unit sums over rows of dy*x
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restrict__ dy_ws,
                                                      const float* __restrict__ dstates,
                                                      const float* __restrict__ cabt, float* __restrict__ partD) {
@@ -640,9 +602,9 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   const float* ds = dstates + dst_off(p, u.bt, u.c, u.h);
 
   int n = wave * 16 + cm;
-  bool vn = n < p.N;
+  bool vn = FULL || n < p.N;
   RowMap rm;
-  rm = make_rowmap(p, u, g4, 0);
+  rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], bv[16];
   PnRegs<PT> sv;
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
@@ -671,8 +633,8 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
     pn_store<PT>(sv, s.dss);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
-      vn = n < p.N;
-      rm = make_rowmap(p, u, g4, n0 + NS);
+      vn = FULL || n < p.N;
+      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
       lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       pn_load<PT>(p, ds, n0 + NS, sv);
@@ -795,10 +757,10 @@ int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t s
 
 int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* dm, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+  ISSM_DISPATCH(p, {
     const size_t sm = sizeof(BwdStSmem<PT_>);
-    if (int e = set_lds(k_bwd_dstates<PT_, IOB_, DTB_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_dstates<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
+    if (int e = set_lds(k_bwd_dstates<PT_, IOB_, DTB_, FULL_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_dstates<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
   });
   return (int)hipGetLastError();
 }
@@ -813,10 +775,10 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
 int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
                      const float* g_last, float* partA, float* partBias, hipStream_t st) {
   const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
-  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+  ISSM_DISPATCH(p, {
     const size_t sm = sizeof(BwdChunkSmem<PT_>);
-    if (int e = set_lds(k_bwd_chunk<PT_, IOB_, DTB_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_chunk<PT_, IOB_, DTB_>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
+    if (int e = set_lds(k_bwd_chunk<PT_, IOB_, DTB_, FULL_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk<PT_, IOB_, DTB_, FULL_>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
                        dm, g_last, partA, partBias);
   });
   return (int)hipGetLastError();
@@ -825,10 +787,10 @@ int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const
 int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const float* cabt, float* partD,
                   hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+  ISSM_DISPATCH(p, {
     const size_t sm = sizeof(BwdDxSmem<PT_>);
-    if (int e = set_lds(k_bwd_dx<PT_, IOB_, DTB_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_dx<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
+    if (int e = set_lds(k_bwd_dx<PT_, IOB_, DTB_, FULL_>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_dx<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
   });
   return (int)hipGetLastError();
 }

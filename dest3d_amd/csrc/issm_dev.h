@@ -229,19 +229,21 @@ __device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
 // Where the lane's 16 chunk rows live in memory.  Element k = 4J + j is chunk row 16J + 4 g4 + j,
 // i.e. physical row base + step * (16J + j): a per-lane part (base) plus a part that is the same
 // for the whole wave, so that in a full chunk the address of every element is a scalar base
-// plus ONE per-lane offset.  `full` (uniform) says that all 64 rows and all 64 columns of the
-// slice exist; otherwise rows >= nvalid and lanes with !vn read as zero.
+// plus ONE per-lane offset.  `full` (a compile-time constant of the kernel variant) says that all 64
+// rows and all 64 columns of every slice exist; otherwise rows >= nvalid and lanes with !vn read as zero.
 struct RowMap {
   int base, step, nvalid;
   bool full;
 };
+template <bool FULL>
 __device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4, int n0) {
   RowMap r;
   const int t0 = u.c * CS + 4 * g4;
   r.base = u.dir ? p.L - 1 - t0 : t0;
   r.step = u.dir ? -1 : 1;
   r.nvalid = min(CS, p.L - u.c * CS);
-  r.full = (r.nvalid == CS) && (n0 + NS <= p.N);
+  // FULL kernels are only launched when every chunk and every column slice is complete
+  r.full = FULL;
   return r;
 }
 // Lane's 16 values of column n of a (B,L,G|H,N)-shaped tensor.
@@ -250,7 +252,10 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
                                              const RowMap& rm, float (&out)[16]) {
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   const T* q = (const T*)t.ptr + ((long)b * t.s0 + (long)third * t.s2);
-  const long ss = (long)rm.step * t.s1;  // uniform
+  long ss = (long)rm.step * t.s1;  // uniform
+  // opaque to the optimiser: the 16 row offsets are derived here, next to their use, instead of being
+  // hoisted out of an enclosing loop into (scarce) scalar registers
+  asm volatile("" : "+s"(ss));
   T r[16];
   if (rm.full) {
     const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n);
@@ -268,6 +273,53 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
     }
 #pragma unroll
     for (int k = 0; k < 16; ++k) out[k] = ok[k] ? (BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k]) : 0.0f;
+  }
+}
+// Store of the lane's 16 values to column n of a (B,L,G|H,N)-shaped tensor (absent rows / columns skipped).
+template <bool BF>
+__device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third, int n, bool vn, int g4,
+                                              const RowMap& rm, const float (&v)[16]) {
+  typedef typename std::conditional<BF, uint16_t, float>::type T;
+  T* q = (T*)const_cast<void*>(t.ptr) + ((long)b * t.s0 + (long)third * t.s2);
+  long ss = (long)rm.step * t.s1;
+  asm volatile("" : "+s"(ss));
+  if (rm.full) {
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      T* d = q + (16 * (k >> 2) + (k & 3)) * ss;
+      if (BF) d[lo] = (T)f_to_bf16(v[k]); else d[lo] = (T)v[k];
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (vn && lane_row(k, g4) < rm.nvalid) {
+        T* d = q + ((long)rm.base * t.s1 + n + (16 * (k >> 2) + (k & 3)) * ss);
+        if (BF) *d = (T)f_to_bf16(v[k]); else *d = (T)v[k];
+      }
+    }
+  }
+}
+// Lane's values of column n of a (P x N) fp32 slab: index q <-> row 16 (q >> 2) + 4 g4 + (q & 3).
+template <int CNT>
+__device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int P, int N, int n, bool vn, int g4,
+                                             bool full, float (&out)[CNT]) {
+  asm volatile("" : "+s"(N));
+  if (full) {
+    const unsigned lo = (unsigned)(4 * g4 * N + n);
+#pragma unroll
+    for (int q = 0; q < CNT; ++q) out[q] = (src + (16 * (q >> 2) + (q & 3)) * N)[lo];
+  } else {
+    float r[CNT];
+    bool ok[CNT];
+#pragma unroll
+    for (int q = 0; q < CNT; ++q) {
+      const int pp = 16 * (q >> 2) + 4 * g4 + (q & 3);
+      ok[q] = vn && pp < P;
+      r[q] = src[ok[q] ? (long)pp * N + n : 0];
+    }
+#pragma unroll
+    for (int q = 0; q < CNT; ++q) out[q] = ok[q] ? r[q] : 0.0f;
   }
 }
 // dt transform (bias -> softplus -> clamp) of the lane's rows and the inclusive running sum of
@@ -322,27 +374,69 @@ __device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, i
 // ------------------------------------------------------------------ cooperative tile loaders
 // The unit's (64 x P) tile of a (B,L,H,P) tensor, zero padded to 16*PT columns: registers, then
 // LDS dst[l][p] (leading dimension ld).  Element e = tid + 256 i is (l, p) = (e / 16PT, e % 16PT).
+// Thread `tid` owns PT groups of four adjacent columns: group i is element e4 = tid + 256 i, i.e.
+// (l, p) = (e4 / 4PT, 4 (e4 % 4PT)).  When the tensor allows it (uniform test) a group is one 8- or 16-byte
+// access.
+__device__ __forceinline__ bool lp_vec_ok(const KP& p, const TensorD& t, int esize) {
+  return ((p.P & 3) == 0) && (((t.s0 | t.s1 | t.s2) & 3) == 0) && ((((uintptr_t)t.ptr) & (4 * esize - 1)) == 0);
+}
 template <bool BF, int PT>
 __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const TensorD& t,
                                         float (&v)[CS * PT * 16 / NTHREADS], int tid = threadIdx.x) {
-  constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
-  int off[CNT];
+  constexpr int G4 = 4 * PT;  // groups per row
+  typedef typename std::conditional<BF, uint16_t, float>::type T;
+  const T* q = (const T*)t.ptr + ((long)u.b * t.s0 + (long)u.h * t.s2);
+  const int nvalid = min(CS, p.L - u.c * CS);
+  const long ss = (long)(u.dir ? -1 : 1) * t.s1;
+  const long r0 = (long)(u.dir ? p.L - 1 - u.c * CS : u.c * CS) * t.s1;
+  if (lp_vec_ok(p, t, sizeof(T))) {
+    typedef typename std::conditional<BF, uint2, f4>::type V;
+    V r[PT];
+    bool ok[PT];
 #pragma unroll
-  for (int i = 0; i < CNT; ++i) {
-    const int e = tid + i * NTHREADS;
-    const int l = e / PPAD, pp = e % PPAD, tt = u.c * CS + l;
-    off[i] = ((pp < p.P) && (tt < p.L)) ? phys_row(p, u.dir, tt) * (int)t.s1 + pp : -1;
+    for (int i = 0; i < PT; ++i) {
+      const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
+      ok[i] = p4 < p.P && l < nvalid;
+      r[i] = *(const V*)(q + (ok[i] ? r0 + l * ss + p4 : 0));
+    }
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      if (BF) {
+        const uint2 w = *(const uint2*)&r[i];
+        v[4 * i + 0] = ok[i] ? __uint_as_float(w.x << 16) : 0.0f;
+        v[4 * i + 1] = ok[i] ? __uint_as_float(w.x & 0xffff0000u) : 0.0f;
+        v[4 * i + 2] = ok[i] ? __uint_as_float(w.y << 16) : 0.0f;
+        v[4 * i + 3] = ok[i] ? __uint_as_float(w.y & 0xffff0000u) : 0.0f;
+      } else {
+        const f4 w = *(const f4*)&r[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[4 * i + j] = ok[i] ? w[j] : 0.0f;
+      }
+    }
+  } else {
+    T r[4 * PT];
+    bool ok[4 * PT];
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ok[4 * i + j] = p4 + j < p.P && l < nvalid;
+        r[4 * i + j] = q[ok[4 * i + j] ? r0 + l * ss + p4 + j : 0];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4 * PT; ++e) v[e] = ok[e] ? (BF ? bf16_to_f((uint16_t)r[e]) : (float)r[e]) : 0.0f;
   }
-  gload<BF, CNT>(t.ptr, (long)u.b * t.s0 + (long)u.h * t.s2, off, v);
 }
 template <int PT>
 __device__ __forceinline__ void lp_store(const float (&v)[CS * PT * 16 / NTHREADS], float* dst, int ld,
                                          int tid = threadIdx.x) {
-  constexpr int PPAD = PT * 16, CNT = CS * PPAD / NTHREADS;
+  constexpr int G4 = 4 * PT;
 #pragma unroll
-  for (int i = 0; i < CNT; ++i) {
-    const int e = tid + i * NTHREADS;
-    dst[(e / PPAD) * ld + (e % PPAD)] = v[i];
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS;
+    *(f4*)(dst + (e4 / G4) * ld + (e4 % G4) * 4) = (f4){v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]};
   }
 }
 // dy tile: from the caller's dout (io dtype) or from the gated fp32 (Bt,L,H,P) workspace copy.
@@ -435,22 +529,29 @@ __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   return (((long)bt * p.nc + c) * p.H + h) * CS * CS;
 }
 
-// Kernel dispatch on (P tiles, io dtype, dt dtype): the statement sees PT_, IOB_, DTB_ as constants.
-#define ISSM_DISPATCH_DT(iob, dtb, ...)                                \
+// Kernel dispatch on (P tiles, io dtype, dt dtype, complete tiles): the statement sees PT_, IOB_, DTB_, FULL_
+// as constants.
+#define ISSM_DISPATCH_FULL(full, ...)                                  \
+  if (full) { constexpr bool FULL_ = true; __VA_ARGS__ }               \
+  else { constexpr bool FULL_ = false; __VA_ARGS__ }
+#define ISSM_DISPATCH_DT(iob, dtb, full, ...)                          \
   if (iob) {                                                           \
     constexpr bool IOB_ = true;                                        \
-    if (dtb) { constexpr bool DTB_ = true; __VA_ARGS__ }               \
-    else { constexpr bool DTB_ = false; __VA_ARGS__ }                  \
+    if (dtb) { constexpr bool DTB_ = true; ISSM_DISPATCH_FULL(full, __VA_ARGS__) }  \
+    else { constexpr bool DTB_ = false; ISSM_DISPATCH_FULL(full, __VA_ARGS__) }     \
   } else {                                                             \
     constexpr bool IOB_ = false;                                       \
-    if (dtb) { constexpr bool DTB_ = true; __VA_ARGS__ }               \
-    else { constexpr bool DTB_ = false; __VA_ARGS__ }                  \
+    if (dtb) { constexpr bool DTB_ = true; ISSM_DISPATCH_FULL(full, __VA_ARGS__) }  \
+    else { constexpr bool DTB_ = false; ISSM_DISPATCH_FULL(full, __VA_ARGS__) }     \
   }
-#define ISSM_DISPATCH(pt, iob, dtb, ...)                                                   \
-  do {                                                                                     \
-    if ((pt) <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) }      \
-    else if ((pt) == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) } \
-    else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob, dtb, __VA_ARGS__) }                \
+#define ISSM_DISPATCH(p, ...)                                                                        \
+  do {                                                                                               \
+    const int pt_ = ((p).P + 15) / 16;                                                               \
+    const bool iob_ = (p).io_dt != 0, dtb_ = (p).dt_dt != 0;                                         \
+    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0) && ((p).P % 16 == 0);                  \
+    if (pt_ <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }        \
+    else if (pt_ == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }   \
+    else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }                 \
   } while (0)
 
 }  // namespace issm

@@ -82,7 +82,7 @@ __device__ __forceinline__ void m_diag_level(f4& acc, const Frag& cs, const Frag
     }
 }
 
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __restrict__ states,
                                                           float* __restrict__ cs_last, float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -96,9 +96,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 
   // column-lane operands of the first slice and the x tile are in flight together
   int n = wave * 16 + cm;
-  bool vn = n < p.N;
+  bool vn = FULL || n < p.N;
   RowMap rm;
-  rm = make_rowmap(p, u, g4, 0);
+  rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], bv[16], cv[16];
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
@@ -132,8 +132,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
     const bool vn_cur = vn;
     if (n0 + NS < p.N) {  // prefetch the next slice
       n = n0 + NS + wave * 16 + cm;
-      vn = n < p.N;
-      rm = make_rowmap(p, u, g4, n0 + NS);
+      vn = FULL || n < p.N;
+      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
       lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
@@ -293,7 +293,7 @@ struct FwdScanSmem {
   float hs[PT * 16 * LDN];  // H [p][n]
 };
 
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states,
                                                          const float* __restrict__ cabt, float* __restrict__ out_x) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -306,9 +306,9 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   const float* hsrc = states + st_off(p, u.bt, u.c, u.h);
 
   int n = wave * 16 + cm;
-  bool vn = n < p.N;
+  bool vn = FULL || n < p.N;
   RowMap rm;
-  rm = make_rowmap(p, u, g4, 0);
+  rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], cv[16];
   PnRegs<PT> hv;
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
@@ -336,8 +336,8 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     pn_store<PT>(hv, s.hs);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
-      vn = n < p.N;
-      rm = make_rowmap(p, u, g4, n0 + NS);
+      vn = FULL || n < p.N;
+      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
       pn_load<PT>(p, hsrc, n0 + NS, hv);
@@ -388,10 +388,10 @@ static int set_lds(K kernel, size_t bytes) {
 
 int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+  ISSM_DISPATCH(p, {
     const size_t sm = sizeof(FwdLocalSmem<PT_>);
-    if (int e = set_lds(k_chunk_local<PT_, IOB_, DTB_>, sm)) return e;
-    hipLaunchKernelGGL((k_chunk_local<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
+    if (int e = set_lds(k_chunk_local<PT_, IOB_, DTB_, FULL_>, sm)) return e;
+    hipLaunchKernelGGL((k_chunk_local<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
   });
   return (int)hipGetLastError();
 }
@@ -405,10 +405,10 @@ int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream
 
 int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float* out_x, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
-  ISSM_DISPATCH((p.P + 15) / 16, p.io_dt != 0, p.dt_dt != 0, {
+  ISSM_DISPATCH(p, {
     const size_t sm = sizeof(FwdScanSmem<PT_>);
-    if (int e = set_lds(k_chunk_scan<PT_, IOB_, DTB_>, sm)) return e;
-    hipLaunchKernelGGL((k_chunk_scan<PT_, IOB_, DTB_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
+    if (int e = set_lds(k_chunk_scan<PT_, IOB_, DTB_, FULL_>, sm)) return e;
+    hipLaunchKernelGGL((k_chunk_scan<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
   });
   return (int)hipGetLastError();
 }
