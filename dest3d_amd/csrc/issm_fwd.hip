@@ -14,8 +14,12 @@
 //        exp(cs[l]-cs[s]) = exp(cs[l]-cs[r]) * exp(cs[r]-cs[s]).
 // dt' >= 0 makes cs monotone in l for every n, so both factors lie between 1 and the
 // product: nothing overflows that the exact value would not.  Level w therefore is an
-// ordinary product Cw . Bw^T of rescaled operands, restricted to its blocks; the diagonal
-// l == s is the plain product C . (B dt')^T.
+// ordinary product Cw . Bw^T of rescaled operands, restricted to its blocks.  Levels 32 and 16
+// are products of whole 16-row tiles, levels 8 and 4 live inside a diagonal tile (there one
+// operand t = C exp2(cs - ref) on upper rows, Bd exp2(ref - cs) on lower rows serves as both
+// factors: t . t^T holds the wanted entries where the row is upper and the column lower), and
+// the pairs of levels 2, 1 and the diagonal belong to a single lane of the column-lane layout,
+// which evaluates them directly with one exp2 per pair.
 #include "issm_dev.h"
 
 namespace issm {
@@ -46,28 +50,11 @@ __device__ __forceinline__ Frag frag_row_bcast(const float* tile, int row, int g
   return f;
 }
 
-// Off-diagonal 16x16 block (I, J) of M at the level whose reference row is R:
-//   acc += (C_I * exp2(cs_I - cs_R)) . (Bd_J * exp2(cs_R - cs_J))^T   over the slice's 64 columns.
-__device__ __forceinline__ void m_offdiag(f4& acc, const float* csL, const float* ccL, const float* bdL, int I,
-                                          int J, int R, int cm, int g4) {
-  const Frag ci = frag_rows(csL, I * 16, cm, g4), cc = frag_rows(ccL, I * 16, cm, g4);
-  const Frag cj = frag_rows(csL, J * 16, cm, g4), bd = frag_rows(bdL, J * 16, cm, g4);
-  const Frag cr = frag_row_bcast(csL, R, g4);
-#pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float a = cc.v[kb][j] * ex2(ci.v[kb][j] - cr.v[kb][j]);
-      const float b = bd.v[kb][j] * ex2(cr.v[kb][j] - cj.v[kb][j]);
-      acc = mfma4(a, b, acc);
-    }
-}
-
-// One sub-16 level (w = 2^LV) of the wave's diagonal block, operands built in registers from the
-// wave's own row fragments; the reference row of lane row cm is another row of the same block.
+// Level 8 (LV = 3) or 4 (LV = 2) of the wave's diagonal block, operands built in registers from the wave's
+// own row fragments; the reference row of lane row cm is another row of the same block.
 template <int LV>
-__device__ __forceinline__ void m_diag_level(f4& acc, const Frag& cs, const Frag& cc, const Frag& bd, int cm,
-                                             int g4) {
+__device__ __forceinline__ void m_mid_level(f4& acc, const Frag& cs, const Frag& cc, const Frag& bd, int cm,
+                                            int g4) {
   constexpr int w = 1 << LV;
   const int src = ((cm & ~(2 * w - 1)) + w - 1) + 16 * g4;
   const bool upper = (cm & w) != 0;
@@ -76,10 +63,22 @@ __device__ __forceinline__ void m_diag_level(f4& acc, const Frag& cs, const Frag
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float c = cs.v[kb][j];
-      const float ref = __shfl(c, src, 64);
-      const float e = ex2(upper ? c - ref : ref - c);
-      acc = mfma4(upper ? cc.v[kb][j] * e : 0.0f, upper ? 0.0f : bd.v[kb][j] * e, acc);
+      const float d = c - __shfl(c, src, 64);
+      const float t = (upper ? cc.v[kb][j] : bd.v[kb][j]) * ex2(upper ? d : -d);
+      acc = mfma4(t, t, acc);
     }
+}
+
+// sum over the 16 lanes of a row (lanes sharing g4); the total is valid in the lane with cm == 15
+__device__ __forceinline__ float row_sum16(float v) {
+#define ISSM_DPP_ADD(ctrl) \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+  ISSM_DPP_ADD(0x111);  // row_shr:1
+  ISSM_DPP_ADD(0x112);  // row_shr:2
+  ISSM_DPP_ADD(0x114);  // row_shr:4
+  ISSM_DPP_ADD(0x118);  // row_shr:8
+#undef ISSM_DPP_ADD
+  return v;
 }
 
 template <int PT, bool IOB, bool DTB, bool FULL>
@@ -108,9 +107,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
     lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
     lp_store<PT>(xv, s.xs, LDPT);
   }
-  // accumulators of M: up to two off-diagonal blocks, the four sub-16 levels and the diagonal
-  f4 o1 = {0, 0, 0, 0}, o2 = {0, 0, 0, 0}, a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0}, a2 = {0, 0, 0, 0},
-     a1 = {0, 0, 0, 0}, a0 = {0, 0, 0, 0};
+  // accumulators of M.  od: the six off-diagonal blocks (1,0) (3,2) | (2,0) (2,1) (3,0) (3,1), each wave
+  // summing over its own 16 columns of every slice; a8 / a4: levels 8 and 4 of the wave's diagonal
+  // block; sp: the lane's in-group pairs (J, jl >= js) of its own column.
+  f4 od[6], a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0};
+#pragma unroll
+  for (int b = 0; b < 6; ++b) od[b] = (f4){0, 0, 0, 0};
+  float sp[40];
+#pragma unroll
+  for (int i = 0; i < 40; ++i) sp[i] = 0.0f;
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     float dtp[16], cs[16], dummy[16];
@@ -126,6 +131,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
         s.bd[o] = bd[k];
         s.cc[o] = cv[k];
       }
+      // pairs inside the lane's groups of four rows (levels 2, 1 and the diagonal)
+#pragma unroll
+      for (int J = 0; J < 4; ++J)
+#pragma unroll
+        for (int jl = 0; jl < 4; ++jl)
+#pragma unroll
+          for (int js = 0; js <= jl; ++js) {
+            const int kl = 4 * J + jl, ks = 4 * J + js;
+            const float cb = cv[kl] * bd[ks];
+            sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * ex2(cs[kl] - cs[ks]);
+          }
     }
     if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
     const int n_cur = n;
@@ -161,63 +177,90 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int pp = pt * 16 + 4 * g4 + r;
-          if (pp < p.P && vn_cur) dst[(long)pp * p.N + n_cur] = acc[pt][r];
+          if ((FULL || (pp < p.P && vn_cur))) dst[(long)pp * p.N + n_cur] = acc[pt][r];
         }
     }
 
     if (want_m) {
-      // row-lane phase: this wave's diagonal block from its own row fragments
+      // row-lane phase, levels 8 and 4: this wave's diagonal block from its own row fragments
       {
         const Frag fc = frag_rows(s.cs, wave * 16, cm, g4);
         const Frag fcc = frag_rows(s.cc, wave * 16, cm, g4);
         const Frag fbd = frag_rows(s.bd, wave * 16, cm, g4);
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) a0 = mfma4(fcc.v[kb][j], fbd.v[kb][j], a0);
-        pin4(a0);
-        m_diag_level<3>(a8, fc, fcc, fbd, cm, g4);
+        m_mid_level<3>(a8, fc, fcc, fbd, cm, g4);
         pin4(a8);
-        m_diag_level<2>(a4, fc, fcc, fbd, cm, g4);
+        m_mid_level<2>(a4, fc, fcc, fbd, cm, g4);
         pin4(a4);
-        m_diag_level<1>(a2, fc, fcc, fbd, cm, g4);
-        pin4(a2);
-        m_diag_level<0>(a1, fc, fcc, fbd, cm, g4);
-        pin4(a1);
       }
-      // off-diagonal blocks: level 16 -> (1,0) ref row 15, (3,2) ref row 47; level 32 -> ref row 31
-      if (wave == 0) {
-        m_offdiag(o1, s.cs, s.cc, s.bd, 1, 0, 15, cm, g4);
-        pin4(o1);
-        m_offdiag(o2, s.cs, s.cc, s.bd, 2, 0, 31, cm, g4);
-      } else if (wave == 1) {
-        m_offdiag(o1, s.cs, s.cc, s.bd, 2, 1, 31, cm, g4);
-      } else if (wave == 2) {
-        m_offdiag(o1, s.cs, s.cc, s.bd, 3, 2, 47, cm, g4);
-      } else {
-        m_offdiag(o1, s.cs, s.cc, s.bd, 3, 0, 31, cm, g4);
-        pin4(o1);
-        m_offdiag(o2, s.cs, s.cc, s.bd, 3, 1, 31, cm, g4);
+      // levels 16 and 32: all six off-diagonal blocks over this wave's 16 columns (4 MFMA steps each)
+      {
+        const int co = wave * 16 + 4 * g4;
+        auto rows = [&](const float* tile, int T) { return *(const f4*)(tile + (T * 16 + cm) * LDN + co); };
+        auto ref = [&](int R) { return *(const f4*)(s.cs + R * LDN + co); };
+        const f4 r15 = ref(15), r31 = ref(31), r47 = ref(47);
+        const f4 c0 = rows(s.cs, 0), c1 = rows(s.cs, 1), c2 = rows(s.cs, 2), c3 = rows(s.cs, 3);
+        const f4 b0 = rows(s.bd, 0), b1 = rows(s.bd, 1), b2 = rows(s.bd, 2);
+        const f4 q1 = rows(s.cc, 1), q2 = rows(s.cc, 2), q3 = rows(s.cc, 3);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float A1 = q1[j] * ex2(c1[j] - r15[j]), B0 = b0[j] * ex2(r15[j] - c0[j]);    // level 16, rows 0..31
+          const float A3 = q3[j] * ex2(c3[j] - r47[j]), B2 = b2[j] * ex2(r47[j] - c2[j]);    // level 16, rows 32..63
+          const float A2w = q2[j] * ex2(c2[j] - r31[j]), A3w = q3[j] * ex2(c3[j] - r31[j]);  // level 32
+          const float B0w = b0[j] * ex2(r31[j] - c0[j]), B1w = b1[j] * ex2(r31[j] - c1[j]);
+          od[0] = mfma4(A1, B0, od[0]);
+          od[1] = mfma4(A3, B2, od[1]);
+          od[2] = mfma4(A2w, B0w, od[2]);
+          od[3] = mfma4(A2w, B1w, od[3]);
+          od[4] = mfma4(A3w, B0w, od[4]);
+          od[5] = mfma4(A3w, B1w, od[5]);
+        }
       }
       __syncthreads();  // before the next slice overwrites the LDS tiles
     }
   }
 
   if (want_m) {
-    float* m = cabt + sq_off(p, u.bt, u.c, u.h);
-    auto put = [&](const f4& a, int I, int J) {
+    // combine the waves' partial sums through LDS (the slice tiles are free now)
+    static_assert(4 * 6 * 4 * 64 + 4 * 4 * 40 <= 3 * CS * LDN, "reduction scratch must fit in the slice tiles");
+    float* red_od = s.cs;                    // [wave][block][r][lane], runs on into the bd / cc tiles
+    float* red_sp = s.cs + 4 * 6 * 4 * 64;   // [wave][g4][40]
 #pragma unroll
-      for (int r = 0; r < 4; ++r) m[(I * 16 + 4 * g4 + r) * CS + J * 16 + cm] = a[r];
-    };
-    if (wave == 0) { put(o1, 1, 0); put(o2, 2, 0); }
-    else if (wave == 1) put(o1, 2, 1);
-    else if (wave == 2) put(o1, 3, 2);
-    else { put(o1, 3, 0); put(o2, 3, 1); }
+    for (int b = 0; b < 6; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red_od[((wave * 6 + b) * 4 + r) * 64 + lane] = od[b][r];
+#pragma unroll
+    for (int i = 0; i < 40; ++i) {
+      const float t = row_sum16(sp[i]);
+      if (cm == 15) red_sp[(wave * 4 + g4) * 40 + i] = t;
+    }
+    __syncthreads();
+    float* m = cabt + sq_off(p, u.bt, u.c, u.h);
+    // off-diagonal blocks: thread tid owns entry (r, lane) = (tid >> 6, tid & 63) of each block
+    {
+      const int r = tid >> 6, ln = tid & 63, row = 4 * (ln >> 4) + r, col = ln & 15;
+#pragma unroll
+      for (int b = 0; b < 6; ++b) {
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v += red_od[((w * 6 + b) * 4 + r) * 64 + ln];
+        const int I = b == 0 ? 1 : b == 1 ? 3 : b < 4 ? 2 : 3;
+        const int J = b == 0 ? 0 : b == 1 ? 2 : (b & 1) ? 1 : 0;
+        m[(I * 16 + row) * CS + J * 16 + col] = v;
+      }
+    }
+    // diagonal block of this wave: row l = 4 g4 + r, column sc = cm
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int l = 4 * g4 + r, sc = cm;  // within the diagonal block
-      const int d = l ^ sc;
-      float v = d == 0 ? a0[r] : d >= 8 ? a8[r] : d >= 4 ? a4[r] : d >= 2 ? a2[r] : a1[r];
+      const int l = 4 * g4 + r, sc = cm, d = l ^ sc;
+      float v;
+      if (d >= 8) v = a8[r];
+      else if (d >= 4) v = a4[r];
+      else {  // same group of four rows: pair (jl, js) = (r, sc & 3) of group g4 in tile `wave`
+        const int js = sc & 3, idx = 10 * wave + r * (r + 1) / 2 + (js <= r ? js : 0);
+        v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v += red_sp[(w * 4 + g4) * 40 + idx];
+      }
       if (sc > l) v = 0.0f;
       m[(wave * 16 + l) * CS + wave * 16 + sc] = v;
     }
