@@ -79,8 +79,8 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
   }
   {
     float dv[CS * PT * 16 / NTHREADS], xv[CS * PT * 16 / NTHREADS];
-    dy_load<IOB, PT>(p, u, dy_ws, dv);
-    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    dy_load<IOB, PT, FULL>(p, u, dy_ws, dv);
+    lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
     lp_store<PT>(dv, s.dys, LDPT);
     lp_store<PT>(xv, s.xs, LDPT);
   }
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   const RowMap rm = make_rowmap<FULL>(p, u, g4, ns * NS);
   const int lim = vn ? rm.nvalid - 4 * g4 : 0;
   auto rowk = [&](int k) { return 16 * (k >> 2) + (k & 3); };
-  const bool pn_full = rm.full && p.P == PT * 16;
+  constexpr bool pn_full = FULL;
 
   float Bv[16], Cv[16];
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);
@@ -444,8 +444,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       f4 mv[4];
       int tq = tid;
       asm volatile("" : "+v"(tq));
-      dy_load<IOB, PT>(p, u, dy_ws, dv, tq);
-      lp_load<IOB, PT>(p, u, p.x[u.dir], xv, tq);
+      dy_load<IOB, PT, FULL>(p, u, dy_ws, dv, tq);
+      lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv, tq);
       tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv, tq);
       __syncthreads();  // the previous head no longer reads the LDS tiles
       lp_store<PT>(dv, s.dys, LDPT, tq);
@@ -613,7 +613,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   {
     float dv[CS * PT * 16 / NTHREADS];
     f4 mv[4];
-    dy_load<IOB, PT>(p, u, dy_ws, dv);
+    dy_load<IOB, PT, FULL>(p, u, dy_ws, dv);
     tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
     lp_store<PT>(dv, s.dys, LDPT);
     tril_store(mv, s.ms);

@@ -252,15 +252,17 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
                                              const RowMap& rm, float (&out)[16]) {
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   const T* q = (const T*)t.ptr + ((long)b * t.s0 + (long)third * t.s2);
-  long ss = (long)rm.step * t.s1;  // uniform
-  // opaque to the optimiser: the 16 row offsets are derived here, next to their use, instead of being
-  // hoisted out of an enclosing loop into (scarce) scalar registers
-  asm volatile("" : "+s"(ss));
+  const long ss = (long)rm.step * t.s1;  // uniform
   T r[16];
   if (rm.full) {
-    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n);
+    // 32-bit offsets (the host checks that seqlen * stride fits): address = scalar base + per-lane offset.
+    // ks is made opaque so that its multiples are formed here, next to their use, instead of being
+    // hoisted out of an enclosing loop into (scarce) scalar registers.
+    const int lo = rm.base * (int)t.s1 + n;
+    int ks = rm.step * (int)t.s1;
+    asm volatile("" : "+s"(ks));
 #pragma unroll
-    for (int k = 0; k < 16; ++k) r[k] = (q + (16 * (k >> 2) + (k & 3)) * ss)[lo];
+    for (int k = 0; k < 16; ++k) r[k] = q[(unsigned)(lo + (16 * (k >> 2) + (k & 3)) * ks)];
 #pragma unroll
     for (int k = 0; k < 16; ++k) out[k] = BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k];
   } else {
@@ -281,14 +283,15 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
                                               const RowMap& rm, const float (&v)[16]) {
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   T* q = (T*)const_cast<void*>(t.ptr) + ((long)b * t.s0 + (long)third * t.s2);
-  long ss = (long)rm.step * t.s1;
-  asm volatile("" : "+s"(ss));
+  const long ss = (long)rm.step * t.s1;
   if (rm.full) {
-    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n);
+    const int lo = rm.base * (int)t.s1 + n;
+    int ks = rm.step * (int)t.s1;
+    asm volatile("" : "+s"(ks));
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      T* d = q + (16 * (k >> 2) + (k & 3)) * ss;
-      if (BF) d[lo] = (T)f_to_bf16(v[k]); else d[lo] = (T)v[k];
+      const unsigned o = (unsigned)(lo + (16 * (k >> 2) + (k & 3)) * ks);
+      if (BF) q[o] = (T)f_to_bf16(v[k]); else q[o] = (T)v[k];
     }
   } else {
 #pragma unroll
@@ -304,11 +307,11 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
 template <int CNT>
 __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int P, int N, int n, bool vn, int g4,
                                              bool full, float (&out)[CNT]) {
-  asm volatile("" : "+s"(N));
   if (full) {
-    const unsigned lo = (unsigned)(4 * g4 * N + n);
+    const int lo = 4 * g4 * N + n;
+    asm volatile("" : "+s"(N));
 #pragma unroll
-    for (int q = 0; q < CNT; ++q) out[q] = (src + (16 * (q >> 2) + (q & 3)) * N)[lo];
+    for (int q = 0; q < CNT; ++q) out[q] = src[(unsigned)(lo + (16 * (q >> 2) + (q & 3)) * N)];
   } else {
     float r[CNT];
     bool ok[CNT];
@@ -380,7 +383,7 @@ __device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, i
 __device__ __forceinline__ bool lp_vec_ok(const KP& p, const TensorD& t, int esize) {
   return ((p.P & 3) == 0) && (((t.s0 | t.s1 | t.s2) & 3) == 0) && ((((uintptr_t)t.ptr) & (4 * esize - 1)) == 0);
 }
-template <bool BF, int PT>
+template <bool BF, int PT, bool FULL = false>
 __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const TensorD& t,
                                         float (&v)[CS * PT * 16 / NTHREADS], int tid = threadIdx.x) {
   constexpr int G4 = 4 * PT;  // groups per row
@@ -396,7 +399,7 @@ __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const Tensor
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
-      ok[i] = p4 < p.P && l < nvalid;
+      ok[i] = FULL || (p4 < p.P && l < nvalid);
       r[i] = *(const V*)(q + (ok[i] ? r0 + l * ss + p4 : 0));
     }
 #pragma unroll
@@ -421,7 +424,7 @@ __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const Tensor
       const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        ok[4 * i + j] = p4 + j < p.P && l < nvalid;
+        ok[4 * i + j] = FULL || (p4 + j < p.P && l < nvalid);
         r[4 * i + j] = q[ok[4 * i + j] ? r0 + l * ss + p4 + j : 0];
       }
     }
@@ -440,7 +443,7 @@ __device__ __forceinline__ void lp_store(const float (&v)[CS * PT * 16 / NTHREAD
   }
 }
 // dy tile: from the caller's dout (io dtype) or from the gated fp32 (Bt,L,H,P) workspace copy.
-template <bool BF, int PT>
+template <bool BF, int PT, bool FULL = false>
 __device__ __forceinline__ void dy_load(const KP& p, const Unit& u, const float* dy_ws,
                                         float (&v)[CS * PT * 16 / NTHREADS], int tid = threadIdx.x) {
   if (dy_ws) {
@@ -449,9 +452,9 @@ __device__ __forceinline__ void dy_load(const KP& p, const Unit& u, const float*
     t.s0 = (long)p.L * p.H * p.P;
     t.s1 = (long)p.H * p.P;
     t.s2 = p.P;
-    lp_load<false, PT>(p, u, t, v, tid);
+    lp_load<false, PT, FULL>(p, u, t, v, tid);
   } else {
-    lp_load<BF, PT>(p, u, p.dout[u.dir], v, tid);
+    lp_load<BF, PT, FULL>(p, u, p.dout[u.dir], v, tid);
   }
 }
 

@@ -104,7 +104,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   {
     float xv[CS * PT * 16 / NTHREADS];
-    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
     lp_store<PT>(xv, s.xs, LDPT);
   }
   // accumulators of M.  od: the six off-diagonal blocks (1,0) (3,2) | (2,0) (2,1) (3,0) (3,1), each wave
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   {
     float xv[CS * PT * 16 / NTHREADS];
     f4 mv[4];
-    lp_load<IOB, PT>(p, u, p.x[u.dir], xv);
+    lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
     tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
     lp_store<PT>(xv, s.xs, LDPT);
     tril_store(mv, s.ms);
