@@ -71,10 +71,12 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
   int n = wave * 16 + cm;
   bool vn = FULL || n < p.N;
   RowMap rm;
+  Coef cf;
   float raw[16], cv[16];
   if (dstates) {
     rm = make_rowmap<FULL>(p, u, g4, 0);
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+    cf = lane_coef(p, u.h, n, vn);
     lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   }
   {
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     float ct[16];
     {
       float dtp[16], cs[16], dummy[16];
-      lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
+      lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k) ct[k] = cv[k] * ex2(cs[k]);
     }
@@ -116,6 +118,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      cf = lane_coef(p, u.h, n, vn);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
     f4 acc[PT];
@@ -437,6 +440,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+    const Coef cf = lane_coef(p, u.h, n, vn);
+    const float gl = (g4 == 3 && vn) ? g_last[vec_off(p, u.bt, u.c, u.h) + n] : 0.0f;
     lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
     lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
     {
@@ -455,11 +460,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     __syncthreads();
 
     // ---- dt transform and running sum down the chunk (log2 domain)
-    const float An = vn ? p.A[u.h * p.N + n] : 0.0f;
+    const float An = cf.A;
     float dtp[16], cs[16], dfac[16];
     float last;
     {
-      last = lane_prep<true>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dfac);
+      last = lane_prep<true>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dfac);
     }
     float Bd[16];
 #pragma unroll
@@ -513,13 +518,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
+    // the second direction adds to the first one's ddt: fetch it while the last levels run
+    float old[16];
+    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
+    __builtin_amdgcn_sched_barrier(0);
     bwd_small_levels(cs, Bd, Cv, s.dms, e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase: everything below is local to the lane except the scans over rows
     pin16(e1); pin16(x2);
-    float old[16];
-    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     float dcs[16], val[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -529,7 +536,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       val[k] = Bv[k] * E1;
       dcs[k] = Cv[k] * X2 - Bd[k] * E1;
     }
-    if (g4 == 3 && vn) dcs[15] += g_last[vec_off(p, u.bt, u.c, u.h) + n];
+    dcs[15] += gl;
     {
       float carry = 0.0f;  // sum over all rows after the current tile
 #pragma unroll
@@ -604,10 +611,12 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   int n = wave * 16 + cm;
   bool vn = FULL || n < p.N;
   RowMap rm;
+  Coef cf;
   rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], bv[16];
   PnRegs<PT> sv;
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  cf = lane_coef(p, u.h, n, vn);
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
   pn_load<PT>(p, ds, 0, sv);
   {
@@ -625,7 +634,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     {
       float dtp[16], cs[16], dummy[16];
-      const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
+      const float last = lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k)
         s.bt[lane_row(k, g4) * LDN + wave * 16 + cm] = bv[k] * dtp[k] * ex2(last - cs[k]);
@@ -636,6 +645,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      cf = lane_coef(p, u.h, n, vn);
       lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       pn_load<PT>(p, ds, n0 + NS, sv);
     }

@@ -329,12 +329,23 @@ __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int 
 // dt' * A * log2(e) down the chunk (so decays are exp2 of differences).  `raw` holds the loaded
 // dt values.  dfac (if WANT_DFAC) receives d dt' / d dt: the softplus derivative times the clamp
 // mask.  Returns the chunk total (running sum at row 63), the same on all lanes of the column.
+// Per-column coefficients of the dt transform; loaded together with the column's dt values so that
+// their latency is covered by the same prefetch.
+struct Coef {
+  float A, bias;
+};
+__device__ __forceinline__ Coef lane_coef(const KP& p, int h, int n, bool vn) {
+  Coef c;
+  c.A = vn ? p.A[h * p.N + n] : 0.0f;
+  c.bias = (vn && p.dt_bias) ? p.dt_bias[h * p.N + n] : 0.0f;
+  return c;
+}
 template <bool WANT_DFAC>
-__device__ __forceinline__ float lane_prep(const KP& p, int h, int n, bool vn, int cm, int g4, const RowMap& rm,
+__device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn, int cm, int g4, const RowMap& rm,
                                            const float (&raw)[16], float (&dtp)[16], float (&cs)[16],
                                            float (&dfac)[16]) {
-  const float A2 = vn ? p.A[h * p.N + n] * LOG2E : 0.0f;
-  const float bias = (vn && p.dt_bias) ? p.dt_bias[h * p.N + n] : 0.0f;
+  const float A2 = cf.A * LOG2E;
+  const float bias = cf.bias;
   if (p.flags & F_SOFTPLUS) {
 #pragma unroll
     for (int k = 0; k < 16; ++k) {

@@ -97,9 +97,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   int n = wave * 16 + cm;
   bool vn = FULL || n < p.N;
   RowMap rm;
+  Coef cf;
   rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], bv[16], cv[16];
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  cf = lane_coef(p, u.h, n, vn);
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   {
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     float dtp[16], cs[16], dummy[16];
-    const float last = lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
+    const float last = lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
     float bd[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) bd[k] = bv[k] * dtp[k];
@@ -151,6 +153,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      cf = lane_coef(p, u.h, n, vn);
       lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
@@ -351,10 +354,12 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   int n = wave * 16 + cm;
   bool vn = FULL || n < p.N;
   RowMap rm;
+  Coef cf;
   rm = make_rowmap<FULL>(p, u, g4, 0);
   float raw[16], cv[16];
   PnRegs<PT> hv;
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+  cf = lane_coef(p, u.h, n, vn);
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   pn_load<PT>(p, hsrc, 0, hv);
   {
@@ -372,7 +377,7 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     {
       float dtp[16], cs[16], dummy[16];
-      lane_prep<false>(p, u.h, n, vn, cm, g4, rm, raw, dtp, cs, dummy);
+      lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
 #pragma unroll
       for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
     }
@@ -382,6 +387,7 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      cf = lane_coef(p, u.h, n, vn);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
       pn_load<PT>(p, hsrc, n0 + NS, hv);
     }
