@@ -6,7 +6,7 @@
 //   k_bwd_chunk     per (chunk, group, 64-column slice), looping over the heads of the
 //                   group: ddt, dB, dC and the per-unit partial sums of dA / ddt_bias
 //   k_bwd_dx        dx and the per-unit partial sums of dD
-//   k_colsum ...    fixed-order sums of the partials (bit-reproducible, no atomics)
+//   k_bwd_reduce    fixed-order sums of the partials (bit-reproducible, no atomics), one launch
 //
 // With Bd = B dt', E(l,s) = exp(cs[l]-cs[s]) and per state column n
 //   Q[m] = sum_p x[m,p] dS[p],  R[l] = sum_p dy[l,p] H[p],
@@ -698,13 +698,22 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
 }
 
 // ------------------------------------------------------------------- reductions
+// All final reductions run as ONE launch (they are independent of each other and tiny, so separate
+// launches would cost more in dispatch latency than in work); blocks are dealt to the jobs in order.
+struct ReduceJobs {
+  const float *partA, *partBias, *partD, *dh0_dir;
+  float *dA, *dbias, *dD, *dh0;
+  int J, nHN, H, P, d_hdim, ndir;
+  long n_h0;
+  int b_A, b_bias, b_D, b_h0;  // first block of each job; b_h0 .. gridDim.x is the dh0 job
+};
+
 // Column sums of a (J, ncols) fp32 matrix in a fixed order (bit-reproducible, no atomics):
 // block = 32 columns x 8 row groups; row group g adds rows g, g+8, ... and the 8 group sums are
 // combined in order.
-__global__ __launch_bounds__(NTHREADS) void k_colsum(const float* __restrict__ src, int J, int ncols,
-                                                     float* __restrict__ dst) {
-  __shared__ float red[8 * 32];
-  const int c = blockIdx.x * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
+__device__ __forceinline__ void colsum_block(const float* __restrict__ src, int J, int ncols, float* __restrict__ dst,
+                                             int blk, float* red) {
+  const int c = blk * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
   float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   if (c < ncols) {
     int j = g;
@@ -727,10 +736,8 @@ __global__ __launch_bounds__(NTHREADS) void k_colsum(const float* __restrict__ s
 }
 
 // dD[h] = sum over units and p of partD[(j*H + h)*P + p]: one block per head.
-__global__ __launch_bounds__(NTHREADS) void k_dd_scalar(const float* __restrict__ partD, int J, int H, int P,
-                                                        float* __restrict__ dD) {
-  __shared__ float red[NTHREADS];
-  const int h = blockIdx.x;
+__device__ __forceinline__ void dd_scalar_block(const float* __restrict__ partD, int J, int H, int P,
+                                                float* __restrict__ dD, int h, float* red) {
   float a = 0.0f;
   for (int e = threadIdx.x; e < J * P; e += NTHREADS) a += partD[((long)(e / P) * H + h) * P + (e % P)];
   red[threadIdx.x] = a;
@@ -742,14 +749,25 @@ __global__ __launch_bounds__(NTHREADS) void k_dd_scalar(const float* __restrict_
   if (threadIdx.x == 0) dD[h] = red[0];
 }
 
-// dh0 = sum over directions of dh0_dir
-__global__ __launch_bounds__(NTHREADS) void k_dh0(const float* __restrict__ dh0_dir, long n, int ndir,
-                                                  float* __restrict__ dh0) {
-  const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
-  if (id >= n) return;
-  float a = dh0_dir[id];
-  if (ndir > 1) a += dh0_dir[n + id];
-  dh0[id] = a;
+__global__ __launch_bounds__(NTHREADS) void k_bwd_reduce(ReduceJobs j) {
+  __shared__ float red[NTHREADS];
+  const int b = blockIdx.x;
+  if (b < j.b_bias) {
+    colsum_block(j.partA, j.J, j.nHN, j.dA, b - j.b_A, red);
+  } else if (b < j.b_D) {
+    colsum_block(j.partBias, j.J, j.nHN, j.dbias, b - j.b_bias, red);
+  } else if (b < j.b_h0) {
+    if (j.d_hdim) colsum_block(j.partD, j.J, j.H * j.P, j.dD, b - j.b_D, red);
+    else dd_scalar_block(j.partD, j.J, j.H, j.P, j.dD, b - j.b_D, red);
+  } else {
+    // dh0 = sum over directions of dh0_dir
+    const long id = (long)(b - j.b_h0) * NTHREADS + threadIdx.x;
+    if (id < j.n_h0) {
+      float a = j.dh0_dir[id];
+      if (j.ndir > 1) a += j.dh0_dir[j.n_h0 + id];
+      j.dh0[id] = a;
+    }
+  }
 }
 
 // -------------------------------------------------------------------- launchers
@@ -807,21 +825,19 @@ int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const f
 
 int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, const float* partD,
                       const float* dh0_dir, float* dA, float* dbias, float* dD, float* dh0, hipStream_t st) {
-  const int J = p.B * p.ndir * p.nc;
-  const int nHN = p.H * p.N;
-  if (dA) hipLaunchKernelGGL(k_colsum, dim3((nHN + 31) / 32), dim3(NTHREADS), 0, st, partA, J, nHN, dA);
-  if (dbias) hipLaunchKernelGGL(k_colsum, dim3((nHN + 31) / 32), dim3(NTHREADS), 0, st, partBias, J, nHN, dbias);
-  if (dD) {
-    if (p.flags & F_D_HDIM)
-      hipLaunchKernelGGL(k_colsum, dim3((p.H * p.P + 31) / 32), dim3(NTHREADS), 0, st, partD, J, p.H * p.P, dD);
-    else
-      hipLaunchKernelGGL(k_dd_scalar, dim3(p.H), dim3(NTHREADS), 0, st, partD, J, p.H, p.P, dD);
-  }
-  if (dh0) {
-    const long n = (long)p.B * p.H * p.P * p.N;
-    hipLaunchKernelGGL(k_dh0, dim3((unsigned)((n + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st, dh0_dir, n, p.ndir,
-                       dh0);
-  }
+  ReduceJobs j;
+  j.partA = partA; j.partBias = partBias; j.partD = partD; j.dh0_dir = dh0_dir;
+  j.dA = dA; j.dbias = dbias; j.dD = dD; j.dh0 = dh0;
+  j.J = p.B * p.ndir * p.nc; j.nHN = p.H * p.N; j.H = p.H; j.P = p.P; j.ndir = p.ndir;
+  j.d_hdim = (p.flags & F_D_HDIM) ? 1 : 0;
+  j.n_h0 = (long)p.B * p.H * p.P * p.N;
+  int nb = 0;
+  j.b_A = nb; if (dA) nb += (j.nHN + 31) / 32;
+  j.b_bias = nb; if (dbias) nb += (j.nHN + 31) / 32;
+  j.b_D = nb; if (dD) nb += j.d_hdim ? (p.H * p.P + 31) / 32 : p.H;
+  j.b_h0 = nb; if (dh0) nb += (int)((j.n_h0 + NTHREADS - 1) / NTHREADS);
+  if (nb == 0) return 0;
+  hipLaunchKernelGGL(k_bwd_reduce, dim3(nb), dim3(NTHREADS), 0, st, j);
   return (int)hipGetLastError();
 }
 

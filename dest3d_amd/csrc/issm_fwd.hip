@@ -59,14 +59,18 @@ __device__ __forceinline__ void m_mid_level(f4& acc, const Frag& cs, const Frag&
   const int src = ((cm & ~(2 * w - 1)) + w - 1) + 16 * g4;
   const bool upper = (cm & w) != 0;
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
+  for (int kb = 0; kb < 4; ++kb) {
+    float ref[4], t[4];  // four cross-lane fetches in flight together
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ref[j] = __shfl(cs.v[kb][j], src, 64);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float c = cs.v[kb][j];
-      const float d = c - __shfl(c, src, 64);
-      const float t = (upper ? cc.v[kb][j] : bd.v[kb][j]) * ex2(upper ? d : -d);
-      acc = mfma4(t, t, acc);
+      const float d = cs.v[kb][j] - ref[j];
+      t[j] = (upper ? cc.v[kb][j] : bd.v[kb][j]) * ex2(upper ? d : -d);
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = mfma4(t[j], t[j], acc);
+  }
 }
 
 // sum over the 16 lanes of a row (lanes sharing g4); the total is valid in the lane with cm == 15
@@ -119,20 +123,48 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 #pragma unroll
   for (int i = 0; i < 40; ++i) sp[i] = 0.0f;
 
+  __syncthreads();  // x tile complete
   for (int n0 = 0; n0 < p.N; n0 += NS) {
+    // ---- column-lane phase, registers only (overlaps other waves still in the previous slice's row-lane phase)
     float dtp[16], cs[16], dummy[16];
     const float last = lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
     float bd[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) bd[k] = bv[k] * dtp[k];
-    if (want_m) {
+    if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
+
+    if (want_s) {
+      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
+      f4 acc[PT];
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const int o = lane_row(k, g4) * LDN + wave * 16 + cm;
-        s.cs[o] = cs[k];
-        s.bd[o] = bd[k];
-        s.cc[o] = cv[k];
+      for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
+#pragma unroll
+      for (int J = 0; J < 4; ++J) {
+        // the tile's x operands are fetched as one batch of LDS reads, then consumed
+        float xa[4][PT], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float* xr = s.xs + lane_row(4 * J + j, g4) * LDPT + cm;
+#pragma unroll
+          for (int pt = 0; pt < PT; ++pt) xa[j][pt] = xr[pt * 16];
+          b[j] = bd[4 * J + j] * ex2(last - cs[4 * J + j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(xa[j][pt], b[j], acc[pt]);
       }
+      float* dst = states + st_off(p, u.bt, u.c, u.h);
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int pp = pt * 16 + 4 * g4 + r;
+          if ((FULL || (pp < p.P && vn))) dst[(long)pp * p.N + n] = acc[pt][r];
+        }
+    }
+
+    if (want_m) {
       // pairs inside the lane's groups of four rows (levels 2, 1 and the diagonal)
 #pragma unroll
       for (int J = 0; J < 4; ++J)
@@ -144,11 +176,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
             const float cb = cv[kl] * bd[ks];
             sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * ex2(cs[kl] - cs[ks]);
           }
+      if (n0 > 0) __syncthreads();  // every wave has finished reading the previous slice's LDS tiles
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int o = lane_row(k, g4) * LDN + wave * 16 + cm;
+        s.cs[o] = cs[k];
+        s.bd[o] = bd[k];
+        s.cc[o] = cv[k];
+      }
     }
-    if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
-    const int n_cur = n;
-    const bool vn_cur = vn;
-    if (n0 + NS < p.N) {  // prefetch the next slice
+    if (n0 + NS < p.N) {  // prefetch the next slice into the registers that have just been consumed
       n = n0 + NS + wave * 16 + cm;
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
@@ -157,35 +194,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
       lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
       lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
-    __syncthreads();  // x tile (first slice) and the slice's LDS tiles are complete
-
-    if (want_s) {
-      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
-      f4 acc[PT];
-#pragma unroll
-      for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-#pragma unroll
-      for (int J = 0; J < 4; ++J)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int k = 4 * J + j;
-          const float b = bd[k] * ex2(last - cs[k]);
-          const float* xr = s.xs + lane_row(k, g4) * LDPT + cm;
-#pragma unroll
-          for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(xr[pt * 16], b, acc[pt]);
-        }
-      float* dst = states + st_off(p, u.bt, u.c, u.h);
-#pragma unroll
-      for (int pt = 0; pt < PT; ++pt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int pp = pt * 16 + 4 * g4 + r;
-          if ((FULL || (pp < p.P && vn_cur))) dst[(long)pp * p.N + n_cur] = acc[pt][r];
-        }
-    }
 
     if (want_m) {
-      // row-lane phase, levels 8 and 4: this wave's diagonal block from its own row fragments
+      __syncthreads();  // the slice's LDS tiles are complete
+      // ---- row-lane phase, levels 8 and 4: this wave's diagonal block from its own row fragments
       {
         const Frag fc = frag_rows(s.cs, wave * 16, cm, g4);
         const Frag fcc = frag_rows(s.cc, wave * 16, cm, g4);
@@ -218,11 +230,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
           od[5] = mfma4(A3w, B1w, od[5]);
         }
       }
-      __syncthreads();  // before the next slice overwrites the LDS tiles
     }
   }
 
   if (want_m) {
+    __syncthreads();  // all waves are done with the last slice's tiles
     // combine the waves' partial sums through LDS (the slice tiles are free now)
     static_assert(4 * 6 * 4 * 64 + 4 * 4 * 40 <= 3 * CS * LDN, "reduction scratch must fit in the slice tiles");
     float* red_od = s.cs;                    // [wave][block][r][lane], runs on into the bd / cc tiles
