@@ -140,6 +140,16 @@ class Runner:
         return res
 
 
+# Memory traffic per launch at the headline workload, from two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the
+# plain 256 MiB copy of --calib-copy (fetch x2.000, write x1.000); the summary is kept under profiles/.
+# k_bwd_chunk is launched once per direction: the figure is per launch.  Override with --traffic.
+MEASURED_TRAFFIC_BYTES = {
+    "chunk_local": 275.1e6, "state_passing_fwd": 161.6e6, "chunk_scan": 260.7e6, "bwd_dstates": 256.4e6,
+    "state_passing_bwd": 214.0e6, "bwd_chunk": 301.3e6, "bwd_dx": 277.8e6,
+}
+
+
 def stage_work(ndir):
     """Algorithmic FLOPs (2*MAC; exps not counted) and bytes per launch of each kernel."""
     B_, L_, H, P, N, cs = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "cs"))
@@ -219,7 +229,7 @@ def main():
         achieved = amount / (stages[dom] * 1e-6) / 1e9
         roof = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": achieved / PEAK_HBM_GBS, "traffic": None, "kernel": dom}
-    roof["traffic"] = args.traffic
+    roof["traffic"] = args.traffic if args.traffic is not None else MEASURED_TRAFFIC_BYTES.get(dom)
     per_stage = {}
     for k, (b, amt) in work.items():
         rate = amt / (stages[k] * 1e-6)
