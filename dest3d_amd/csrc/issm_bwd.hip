@@ -240,9 +240,9 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 // sums live in registers of one lane; only x, dy and dM (shared by the four waves) go through LDS.
 template <int PT>
 struct BwdChunkSmem {
-  static constexpr int LDPT = PT * 16 + 4;
-  float xs[CS * LDPT];
-  float dys[CS * LDPT];
+  static constexpr int KW = 32 * ((PT + 1) / 2);  // head dimension padded to whole K = 32 steps
+  SplitTile<KW> xs;   // x tile [l][p] as bf16 (hi, lo)
+  SplitTile<KW> dys;  // dy tile
   float dms[CS * LDC];
   float dbc[32 * NTHREADS];  // per-lane dB / dC accumulators [k][tid]
 };
@@ -403,7 +403,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT;
+  constexpr int KW = SM::KW, LDS_ = SplitTile<KW>::LD, KT = KW / 32;
   constexpr int KP_ = PT * 4;  // dS / H values per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
@@ -431,6 +431,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   float Bv[16], Cv[16];
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, Cv);
+  // columns of the split tiles beyond the loaded 16 PT (padding up to whole K steps) stay zero
+  if (KW > 16 * PT) {
+    for (int e = tid; e < CS * (KW - 16 * PT); e += NTHREADS) {
+      const int o = (e / (KW - 16 * PT)) * LDS_ + 16 * PT + e % (KW - 16 * PT);
+      s.xs.hi[o] = s.xs.lo[o] = s.dys.hi[o] = s.dys.lo[o] = 0;
+    }
+  }
   // dB / dC accumulators over the heads of the group: private to the lane, kept in LDS
 #pragma unroll
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
@@ -453,8 +460,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv, tq);
       tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv, tq);
       __syncthreads();  // the previous head no longer reads the LDS tiles
-      lp_store<PT>(dv, s.dys, LDPT, tq);
-      lp_store<PT>(xv, s.xs, LDPT, tq);
+      lp_store_split<PT, LDS_>(dv, s.dys.hi, s.dys.lo, tq);
+      lp_store_split<PT, LDS_>(xv, s.xs.hi, s.xs.lo, tq);
       tril_store(mv, s.dms, tq);
     }
     __syncthreads();
@@ -477,24 +484,37 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     int cq = cm, gq = g4;
     asm volatile("" : "+v"(cq), "+v"(gq));
     float e1[16], x2[16];
+    {
+      // Q = x . dS and R = dy . H contract over the head dimension: split-bf16 products, K = 32 per step.
+      // k-slot s of step t <-> lane value q = 8 t + s <-> p = 16 (q >> 2) + 4 g4 + (q & 3).
+      bf8 dsh[KT], dsl[KT], hh_[KT], hl_[KT];
 #pragma unroll
-    for (int I = 0; I < 4; ++I) {
-      f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+      for (int t = 0; t < KT; ++t) {
+        float a[8], b[8];
 #pragma unroll
-      for (int kb = 0; kb < PT; ++kb) {
-        const f4 ax = *(const f4*)(s.xs + (I * 16 + cq) * LDPT + kb * 16 + 4 * gq);
-        const f4 ay = *(const f4*)(s.dys + (I * 16 + cq) * LDPT + kb * 16 + 4 * gq);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          q = mfma4(ax[j], dsv[4 * kb + j], q);
-          r = mfma4(ay[j], hv[4 * kb + j], r);
+        for (int j = 0; j < 8; ++j) {
+          a[j] = 8 * t + j < KP_ ? dsv[(8 * t + j) % KP_] : 0.0f;
+          b[j] = 8 * t + j < KP_ ? hv[(8 * t + j) % KP_] : 0.0f;
         }
+        split8(a, dsh[t], dsl[t]);
+        split8(b, hh_[t], hl_[t]);
       }
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int k = 4 * I + rr;
-        e1[k] = ex2(last - cs[k]) * q[rr];
-        x2[k] = ex2(cs[k]) * r[rr];
+      for (int I = 0; I < 4; ++I) {
+        f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+          const bf8 xh = split_frag<LDS_>(s.xs.hi, I * 16 + cq, gq, t), xl = split_frag<LDS_>(s.xs.lo, I * 16 + cq, gq, t);
+          const bf8 yh = split_frag<LDS_>(s.dys.hi, I * 16 + cq, gq, t), yl = split_frag<LDS_>(s.dys.lo, I * 16 + cq, gq, t);
+          q = mfma_split(xh, xl, dsh[t], dsl[t], q);
+          r = mfma_split(yh, yl, hh_[t], hl_[t], r);
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int k = 4 * I + rr;
+          e1[k] = ex2(last - cs[k]) * q[rr];
+          x2[k] = ex2(cs[k]) * r[rr];
+        }
       }
     }
 

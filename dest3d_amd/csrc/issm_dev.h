@@ -187,6 +187,73 @@ __device__ __forceinline__ void mma16_mk(f4& acc, const float* a, int lda, int m
   acc = mfma4(av.w, bp[3 * ldb], acc);
 }
 
+// ------------------------------------------------------------------ split-bf16 products
+// v_mfma_f32_16x16x4_f32 shares the vector ALU's issue slots (measured: its time adds to the VALU time
+// instead of overlapping it), while v_mfma_f32_16x16x32_bf16 does 8x the multiply-adds in about half the
+// time.  Where both operands of a product are reused often enough to amortise the conversion, an fp32
+// product a.b is therefore evaluated as  ah.bh + ah.bl + al.bh  with a = ah + al, ah = bf16(a),
+// al = bf16(a - ah) (16 significand bits per operand; the dropped al.bl term is <= 2^-16 |a.b|) and fp32
+// accumulation.  One instruction contracts over K = 32: lane (cm, g4) supplies k-slots 0..7 of group g4.
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f4 mfma_bf(bf8 a, bf8 b, f4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+// acc += A.B with both operands given as (hi, lo) pairs
+__device__ __forceinline__ f4 mfma_split(bf8 ah, bf8 al, bf8 bh, bf8 bl, f4 c) {
+  c = mfma_bf(al, bh, c);
+  c = mfma_bf(ah, bl, c);
+  return mfma_bf(ah, bh, c);
+}
+__device__ __forceinline__ void split4(const float (&v)[4], bf4& hi, bf4& lo) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const __bf16 h = (__bf16)v[j];
+    hi[j] = h;
+    lo[j] = (__bf16)(v[j] - (float)h);
+  }
+}
+// eight fp32 values of a lane (k-slots 0..7) -> (hi, lo) fragments
+__device__ __forceinline__ void split8(const float (&v)[8], bf8& hi, bf8& lo) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const __bf16 h = (__bf16)v[j];
+    hi[j] = h;
+    lo[j] = (__bf16)(v[j] - (float)h);
+  }
+}
+// Row-major bf16 tiles [rows][SplitLd] holding the hi and the lo halves of an fp32 (rows x KW) tile, KW a
+// multiple of 32.  Fragment of K-step t for lane (row, g4): columns 32t + 4 g4 .. +3 and 32t + 16 + 4 g4 .. +3,
+// i.e. k-slot s <-> column 32t + 16 (s >> 2) + 4 g4 + (s & 3).
+template <int KW>
+struct SplitTile {
+  static constexpr int LD = KW + 8;
+  uint16_t hi[CS * LD];
+  uint16_t lo[CS * LD];
+};
+template <int LD>
+__device__ __forceinline__ bf8 split_frag(const uint16_t* tile, int row, int g4, int t) {
+  const uint16_t* q = tile + row * LD + 32 * t + 4 * g4;
+  const bf4 a = *(const bf4*)q, b = *(const bf4*)(q + 16);
+  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// Store of a cooperative (64 x 16 PT) register tile (layout of lp_load) as split bf16 tiles.
+template <int PT, int LD>
+__device__ __forceinline__ void lp_store_split(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* hi, uint16_t* lo,
+                                               int tid = threadIdx.x) {
+  constexpr int G4 = 4 * PT;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS, o = (e4 / G4) * LD + (e4 % G4) * 4;
+    const float w[4] = {v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]};
+    bf4 h, l;
+    split4(w, h, l);
+    *(bf4*)(hi + o) = h;
+    *(bf4*)(lo + o) = l;
+  }
+}
+
 // Decode a unit id -> (b, dir, c, h); h is fastest so that the heads of one chunk run back to
 // back and share the B/C tiles in cache.
 struct Unit {
