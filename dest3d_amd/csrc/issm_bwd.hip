@@ -52,6 +52,7 @@ struct BwdStSmem {
   static constexpr int LDPT = PT * 16 + 4;
   float dys[CS * LDPT];
   float xs[CS * LDPT];
+  SplitTile<CS> dyt;  // dy tile transposed, [p][l], as bf16 (hi, lo): operand of dH
 };
 
 // dH[p][n] = sum_l dy[l][p] * C[l][n] exp2(cs[l][n]): contraction over rows, so the B operand
@@ -85,6 +86,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
     lp_store<PT>(dv, s.dys, LDPT);
     lp_store<PT>(xv, s.xs, LDPT);
+    if (dstates) lp_store_split_t<PT, SplitTile<CS>::LD>(dv, s.dyt.hi, s.dyt.lo);
   }
   __syncthreads();
 
@@ -124,12 +126,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     f4 acc[PT];
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const float* yr = s.dys + lane_row(k, g4) * LDPT + cm;
-#pragma unroll
-      for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(yr[pt * 16], ct[k], acc[pt]);
-    }
+    rows_product_split<PT, SplitTile<CS>::LD>(acc, s.dyt.hi, s.dyt.lo, ct, cm, g4);
     float* dst = dstates + dst_off(p, u.bt, u.c, u.h);
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt)

@@ -254,6 +254,45 @@ __device__ __forceinline__ void lp_store_split(const float (&v)[CS * PT * 16 / N
   }
 }
 
+// Same register tile stored transposed, [p][l] (rows = head dimension, KW = CS columns), for products that
+// contract over the rows of the chunk.
+template <int PT, int LD>
+__device__ __forceinline__ void lp_store_split_t(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* hi,
+                                                 uint16_t* lo, int tid = threadIdx.x) {
+  constexpr int G4 = 4 * PT;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float w = v[4 * i + j];
+      const __bf16 h = (__bf16)w;
+      const __bf16 lw = (__bf16)(w - (float)h);
+      hi[(p4 + j) * LD + l] = __builtin_bit_cast(uint16_t, h);
+      lo[(p4 + j) * LD + l] = __builtin_bit_cast(uint16_t, lw);
+    }
+  }
+}
+// acc[pt] += (tile^T)(16 pt .. +15, :) . b  for a product over the 64 chunk rows whose B operand is the lane's
+// 16 column-lane values (k = 4J + j <-> row 16J + 4 g4 + j): two K = 32 steps, step t <-> values 8t .. 8t+7.
+template <int PT, int LD>
+__device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t* thi, const uint16_t* tlo,
+                                                   const float (&b)[16], int cm, int g4) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    float w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = b[8 * t + j];
+    bf8 bh, bl;
+    split8(w, bh, bl);
+#pragma unroll
+    for (int pt = 0; pt < PT; ++pt) {
+      const bf8 ah = split_frag<LD>(thi, pt * 16 + cm, g4, t), al = split_frag<LD>(tlo, pt * 16 + cm, g4, t);
+      acc[pt] = mfma_split(ah, al, bh, bl, acc[pt]);
+    }
+  }
+}
+
 // Decode a unit id -> (b, dir, c, h); h is fastest so that the heads of one chunk run back to
 // back and share the B/C tiles in cache.
 struct Unit {

@@ -26,8 +26,7 @@ namespace issm {
 
 template <int PT>
 struct FwdLocalSmem {
-  static constexpr int LDPT = PT * 16 + 4;
-  float xs[CS * LDPT];  // x tile [l][p]
+  SplitTile<CS> xt;     // x tile transposed, [p][l], as bf16 (hi, lo)
   float cs[CS * LDN];   // running sum of dt'*A*log2e [l][n] of the current slice
   float bd[CS * LDN];   // B*dt' [l][n]
   float cc[CS * LDN];   // C [l][n]
@@ -91,7 +90,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef FwdLocalSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT;
+  constexpr int LDT = SplitTile<CS>::LD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -111,7 +110,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   {
     float xv[CS * PT * 16 / NTHREADS];
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
-    lp_store<PT>(xv, s.xs, LDPT);
+    lp_store_split_t<PT, LDT>(xv, s.xt.hi, s.xt.lo);
   }
   // accumulators of M.  od: the six off-diagonal blocks (1,0) (3,2) | (2,0) (2,1) (3,0) (3,1), each wave
   // summing over its own 16 columns of every slice; a8 / a4: levels 8 and 4 of the wave's diagonal
@@ -134,25 +133,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
     if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
 
     if (want_s) {
-      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
+      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers,
+      // split-bf16 product over the 64 rows
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
+      {
+        float b[16];
 #pragma unroll
-      for (int J = 0; J < 4; ++J) {
-        // the tile's x operands are fetched as one batch of LDS reads, then consumed
-        float xa[4][PT], b[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float* xr = s.xs + lane_row(4 * J + j, g4) * LDPT + cm;
-#pragma unroll
-          for (int pt = 0; pt < PT; ++pt) xa[j][pt] = xr[pt * 16];
-          b[j] = bd[4 * J + j] * ex2(last - cs[4 * J + j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma4(xa[j][pt], b[j], acc[pt]);
+        for (int kk = 0; kk < 16; ++kk) b[kk] = bd[kk] * ex2(last - cs[kk]);
+        rows_product_split<PT, LDT>(acc, s.xt.hi, s.xt.lo, b, cm, g4);
       }
       float* dst = states + st_off(p, u.bt, u.c, u.h);
 #pragma unroll
