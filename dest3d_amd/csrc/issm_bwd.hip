@@ -423,7 +423,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   const RowMap rm = make_rowmap<FULL>(p, u, g4, ns * NS);
   const int lim = vn ? rm.nvalid - 4 * g4 : 0;
   auto rowk = [&](int k) { return 16 * (k >> 2) + (k & 3); };
-  constexpr bool pn_full = FULL;
+  const bool pn_full = FULL && p.P == PT * 16;
 
   float Bv[16], Cv[16];
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);

@@ -336,7 +336,7 @@ __device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
 // i.e. physical row base + step * (16J + j): a per-lane part (base) plus a part that is the same
 // for the whole wave, so that in a full chunk the address of every element is a scalar base
 // plus ONE per-lane offset.  `full` (a compile-time constant of the kernel variant) says that all 64
-// rows and all 64 columns of every slice exist; otherwise rows >= nvalid and lanes with !vn read as zero.
+// rows and all 64 columns of every slice exist (the head dimension is checked separately at run time); otherwise rows >= nvalid and lanes with !vn read as zero.
 struct RowMap {
   int base, step, nvalid;
   bool full;
@@ -516,7 +516,7 @@ __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const Tensor
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
-      ok[i] = FULL || (p4 < p.P && l < nvalid);
+      ok[i] = p4 < p.P && (FULL || l < nvalid);
       r[i] = *(const V*)(q + (ok[i] ? r0 + l * ss + p4 : 0));
     }
 #pragma unroll
@@ -541,7 +541,7 @@ __device__ __forceinline__ void lp_load(const KP& p, const Unit& u, const Tensor
       const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        ok[4 * i + j] = FULL || (p4 + j < p.P && l < nvalid);
+        ok[4 * i + j] = p4 + j < p.P && (FULL || l < nvalid);
         r[4 * i + j] = q[ok[4 * i + j] ? r0 + l * ss + p4 + j : 0];
       }
     }
@@ -668,7 +668,7 @@ __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   do {                                                                                               \
     const int pt_ = ((p).P + 15) / 16;                                                               \
     const bool iob_ = (p).io_dt != 0, dtb_ = (p).dt_dt != 0;                                         \
-    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0) && ((p).P % 16 == 0);                  \
+    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0);                                       \
     if (pt_ <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }        \
     else if (pt_ == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }   \
     else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }                 \

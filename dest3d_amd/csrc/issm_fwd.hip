@@ -150,7 +150,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int pp = pt * 16 + 4 * g4 + r;
-          if ((FULL || (pp < p.P && vn))) dst[(long)pp * p.N + n] = acc[pt][r];
+          if (pp < p.P && (FULL || vn)) dst[(long)pp * p.N + n] = acc[pt][r];
         }
     }
 

@@ -103,6 +103,9 @@ CASES = [
     (1, 320, 8, 32, 256, 1, dict(softplus=False)),
     (1, 70, 2, 20, 30, 1, dict(D="hp", z=True)),         # N not a multiple of 4, P not a multiple of 16
     (1, 1, 1, 8, 16, 1, dict()),                          # a single token
+    (1, 128, 2, 36, 64, 1, dict(D="hp", z=True)),        # complete chunks / slices, ragged head dimension
+    (2, 64, 2, 20, 128, 2, dict(softplus=False)),
+    (1, 192, 1, 64, 64, 1, dict()),                       # complete tiles, widest head dimension
 ]
 
 
