@@ -10,7 +10,8 @@ Besides the driver's JSON contract the line carries
   roofline      the dominant kernel's achieved fraction of its bound (live HIP-event timing)
   cpu_baseline  the oracle's chunked pure-PyTorch formulation timed on the host cores
   stages_us     average duration of every kernel of the step
-  variants_us   fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants
+  variants_us   fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants (also at the
+                detector's head dimension 36)
 """
 import argparse
 import ctypes as C
@@ -237,11 +238,14 @@ def main():
                         "frac": round(rate / (PEAK_FP32_MFMA_TFLOPS * 1e12 if b == "mfma" else PEAK_HBM_GBS * 1e9), 4)}
     variants = {}
     if not args.no_variants:
-        for name, nd, dt in (("uni_fp32", 1, torch.float32), ("uni_bf16", 1, torch.bfloat16),
-                             ("bidir_bf16", 2, torch.bfloat16)):
+        for name, nd, dt, pdim in (("uni_fp32", 1, torch.float32, 32), ("uni_bf16", 1, torch.bfloat16, 32),
+                                   ("bidir_bf16", 2, torch.bfloat16, 32),
+                                   ("bidir_bf16_headdim36", 2, torch.bfloat16, 36)):  # the detector's head size
+            SHAPE["P"] = pdim
             r = Runner(torch, nd, dt)
             variants[name] = round(r.time_steps(max(args.steps // 2, 5), 5), 2)
             del r
+        SHAPE["P"] = 32
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),
