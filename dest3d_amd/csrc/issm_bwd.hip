@@ -126,7 +126,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     f4 acc[PT];
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-    rows_product_split<PT, SplitTile<CS>::LD>(acc, s.dyt.hi, s.dyt.lo, ct, cm, g4);
+    rows_product_split<PT, SplitTile<CS>::LD>(acc, s.dyt.hi, s.dyt.lo, [&](int k) { return ct[k]; }, cm, g4);
     float* dst = dstates + dst_off(p, u.bt, u.c, u.h);
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt)

@@ -275,14 +275,15 @@ __device__ __forceinline__ void lp_store_split_t(const float (&v)[CS * PT * 16 /
 }
 // acc[pt] += (tile^T)(16 pt .. +15, :) . b  for a product over the 64 chunk rows whose B operand is the lane's
 // 16 column-lane values (k = 4J + j <-> row 16J + 4 g4 + j): two K = 32 steps, step t <-> values 8t .. 8t+7.
-template <int PT, int LD>
-__device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t* thi, const uint16_t* tlo,
-                                                   const float (&b)[16], int cm, int g4) {
+// `b(k)` yields the lane's value k (evaluated step by step, so that only eight are live at a time).
+template <int PT, int LD, typename F>
+__device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t* thi, const uint16_t* tlo, F b,
+                                                   int cm, int g4) {
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     float w[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = b[8 * t + j];
+    for (int j = 0; j < 8; ++j) w[j] = b(8 * t + j);
     bf8 bh, bl;
     split8(w, bh, bl);
 #pragma unroll

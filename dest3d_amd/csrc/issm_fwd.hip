@@ -105,8 +105,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   float raw[16], bv[16], cv[16];
   lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
   cf = lane_coef(p, u.h, n, vn);
-  lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
-  lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   {
     float xv[CS * PT * 16 / NTHREADS];
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
@@ -125,6 +123,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   __syncthreads();  // x tile complete
   for (int n0 = 0; n0 < p.N; n0 += NS) {
     // ---- column-lane phase, registers only (overlaps other waves still in the previous slice's row-lane phase)
+    // B and C of this slice are requested here and first used after the dt transform, which covers their
+    // latency; only dt is prefetched across the row-lane phase (fewer registers live there)
+    lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
+    lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     float dtp[16], cs[16], dummy[16];
     const float last = lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
     float bd[16];
@@ -138,20 +140,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-      {
-        float b[16];
-#pragma unroll
-        for (int kk = 0; kk < 16; ++kk) b[kk] = bd[kk] * ex2(last - cs[kk]);
-        rows_product_split<PT, LDT>(acc, s.xt.hi, s.xt.lo, b, cm, g4);
-      }
+      rows_product_split<PT, LDT>(acc, s.xt.hi, s.xt.lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
+      if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
+        float* d0 = dst + (4 * g4) * p.N + n;
 #pragma unroll
-      for (int pt = 0; pt < PT; ++pt)
+        for (int pt = 0; pt < PT; ++pt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int pp = pt * 16 + 4 * g4 + r;
-          if (pp < p.P && (FULL || vn)) dst[(long)pp * p.N + n] = acc[pt][r];
-        }
+          for (int r = 0; r < 4; ++r) d0[(pt * 16 + r) * p.N] = acc[pt][r];
+      } else {
+#pragma unroll
+        for (int pt = 0; pt < PT; ++pt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int pp = pt * 16 + 4 * g4 + r;
+            if (pp < p.P && vn) dst[(long)pp * p.N + n] = acc[pt][r];
+          }
+      }
     }
 
     if (want_m) {
@@ -175,14 +180,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
         s.cc[o] = cv[k];
       }
     }
-    if (n0 + NS < p.N) {  // prefetch the next slice into the registers that have just been consumed
+    if (n0 + NS < p.N) {  // prefetch the next slice's dt into the registers that have just been consumed
       n = n0 + NS + wave * 16 + cm;
       vn = FULL || n < p.N;
       rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
       lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
       cf = lane_coef(p, u.h, n, vn);
-      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
-      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     }
 
     if (want_m) {
@@ -394,7 +397,8 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
       pn_load<PT>(p, hsrc, n0 + NS, hv);
     }
     __syncthreads();
-    // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows
+    // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows.  (fp32 product: both operands change with
+    // every slice and are used once or twice, so a bf16 split costs more vector work than it saves -- measured)
 #pragma unroll
     for (int kb = 0; kb < NS; kb += 16)
 #pragma unroll
