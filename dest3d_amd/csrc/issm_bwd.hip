@@ -484,34 +484,58 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     {
       // Q = x . dS and R = dy . H contract over the head dimension: split-bf16 products, K = 32 per step.
       // k-slot s of step t <-> lane value q = 8 t + s <-> p = 16 (q >> 2) + 4 g4 + (q & 3).
-      bf8 dsh[KT], dsl[KT], hh_[KT], hl_[KT];
-#pragma unroll
-      for (int t = 0; t < KT; ++t) {
-        float a[8], b[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          a[j] = 8 * t + j < KP_ ? dsv[(8 * t + j) % KP_] : 0.0f;
-          b[j] = 8 * t + j < KP_ ? hv[(8 * t + j) % KP_] : 0.0f;
-        }
-        split8(a, dsh[t], dsl[t]);
-        split8(b, hh_[t], hl_[t]);
-      }
-#pragma unroll
-      for (int I = 0; I < 4; ++I) {
-        f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+      // (Q first, then R: only one pair of split operands is live at a time)
+      auto product = [&](const float (&v)[KP_], const uint16_t* thi, const uint16_t* tlo, f4 (&res)[4]) {
+        bf8 bh[KT], bl[KT];
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
-          const bf8 xh = split_frag<LDS_>(s.xs.hi, I * 16 + cq, gq, t), xl = split_frag<LDS_>(s.xs.lo, I * 16 + cq, gq, t);
-          const bf8 yh = split_frag<LDS_>(s.dys.hi, I * 16 + cq, gq, t), yl = split_frag<LDS_>(s.dys.lo, I * 16 + cq, gq, t);
-          q = mfma_split(xh, xl, dsh[t], dsl[t], q);
-          r = mfma_split(yh, yl, hh_[t], hl_[t], r);
+          float a[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) a[j] = 8 * t + j < KP_ ? v[(8 * t + j) % KP_] : 0.0f;
+          split8(a, bh[t], bl[t]);
         }
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int k = 4 * I + rr;
-          e1[k] = ex2(last - cs[k]) * q[rr];
-          x2[k] = ex2(cs[k]) * r[rr];
+        for (int I = 0; I < 4; ++I) {
+          res[I] = (f4){0, 0, 0, 0};
+#pragma unroll
+          for (int t = 0; t < KT; ++t) {
+            const bf8 ah = split_frag<LDS_>(thi, I * 16 + cq, gq, t), al = split_frag<LDS_>(tlo, I * 16 + cq, gq, t);
+            res[I] = mfma_split(ah, al, bh[t], bl[t], res[I]);
+          }
         }
+      };
+      if constexpr (KT == 1) {
+        // one K step: both products interleaved (two independent accumulation chains)
+        float a[8], b[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { a[j] = dsv[j]; b[j] = hv[j]; }
+        bf8 dsh, dsl, hh_, hl_;
+        split8(a, dsh, dsl);
+        split8(b, hh_, hl_);
+#pragma unroll
+        for (int I = 0; I < 4; ++I) {
+          const bf8 xh = split_frag<LDS_>(s.xs.hi, I * 16 + cq, gq, 0), xl = split_frag<LDS_>(s.xs.lo, I * 16 + cq, gq, 0);
+          const bf8 yh = split_frag<LDS_>(s.dys.hi, I * 16 + cq, gq, 0), yl = split_frag<LDS_>(s.dys.lo, I * 16 + cq, gq, 0);
+          const f4 q = mfma_split(xh, xl, dsh, dsl, (f4){0, 0, 0, 0});
+          const f4 r = mfma_split(yh, yl, hh_, hl_, (f4){0, 0, 0, 0});
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            e1[4 * I + rr] = ex2(last - cs[4 * I + rr]) * q[rr];
+            x2[4 * I + rr] = ex2(cs[4 * I + rr]) * r[rr];
+          }
+        }
+      } else {
+        f4 q[4];
+        product(dsv, s.xs.hi, s.xs.lo, q);
+#pragma unroll
+        for (int I = 0; I < 4; ++I)
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) e1[4 * I + rr] = ex2(last - cs[4 * I + rr]) * q[I][rr];
+        product(hv, s.dys.hi, s.dys.lo, q);
+#pragma unroll
+        for (int I = 0; I < 4; ++I)
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) x2[4 * I + rr] = ex2(cs[4 * I + rr]) * q[I][rr];
       }
     }
 
