@@ -237,7 +237,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 // sums live in registers of one lane; only x, dy and dM (shared by the four waves) go through LDS.
 template <int PT>
 struct BwdChunkSmem {
-  static constexpr int KW = 32 * ((PT + 1) / 2);  // head dimension padded to whole K = 32 steps
+  static constexpr int KW = 16 * PT;  // stored width; the K = 32 steps read missing columns as zero
   SplitTile<KW> xs;   // x tile [l][p] as bf16 (hi, lo)
   SplitTile<KW> dys;  // dy tile
   float dms[CS * LDC];
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int KW = SM::KW, LDS_ = SplitTile<KW>::LD, KT = KW / 32;
+  constexpr int KW = SM::KW, LDS_ = SplitTile<KW>::LD, KT = (PT + 1) / 2;
   constexpr int KP_ = PT * 4;  // dS / H values per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
@@ -428,13 +428,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   float Bv[16], Cv[16];
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, Cv);
-  // columns of the split tiles beyond the loaded 16 PT (padding up to whole K steps) stay zero
-  if (KW > 16 * PT) {
-    for (int e = tid; e < CS * (KW - 16 * PT); e += NTHREADS) {
-      const int o = (e / (KW - 16 * PT)) * LDS_ + 16 * PT + e % (KW - 16 * PT);
-      s.xs.hi[o] = s.xs.lo[o] = s.dys.hi[o] = s.dys.lo[o] = 0;
-    }
-  }
   // dB / dC accumulators over the heads of the group: private to the lane, kept in LDS
 #pragma unroll
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
@@ -499,7 +492,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
           res[I] = (f4){0, 0, 0, 0};
 #pragma unroll
           for (int t = 0; t < KT; ++t) {
-            const bf8 ah = split_frag<LDS_>(thi, I * 16 + cq, gq, t), al = split_frag<LDS_>(tlo, I * 16 + cq, gq, t);
+            // the last step of an odd number of 16-column tiles has only its first half
+            const bool half = (PT & 1) && t == KT - 1;
+            const bf8 ah = half ? split_frag<LDS_, true>(thi, I * 16 + cq, gq, t) : split_frag<LDS_>(thi, I * 16 + cq, gq, t);
+            const bf8 al = half ? split_frag<LDS_, true>(tlo, I * 16 + cq, gq, t) : split_frag<LDS_>(tlo, I * 16 + cq, gq, t);
             res[I] = mfma_split(ah, al, bh[t], bl[t], res[I]);
           }
         }

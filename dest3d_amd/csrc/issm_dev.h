@@ -224,7 +224,7 @@ __device__ __forceinline__ void split8(const float (&v)[8], bf8& hi, bf8& lo) {
   }
 }
 // Row-major bf16 tiles [rows][SplitLd] holding the hi and the lo halves of an fp32 (rows x KW) tile, KW a
-// multiple of 32.  Fragment of K-step t for lane (row, g4): columns 32t + 4 g4 .. +3 and 32t + 16 + 4 g4 .. +3,
+// multiple of 16.  Fragment of K-step t for lane (row, g4): columns 32t + 4 g4 .. +3 and 32t + 16 + 4 g4 .. +3,
 // i.e. k-slot s <-> column 32t + 16 (s >> 2) + 4 g4 + (s & 3).
 template <int KW>
 struct SplitTile {
@@ -232,10 +232,13 @@ struct SplitTile {
   uint16_t hi[CS * LD];
   uint16_t lo[CS * LD];
 };
-template <int LD>
+// (HALF: the tile has no columns 32t + 16 .. 32t + 31; those k-slots read as zero.)
+template <int LD, bool HALF = false>
 __device__ __forceinline__ bf8 split_frag(const uint16_t* tile, int row, int g4, int t) {
   const uint16_t* q = tile + row * LD + 32 * t + 4 * g4;
-  const bf4 a = *(const bf4*)q, b = *(const bf4*)(q + 16);
+  const bf4 a = *(const bf4*)q;
+  bf4 b = {0, 0, 0, 0};
+  if (!HALF) b = *(const bf4*)(q + 16);
   return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 // Store of a cooperative (64 x 16 PT) register tile (layout of lp_load) as split bf16 tiles.
