@@ -28,6 +28,13 @@
  *  - ndir = 2 runs the module's bidirectional pair (models/dest_module.py:565-575) in
  *    one call: direction 1 walks the same dt / A / D / h0 backwards in time with its
  *    own x / Bm / Cm and writes its outputs back in natural (un-flipped) time order.
+ *  - Numerics: cumulative sums, decays, states and all accumulation are fp32 for every
+ *    I/O dtype.  The products x^T.(B dt' decay), dy^T.(C decay), x.dS and dy.H are
+ *    evaluated as three bf16 matrix products with fp32 accumulation on operands split
+ *    into bf16 high and low parts (16 significand bits per operand; relative error of a
+ *    product <= 2^-16); every other product is fp32.  Results are bit-reproducible
+ *    from run to run (fixed-order reductions, no atomics).
+ *  - Strides: stride[1] * seqlen must stay below 2^31 elements (row offsets are 32-bit).
  */
 #ifndef ISSM_H
 #define ISSM_H
