@@ -122,13 +122,14 @@ static int check_common(const issm_scan_args* a) {
   return check_strides(a);
 }
 
-// The kernels address a row of a caller tensor as a 64-bit (batch, head) base plus a 32-bit
-// (time row * stride[1] + column) offset: that offset must fit, and strides may not be negative.
+// The kernels address a row of a caller tensor as a 64-bit (batch, head) base plus a 32-bit BYTE
+// offset (time row * stride[1] + column) * element size: that offset must fit (2^30 elements), and
+// strides may not be negative.
 static int check_td(const issm_tensor& t, const char* name, int dir, long rows, long inner) {
   if (!t.ptr) return ISSM_OK;
   for (int i = 0; i < 3; ++i)
     if (t.stride[i] < 0) return fail(ISSM_E_STRIDE, "%s[%d]: negative stride %ld", name, dir, (long)t.stride[i]);
-  if ((rows - 1) * (long)t.stride[1] + inner > 0x7fffffffL)
+  if ((rows - 1) * (long)t.stride[1] + inner > 0x3fffffffL)
     return fail(ISSM_E_STRIDE, "%s[%d]: seqlen * stride[1] = %ld * %ld exceeds the 32-bit row offset range", name, dir,
                 rows, (long)t.stride[1]);
   return ISSM_OK;

@@ -368,11 +368,14 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
     // 32-bit offsets (the host checks that seqlen * stride fits): address = scalar base + per-lane offset.
     // ks is made opaque so that its multiples are formed here, next to their use, instead of being
     // hoisted out of an enclosing loop into (scarce) scalar registers.
-    const int lo = rm.base * (int)t.s1 + n;
-    int ks = rm.step * (int)t.s1;
+    // BYTE offsets in 32 bits, so that the access is "scalar base + 32-bit per-lane offset" and costs one
+    // integer add per element.
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
+    unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
     asm volatile("" : "+s"(ks));
+    const char* qb = (const char*)q;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) r[k] = q[(unsigned)(lo + (16 * (k >> 2) + (k & 3)) * ks)];
+    for (int k = 0; k < 16; ++k) r[k] = *(const T*)(qb + (lo + (unsigned)(16 * (k >> 2) + (k & 3)) * ks));
 #pragma unroll
     for (int k = 0; k < 16; ++k) out[k] = BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k];
   } else {
@@ -395,13 +398,14 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
   T* q = (T*)const_cast<void*>(t.ptr) + ((long)b * t.s0 + (long)third * t.s2);
   const long ss = (long)rm.step * t.s1;
   if (rm.full) {
-    const int lo = rm.base * (int)t.s1 + n;
-    int ks = rm.step * (int)t.s1;
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
+    unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
     asm volatile("" : "+s"(ks));
+    char* qb = (char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      const unsigned o = (unsigned)(lo + (16 * (k >> 2) + (k & 3)) * ks);
-      if (BF) q[o] = (T)f_to_bf16(v[k]); else q[o] = (T)v[k];
+      T* d = (T*)(qb + (lo + (unsigned)(16 * (k >> 2) + (k & 3)) * ks));
+      if (BF) *d = (T)f_to_bf16(v[k]); else *d = (T)v[k];
     }
   } else {
 #pragma unroll
@@ -418,10 +422,12 @@ template <int CNT>
 __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int P, int N, int n, bool vn, int g4,
                                              bool full, float (&out)[CNT]) {
   if (full) {
-    const int lo = 4 * g4 * N + n;
-    asm volatile("" : "+s"(N));
+    const unsigned lo = (unsigned)(4 * g4 * N + n) * 4u;
+    unsigned nb = (unsigned)N * 4u;
+    asm volatile("" : "+s"(nb));
+    const char* sb = (const char*)src;
 #pragma unroll
-    for (int q = 0; q < CNT; ++q) out[q] = src[(unsigned)(lo + (16 * (q >> 2) + (q & 3)) * N)];
+    for (int q = 0; q < CNT; ++q) out[q] = *(const float*)(sb + (lo + (unsigned)(16 * (q >> 2) + (q & 3)) * nb));
   } else {
     float r[CNT];
     bool ok[CNT];

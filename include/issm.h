@@ -34,7 +34,7 @@
  *    into bf16 high and low parts (16 significand bits per operand; relative error of a
  *    product <= 2^-16); every other product is fp32.  Results are bit-reproducible
  *    from run to run (fixed-order reductions, no atomics).
- *  - Strides: stride[1] * seqlen must stay below 2^31 elements (row offsets are 32-bit).
+ *  - Strides: stride[1] * seqlen must stay below 2^30 elements (row byte offsets are 32-bit).
  */
 #ifndef ISSM_H
 #define ISSM_H
