@@ -93,9 +93,13 @@ __device__ __forceinline__ void stv(void* p, long i, int dt, float v) {
   if (dt) ((uint16_t*)p)[i] = f_to_bf16(v); else ((float*)p)[i] = v;
 }
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// (the hardware exp2 / log2 directly: the arguments here need none of the library's range fix-ups --
+// 1 + exp(x) >= 1 is never denormal and an exp that underflows to 0 is the right answer)
+__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + ex2(-x * LOG2E)); }
 // softplus as the reference evaluates it: log(exp(x) + 1) for x <= 20, identity above
-__device__ __forceinline__ float softplus_(float x) { return x <= 20.0f ? __logf(1.0f + __expf(x)) : x; }
+__device__ __forceinline__ float softplus_(float x) {
+  return x <= 20.0f ? LN2 * __builtin_amdgcn_logf(1.0f + ex2(x * LOG2E)) : x;
+}
 
 // Batched global loads / stores of one element type: all CNT accesses are issued before any
 // value is consumed.  The address is (uniform element offset ubase) + (per-lane 32-bit element
