@@ -167,10 +167,8 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       carry[k][j] = v ? p.dfinal[dir][(((long)b * p.H + h) * p.P + pp) * p.N + n + j] : 0.0f;
     }
   }
-  for (int c = p.nc - 1; c >= 0; --c) {
-    float gp[4] = {0, 0, 0, 0};
-    float dec[4], hn[4][4], dh[4][4];
-    // issue every load of this chunk before the dependent arithmetic
+  // operands of one chunk: decay exponent, H_{c+1} and dH_c of the thread's rows
+  auto load_chunk = [&](int c, float (&dec)[4], float (&hn)[4][4], float (&dh)[4][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) dec[j] = n + j < p.N ? cs_last[vec_off(p, bt, c, h) + n + j] : 0.0f;
 #pragma unroll
@@ -191,6 +189,15 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
         }
       }
     }
+  };
+  float dec[4], hn[4][4], dh[4][4];
+  load_chunk(p.nc - 1, dec, hn, dh);
+  for (int c = p.nc - 1; c >= 0; --c) {
+    float gp[4] = {0, 0, 0, 0};
+    // the next chunk's operands are requested before this chunk's arithmetic and reduction, so that the
+    // recurrence never waits for memory (the loads do not depend on the carry)
+    float dec_n[4], hn_n[4][4], dh_n[4][4];
+    if (c > 0) load_chunk(c - 1, dec_n, hn_n, dh_n);
 #pragma unroll
     for (int j = 0; j < 4; ++j) dec[j] = __expf(dec[j]);
 #pragma unroll
@@ -220,6 +227,14 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       if (ns * 64 + tid < p.N) g_last[vec_off(p, bt, c, h) + ns * 64 + tid] = sum;
     }
     __syncthreads();
+    if (c > 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dec[j] = dec_n[j];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { hn[k][j] = hn_n[k][j]; dh[k][j] = dh_n[k][j]; }
+    }
   }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
