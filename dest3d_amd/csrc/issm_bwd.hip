@@ -190,14 +190,15 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       }
     }
   };
-  float dec[4], hn[4][4], dh[4][4];
+  // The operands of the next two chunks are always in flight (the loads do not depend on the carry), so the
+  // recurrence never waits for memory and enough bytes are outstanding to keep HBM busy.
+  float dec[4], hn[4][4], dh[4][4], dec_1[4], hn_1[4][4], dh_1[4][4];
   load_chunk(p.nc - 1, dec, hn, dh);
+  if (p.nc > 1) load_chunk(p.nc - 2, dec_1, hn_1, dh_1);
   for (int c = p.nc - 1; c >= 0; --c) {
     float gp[4] = {0, 0, 0, 0};
-    // the next chunk's operands are requested before this chunk's arithmetic and reduction, so that the
-    // recurrence never waits for memory (the loads do not depend on the carry)
     float dec_n[4], hn_n[4][4], dh_n[4][4];
-    if (c > 0) load_chunk(c - 1, dec_n, hn_n, dh_n);
+    if (c > 1) load_chunk(c - 2, dec_n, hn_n, dh_n);
 #pragma unroll
     for (int j = 0; j < 4; ++j) dec[j] = __expf(dec[j]);
 #pragma unroll
@@ -227,14 +228,15 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       if (ns * 64 + tid < p.N) g_last[vec_off(p, bt, c, h) + ns * 64 + tid] = sum;
     }
     __syncthreads();
-    if (c > 0) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dec[j] = dec_n[j];
+    for (int j = 0; j < 4; ++j) { dec[j] = dec_1[j]; dec_1[j] = dec_n[j]; }
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
+    for (int k = 0; k < 4; ++k)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { hn[k][j] = hn_n[k][j]; dh[k][j] = dh_n[k][j]; }
-    }
+      for (int j = 0; j < 4; ++j) {
+        hn[k][j] = hn_1[k][j]; dh[k][j] = dh_1[k][j];
+        hn_1[k][j] = hn_n[k][j]; dh_1[k][j] = dh_n[k][j];
+      }
   }
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
