@@ -303,26 +303,36 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
   const long cstride = (long)p.H * p.P * p.N;
   float* sp = states + st_off(p, bt, 0, h) + (long)pp * p.N + n;
   const float* cl = cs_last + vec_off(p, bt, 0, h) + n;
-  for (int c = 0; c < p.nc; ++c) {
-    float sv[4], dv[4];
-    if (full) {
-      const f4 t = *(const f4*)sp;
-      const f4 d = *(const f4*)cl;
-      sv[0] = t.x; sv[1] = t.y; sv[2] = t.z; sv[3] = t.w;
-      dv[0] = d.x; dv[1] = d.y; dv[2] = d.z; dv[3] = d.w;
+  if (full) {
+    // S_c and the chunk decay of the next two chunks are always in flight: the loads do not depend on
+    // the running state, only the store into the slot just read does
+    const long dstride = (long)p.H * p.N;
+    f4 t0 = *(const f4*)sp, d0 = *(const f4*)cl, t1 = t0, d1 = d0;
+    if (p.nc > 1) { t1 = *(const f4*)(sp + cstride); d1 = *(const f4*)(cl + dstride); }
+    for (int c = 0; c < p.nc; ++c) {
+      f4 t2 = t1, d2 = d1;
+      if (c + 2 < p.nc) { t2 = *(const f4*)(sp + 2 * cstride); d2 = *(const f4*)(cl + 2 * dstride); }
       *(f4*)sp = (f4){st[0], st[1], st[2], st[3]};
-    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) st[j] = __expf(d0[j]) * st[j] + t0[j];
+      t0 = t1; d0 = d1; t1 = t2; d1 = d2;
+      sp += cstride;
+      cl += dstride;
+    }
+  } else {
+    for (int c = 0; c < p.nc; ++c) {
+      float sv[4], dv[4];
       for (int j = 0; j < 4; ++j) {
         const bool v = n + j < p.N;
         sv[j] = v ? sp[j] : 0.0f;
         dv[j] = v ? cl[j] : 0.0f;
         if (v) sp[j] = st[j];
       }
-    }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) st[j] = __expf(dv[j]) * st[j] + sv[j];
-    sp += cstride;
-    cl += (long)p.H * p.N;
+      for (int j = 0; j < 4; ++j) st[j] = __expf(dv[j]) * st[j] + sv[j];
+      sp += cstride;
+      cl += (long)p.H * p.N;
+    }
   }
   // slot nc keeps the final state for the backward pass
   for (int j = 0; j < 4; ++j)
