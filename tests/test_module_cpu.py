@@ -4,7 +4,7 @@
 def test_reference_state_dict_names():
     """The parameter names and shapes a reference checkpoint holds for this module
     (dest_module.py:469-513) load into the mirror."""
-    from dest3d_amd.dest_module import MultiHeadISSMScan
+    from dest3d_amd.scan_module import MultiHeadISSMScan
     m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1)
     want = {
         "dt_bias": (8,), "A_log": (8,), "D": (8,), "key_proj.weight": (2 * 288 + 2 + 8, 288),

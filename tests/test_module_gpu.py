@@ -71,7 +71,7 @@ def _module_ref(sd, cfg, in_key, in_query, dist, mask):
 
 @pytest.mark.parametrize("biscan,mask_kind", [(True, None), (True, "float"), (False, "bool")])
 def test_module_matches_fp64_evaluation(biscan, mask_kind):
-    from dest3d_amd.dest_module import MultiHeadISSMScan
+    from dest3d_amd.scan_module import MultiHeadISSMScan
     print(f"[case] module mirror biscan={biscan} mask={mask_kind}", flush=True)
     sys.stdout.flush()
     torch.manual_seed(7)
@@ -114,7 +114,7 @@ def test_six_layer_stack_bf16_at_detector_shape():
     """Six mirror layers at the detector's decoder shape (d_model 288, 8 heads of 36, K = 256 queries,
     L = 1024 keys, batch 8, d_dist 16), bf16 forward + backward, against the same stack in fp32 on the
     bf16-rounded weights and inputs.  The fp32 stack is pinned by test_module_matches_fp64_evaluation."""
-    from dest3d_amd.dest_module import MultiHeadISSMScan
+    from dest3d_amd.scan_module import MultiHeadISSMScan
     print("[case] six-layer bf16 stack B=8 L=1024 K=256 d_model=288", flush=True)
     torch.manual_seed(11)
     layers = torch.nn.ModuleList(MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8,
