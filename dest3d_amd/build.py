@@ -43,5 +43,19 @@ def build(verbose: bool = True) -> str:
     return LIB
 
 
+def build_probe() -> str:
+    """Stand-alone issue-rate probe (matrix vs vector instructions); not part of the library."""
+    out = os.path.join(HERE, "probe_mfma_valu")
+    cmd = [HIPCC, *[f for f in FLAGS if f != "-fPIC"], os.path.join(CSRC, "probe_mfma_valu.hip"), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for the probe:\n{r.stderr}")
+    print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
-    build()
+    if "--probe" in sys.argv[1:]:
+        build_probe()
+    else:
+        build()
