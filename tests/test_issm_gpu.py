@@ -439,3 +439,25 @@ def test_large_bidirectional_fp32_shape():
         _check(name, ai, bi, FWD32)
     for k in ref:
         _check("d" + k, gg[k].grad, ref[k].grad, BWD32)
+
+
+def test_extreme_decay_is_finite_and_accurate():
+    """Decays that underflow within a few rows (|dt' A| up to ~3000 per step) and rows that do not decay at all
+    (dt' = 0) in the same chunk: the level factors never exceed 1, so nothing may overflow.  Accuracy bar here:
+    1e-3 instead of 1e-4 / 1e-3 -- with running sums of dt' A in the thousands, one fp32 ulp of the sum (the
+    reference keeps it in fp32 as well, issm_chunk_state.py:84-104) is already ~5e-4 in the exponent."""
+    _say("extreme decay")
+    d = _problem(1, 192, 2, 32, 64, 1, seed=21, softplus=False)
+    g = torch.Generator().manual_seed(22)
+    dt = torch.rand(1, 192, 2, 64, generator=g) * 3.0
+    dt[:, ::5] = 0.0                                   # rows without decay or input
+    dt[:, 7::11] *= 10.0                               # rows that wipe the state
+    d["dt"] = dt
+    d["A"] = -torch.exp(torch.rand(2, 64, generator=g) * math.log(100.0))
+    y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+    y, fin, gr, _ = _run_operator(d, torch.float32)
+    _check("out", y, y_ref, 1e-3)
+    _check("final_states", fin, fin_ref, 1e-3)
+    for k in GRAD_NAMES:
+        if d[k] is not None:
+            _check("d" + k, gr[k], g_ref[k], 1e-2 if k in ("dt", "A") else 1e-3)
