@@ -11,7 +11,7 @@ Besides the driver's JSON contract the line carries
   cpu_baseline  the oracle's chunked pure-PyTorch formulation timed on the host cores
   stages_us     average duration of every kernel of the step
   variants_us   fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants (also at the
-                detector's head dimension 36)
+                detector's head dimension 36), and of one whole detector layer around the scan
 """
 import argparse
 import ctypes as C
@@ -190,6 +190,31 @@ def cpu_baseline(torch):
             "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional"}
 
 
+def time_module_layer(torch, steps=10, warmup=3):
+    """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
+    keys, batch 8, d_dist 16, bf16), forward + backward through autograd, microseconds.  Includes the PyTorch
+    projections, conv and norms around the scan."""
+    from dest3d_amd.scan_module import MultiHeadISSMScan
+    torch.manual_seed(0)
+    m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1).cuda().bfloat16()
+    key = torch.randn(8, 1024, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    query = torch.randn(8, 256, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    dist = (0.5 * torch.randn(8, 1024, 256, 16, device="cuda")).bfloat16().requires_grad_()
+
+    def step():
+        ok, oq = m(key, query, dist, None)
+        (ok.float().square().mean() + oq.float().square().mean()).backward()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e6
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -246,6 +271,7 @@ def main():
             variants[name] = round(r.time_steps(max(args.steps // 2, 5), 5), 2)
             del r
         SHAPE["P"] = 32
+        variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),

@@ -101,12 +101,30 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
   for (int c = lane; c < p.ncols; c += 64) p.dw_partial[(long)blockIdx.x * p.ncols + c] = dws[c];
 }
 
+// dw[c] = sum over the per-block partials, in a fixed order: block = 32 columns x 8 row groups, row group g
+// adds partials g, g+8, ... with four independent accumulators, then the 8 group sums are combined in order.
 __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_dw(NormP p) {
-  const int c = blockIdx.x * NTHREADS + threadIdx.x;
-  if (c >= p.ncols) return;
-  float a = 0.0f;
-  for (int b = 0; b < p.nblocks; ++b) a += p.dw_partial[(long)b * p.ncols + c];
-  p.dw[c] = a;
+  __shared__ float red[NTHREADS];
+  const int c = blockIdx.x * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  if (c < p.ncols) {
+    int b = g;
+    for (; b + 24 < p.nblocks; b += 32) {
+      a0 += p.dw_partial[(long)b * p.ncols + c];
+      a1 += p.dw_partial[(long)(b + 8) * p.ncols + c];
+      a2 += p.dw_partial[(long)(b + 16) * p.ncols + c];
+      a3 += p.dw_partial[(long)(b + 24) * p.ncols + c];
+    }
+    for (; b < p.nblocks; b += 8) a0 += p.dw_partial[(long)b * p.ncols + c];
+  }
+  red[threadIdx.x] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (g == 0 && c < p.ncols) {
+    float t = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += red[k * 32 + (threadIdx.x & 31)];
+    p.dw[c] = t;
+  }
 }
 
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st) {
@@ -119,7 +137,7 @@ int launch_rmsnorm_bwd(const NormP& p, hipStream_t st) {
   hipLaunchKernelGGL(k_rmsnorm_bwd, dim3(p.nblocks), dim3(64), (size_t)p.ncols * sizeof(float), st, p);
   int e = (int)hipGetLastError();
   if (e) return e;
-  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + NTHREADS - 1) / NTHREADS), dim3(NTHREADS), 0, st, p);
+  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 31) / 32), dim3(NTHREADS), 0, st, p);
   return (int)hipGetLastError();
 }
 
