@@ -24,6 +24,7 @@ EXPORTS = [
     "issm_stage_chunk_scan", "issm_stage_bwd_gate", "issm_stage_bwd_dstates",
     "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_stage_bwd_dx", "issm_stage_bwd_reduce",
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
+    "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
 ]
 
 
@@ -76,6 +77,19 @@ class NormArgs(C.Structure):
     ]
 
 
+class PGenArgs(C.Structure):
+    _fields_ = [
+        ("tokens", C.c_int64), ("K", C.c_int32), ("M", C.c_int32), ("H", C.c_int32), ("G", C.c_int32),
+        ("dtype", C.c_int32), ("has_back", C.c_int32),
+        ("dist", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p),
+        ("dt", C.c_void_p), ("Bm", C.c_void_p), ("Cm", C.c_void_p), ("Bm_back", C.c_void_p), ("Cm_back", C.c_void_p),
+        ("ddt", C.c_void_p), ("dBm", C.c_void_p), ("dCm", C.c_void_p), ("dBm_back", C.c_void_p),
+        ("dCm_back", C.c_void_p),
+        ("ddist", C.c_void_p), ("dbias", C.c_void_p), ("dw_partial", C.c_void_p), ("dW", C.c_void_p),
+        ("stream", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -108,6 +122,9 @@ def load() -> C.CDLL:
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
+    lib.issm_param_gen_bwd_blocks.argtypes = [C.c_int64]
+    lib.issm_param_gen_fwd.argtypes = [P(PGenArgs)]
+    lib.issm_param_gen_bwd.argtypes = [P(PGenArgs)]
     for name in EXPORTS:
         if name != "issm_last_error":
             getattr(lib, name).restype = C.c_int

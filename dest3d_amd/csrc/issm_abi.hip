@@ -25,6 +25,9 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
+int pgen_bwd_blocks(long tokens);
+int launch_pgen_fwd(const PGenP& p, hipStream_t st);
+int launch_pgen_bwd(const PGenP& p, hipStream_t st);
 }  // namespace issm
 
 using namespace issm;
@@ -397,6 +400,47 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* a) {
   int rc = norm_params(a, &p, true);
   if (rc) return rc;
   return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd");
+}
+
+static int pgen_params(const issm_pgen_args* a, PGenP* p, bool bwd) {
+  if (!a) return fail(ISSM_E_NULL, "param_gen: args is NULL");
+  if (a->tokens < 0 || a->K < 0 || a->H < 1 || a->G < 1) return fail(ISSM_E_SHAPE, "param_gen: bad shape");
+  if (a->M != 16) return fail(ISSM_E_UNSUPPORTED, "param_gen: M = %d (only 16 is built)", a->M);
+  if (a->H + 2 * a->G > 12) return fail(ISSM_E_UNSUPPORTED, "param_gen: H + 2G = %d > 12", a->H + 2 * a->G);
+  if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "param_gen: dtype %d", a->dtype);
+  if (a->tokens * (int64_t)a->K * 16 >= ((int64_t)1 << 40)) return fail(ISSM_E_SHAPE, "param_gen: too large");
+  if (!a->dist || !a->W) return fail(ISSM_E_NULL, "param_gen: dist/W is NULL");
+  if (!bwd) {
+    if (!a->bias || !a->dt || !a->Bm || !a->Cm) return fail(ISSM_E_NULL, "param_gen: bias/dt/Bm/Cm is NULL");
+    if (a->has_back && (!a->Bm_back || !a->Cm_back)) return fail(ISSM_E_NULL, "param_gen: Bm_back/Cm_back is NULL");
+  } else {
+    if (!a->dw_partial || !a->dW) return fail(ISSM_E_NULL, "param_gen bwd: dw_partial/dW is NULL");
+  }
+  p->tokens = a->tokens; p->K = a->K; p->H = a->H; p->G = a->G; p->dtype = a->dtype; p->has_back = a->has_back ? 1 : 0;
+  p->dist = a->dist; p->W = a->W; p->bias = a->bias;
+  p->dt = a->dt; p->Bm = a->Bm; p->Cm = a->Cm; p->Bb = a->Bm_back; p->Cb = a->Cm_back;
+  p->ddt = a->ddt; p->dB = a->dBm; p->dC = a->dCm; p->dBb = a->dBm_back; p->dCb = a->dCm_back;
+  p->ddist = a->ddist; p->dbias = a->dbias; p->dw_partial = a->dw_partial; p->dW = a->dW;
+  p->nblocks = pgen_bwd_blocks(a->tokens);
+  return ISSM_OK;
+}
+
+int issm_param_gen_bwd_blocks(int64_t tokens) { return tokens > 0 ? pgen_bwd_blocks(tokens) : 0; }
+
+int issm_param_gen_fwd(const issm_pgen_args* a) {
+  PGenP p;
+  int rc = pgen_params(a, &p, false);
+  if (rc) return rc;
+  if (p.tokens == 0 || p.K == 0) return ISSM_OK;
+  return launched(launch_pgen_fwd(p, (hipStream_t)a->stream), "param_gen_fwd");
+}
+
+int issm_param_gen_bwd(const issm_pgen_args* a) {
+  PGenP p;
+  int rc = pgen_params(a, &p, true);
+  if (rc) return rc;
+  if (p.tokens == 0) return ISSM_OK;
+  return launched(launch_pgen_bwd(p, (hipStream_t)a->stream), "param_gen_bwd");
 }
 
 }  // extern "C"

@@ -78,6 +78,22 @@ struct NormP {
   int nblocks;
 };
 
+// parameters of the dt / B / C generation kernels (param_gen.hip)
+struct PGenP {
+  long tokens;
+  int K, H, G, dtype, has_back;
+  const void* dist;      // (tokens, K, M) io dtype
+  const float* W;        // (R0, M) fp32
+  const float* bias;     // (tokens, R) fp32, R = R0 + (has_back ? 2G : 0)
+  void *dt, *Bm, *Cm, *Bb, *Cb;                    // (tokens, H|G, K) io dtype
+  const void *ddt, *dB, *dC, *dBb, *dCb;           // gradients of the outputs
+  void* ddist;           // (tokens, K, M) io dtype
+  float* dbias;          // (tokens, R) fp32
+  float* dw_partial;     // (nblocks, R0, M) fp32
+  float* dW;             // (R0, M) fp32
+  int nblocks;
+};
+
 __device__ __forceinline__ float bf16_to_f(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float f) {
   uint32_t u = __float_as_uint(f);

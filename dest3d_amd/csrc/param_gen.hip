@@ -1,0 +1,391 @@
+// Generation of the scan's dt / B / C from the pairwise distance encoding (gfx950).
+//
+// DEST builds the per-(token, query) scan parameters as tiny projections of `dist` (tokens, K, M):
+//   base[r][k] = sum_m W[r][m] dist[k][m],   r = 0 .. R0-1,  R0 = H + 2G  (dt heads, B groups, C groups)
+//   dt[h][k] = base[h][k] + bias[h],  B[g][k] = base[H+g][k] + bias[H+g],  C[g][k] = base[H+G+g][k] + bias[H+G+g]
+// and, for the reversed-order scan, a second B / C pair from the same base rows with their own biases
+// (models/dest_module.py:543-553).  As library GEMMs these are thousands of (R0 x M)(M x K) products with
+// M = 16: launch- and layout-bound.  Here one pass reads `dist` once and writes every output; the backward is
+// one pass as well (ddist, per-token bias gradients, per-workgroup partials of dW) plus a fixed-order
+// reduction of the partials.  Everything is memory bound; arithmetic is fp32.
+#include "issm_dev.h"
+
+namespace issm {
+
+constexpr int PG_MAXR0 = 12;  // largest H + 2G built (three 4-row steps of the matrix instruction)
+constexpr int PG_M = 16;      // distance encoding width this kernel is built for
+constexpr int PG_UNR = 4;     // blocks of 16 k whose loads are in flight together in the backward
+constexpr int PG_TOK = 4;     // tokens per workgroup in the backward (one per wave)
+
+template <bool BF>
+__device__ __forceinline__ void load_row16(const void* p, long off, float (&v)[PG_M]) {
+  if (BF) {
+    const uint4* q = (const uint4*)((const uint16_t*)p + off);
+    const uint4 a = q[0], b = q[1];
+    const unsigned w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  } else {
+    const f4* q = (const f4*)((const float*)p + off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f4 a = q[i];
+      v[4 * i] = a.x; v[4 * i + 1] = a.y; v[4 * i + 2] = a.z; v[4 * i + 3] = a.w;
+    }
+  }
+}
+template <bool BF>
+__device__ __forceinline__ void store_row16(void* p, long off, const float (&v)[PG_M]) {
+  if (BF) {
+    unsigned w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = (unsigned)f_to_bf16(v[2 * i]) | ((unsigned)f_to_bf16(v[2 * i + 1]) << 16);
+    uint4* q = (uint4*)((uint16_t*)p + off);
+    q[0] = make_uint4(w[0], w[1], w[2], w[3]);
+    q[1] = make_uint4(w[4], w[5], w[6], w[7]);
+  } else {
+    f4* q = (f4*)((float*)p + off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = (f4){v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]};
+  }
+}
+template <bool BF>
+__device__ __forceinline__ float ld1(const void* p, long i) {
+  return BF ? bf16_to_f(((const uint16_t*)p)[i]) : ((const float*)p)[i];
+}
+template <bool BF>
+__device__ __forceinline__ void st1(void* p, long i, float v) {
+  if (BF) ((uint16_t*)p)[i] = f_to_bf16(v); else ((float*)p)[i] = v;
+}
+
+// two floats -> two bf16 (round to nearest even) in one dword
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float fl2 __attribute__((ext_vector_type(2)));
+  const bf2 h = __builtin_convertvector((fl2){lo, hi}, bf2);
+  return __builtin_bit_cast(unsigned, h);
+}
+
+// Forward: thread = (token, k).  W and the token's biases are uniform across the workgroup's lanes of a token.
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_pgen_fwd(PGenP p) {
+  const int R0 = p.H + 2 * p.G, R = R0 + (p.has_back ? 2 * p.G : 0);
+  const int kchunks = (p.K + NTHREADS - 1) / NTHREADS;
+  const long t = blockIdx.x / kchunks;
+  const int k = (blockIdx.x % kchunks) * NTHREADS + threadIdx.x;
+  if (k >= p.K) return;
+  float d[PG_M];
+  load_row16<BF>(p.dist, (t * p.K + k) * PG_M, d);
+  const float* bias = p.bias + t * R;
+  for (int r = 0; r < R0; ++r) {
+    const float* w = p.W + r * PG_M;  // uniform: scalar loads
+    float s = 0.0f;
+#pragma unroll
+    for (int m = 0; m < PG_M; ++m) s = fmaf(w[m], d[m], s);
+    if (r < p.H) {
+      st1<BF>(p.dt, (t * p.H + r) * p.K + k, s + bias[r]);
+    } else if (r < p.H + p.G) {
+      const int g = r - p.H;
+      st1<BF>(p.Bm, (t * p.G + g) * p.K + k, s + bias[r]);
+      if (p.has_back) st1<BF>(p.Bb, (t * p.G + g) * p.K + k, s + bias[R0 + g]);
+    } else {
+      const int g = r - p.H - p.G;
+      st1<BF>(p.Cm, (t * p.G + g) * p.K + k, s + bias[r]);
+      if (p.has_back) st1<BF>(p.Cb, (t * p.G + g) * p.K + k, s + bias[R0 + p.G + g]);
+    }
+  }
+}
+
+// Gradient row r of token t: dt heads, then B groups, then C groups (`back`: the reversed-order pair, which
+// exists for the B / C rows only).  Returns the element offset of (t, row, k = 0), or -1 when there is none.
+struct GradRows {
+  const void *ddt, *dB, *dC, *dBb, *dCb;
+  int H, G, K;
+  __device__ __forceinline__ const void* base(int r, bool back) const {
+    if (r < H) return back ? nullptr : ddt;
+    if (r < H + G) return back ? dBb : dB;
+    if (r < H + 2 * G) return back ? dCb : dC;
+    return nullptr;
+  }
+  __device__ __forceinline__ long offset(long t, int r) const {
+    if (r < H) return (t * H + r) * K;
+    if (r < H + G) return (t * G + (r - H)) * K;
+    return (t * G + (r - H - G)) * K;
+  }
+};
+
+// Loads without branches: a lane with nothing to read (no such row, k past the end) reads element 0 of `safe`
+// -- any readable buffer of at least 16 bytes -- and the value is replaced by zero afterwards.  Branch-free
+// loads can all be in flight together; a branch per load would serialise them.
+template <bool BF>
+__device__ __forceinline__ float ld1_or0(const void* p, long off, bool ok, const void* safe) {
+  const float v = ld1<BF>(ok ? p : safe, ok ? off : 0);
+  return ok ? v : 0.0f;
+}
+// Four consecutive elements p[off .. off + 3] for k .. k + 3 (k >= kend reads as zero).  `vec`: the address is
+// aligned for one wide load and kend is a multiple of 4.
+template <bool BF>
+__device__ __forceinline__ f4 load4(const void* p, long off, int k, int kend, bool vec, const void* safe) {
+  f4 r;
+  if (vec) {  // uniform
+    const bool ok = p != nullptr && k < kend;
+    const void* q = ok ? p : safe;
+    const long o = ok ? off : 0;
+    if (BF) {
+      const uint2 w = *(const uint2*)((const uint16_t*)q + o);
+      r.x = __uint_as_float(w.x << 16); r.y = __uint_as_float(w.x & 0xffff0000u);
+      r.z = __uint_as_float(w.y << 16); r.w = __uint_as_float(w.y & 0xffff0000u);
+    } else {
+      r = *(const f4*)((const float*)q + o);
+    }
+    if (!ok) r = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) r[v] = ld1_or0<BF>(p, off + v, p != nullptr && k + v < kend, safe);
+  }
+  return r;
+}
+
+// Backward on the matrix cores (v_mfma_f32_16x16x4_f32; lane = (i = lane & 15, q = lane >> 4)).
+// Workgroup = PG_TOK consecutive tokens, a wave owns PG_TOK / 4 of them and walks k in blocks of 16:
+//   ddist^T (m x k) = W^T (m x r) g (r x k)   -- A: lane (m, q) = W[4s + q][m], B: lane (k, q) = g[4s + q][k0 + k];
+//                                                the result lane (k, q) holds ddist[k0 + k][4q .. 4q + 3]: one wide store
+//   dW (r x m)     += g (r x k) dist (k x m)  -- A: lane (r, q) = g[r][k0 + 4q + v], B: lane (m, q) = dist[k0 + 4q + v][m],
+//                                                v = 0..3 (the order of k inside the sum is free)
+//   dbias[r]        = sum_k g[r][k]           -- from the second layout, reduced over q at the end of the token.
+// g of a B / C row is the sum of its forward-order and reversed-order gradients wherever the shared base row is
+// differentiated; the two bias gradients stay apart.
+// FULLK: K is a multiple of 16 * PG_UNR, so no load or store needs a bound on k, and every per-lane address is a
+// pointer advanced once per trip plus a compile-time offset.
+template <bool BF, bool FULLK>
+__global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
+  __shared__ float wred[4][16 * PG_M];
+  const int R0 = p.H + 2 * p.G, R = R0 + (p.has_back ? 2 * p.G : 0);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane & 15, q = lane >> 4;
+  const int K = p.K;
+  const bool vec = (K & 3) == 0;
+  const GradRows gr{p.ddt, p.dB, p.dC, p.has_back ? p.dBb : nullptr, p.has_back ? p.dCb : nullptr, p.H, p.G, K};
+  float wA[3];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) wA[s] = (4 * s + q < R0) ? p.W[(4 * s + q) * PG_M + i] : 0.0f;
+  // row-of-the-lane pointers: layout 2 (row i), layout 1 (rows 4s + q)
+  const void* g2 = gr.base(i, false);
+  const void* g2b = gr.base(i, true);
+  const void *g1[3], *g1b[3];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    g1[s] = gr.base(4 * s + q, false);
+    g1b[s] = gr.base(4 * s + q, true);
+  }
+  const bool any_back = gr.dBb != nullptr || gr.dCb != nullptr;  // uniform
+  f4 accW = {0.0f, 0.0f, 0.0f, 0.0f};
+  constexpr int TPW = PG_TOK / 4;
+  for (int ti = 0; ti < TPW; ++ti) {
+    const long t = (long)blockIdx.x * PG_TOK + wave * TPW + ti;
+    if (t >= p.tokens) break;  // wave-uniform
+    const long o2 = i < R0 ? gr.offset(t, i) : 0;
+    long o1[3];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) o1[s] = (4 * s + q < R0) ? gr.offset(t, 4 * s + q) : 0;
+    float bs = 0.0f, bsb = 0.0f;
+    if constexpr (FULLK) {
+      typedef typename std::conditional<BF, uint16_t, float>::type T;
+      typedef typename std::conditional<BF, uint2, f4>::type T4;
+      const T* nil = (const T*)p.dist;  // what a lane with no row reads (at least 64 * 16 elements long)
+      const bool ok2 = g2 != nullptr, ok2b = g2b != nullptr;
+      const T* pa = ok2 ? (const T*)g2 + o2 + 4 * q : nil;
+      const T* pab = ok2b ? (const T*)g2b + o2 + 4 * q : nil;
+      const T* pd = (const T*)p.dist + (t * K + 4 * q) * PG_M + i;
+      const T *pg[3], *pgb[3];
+      bool okg[3], okgb[3];
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+        okg[s] = g1[s] != nullptr;
+        okgb[s] = g1b[s] != nullptr;
+        pg[s] = okg[s] ? (const T*)g1[s] + o1[s] + i : nil;
+        pgb[s] = okgb[s] ? (const T*)g1b[s] + o1[s] + i : nil;
+      }
+      T* pdd = (T*)p.ddist + (t * K + i) * PG_M + 4 * q;
+      auto widen = [](T4 w) -> f4 {
+        if constexpr (BF) {
+          return (f4){__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                      __uint_as_float(w.y & 0xffff0000u)};
+        } else {
+          return w;
+        }
+      };
+      auto widen1 = [](T w) -> float {
+        if constexpr (BF) return __uint_as_float((unsigned)w << 16);
+        else return w;
+      };
+      const f4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      for (int kb = 0; kb < K; kb += 16 * PG_UNR) {
+        T4 ra[PG_UNR], rab[PG_UNR];
+        T rd[PG_UNR][4], rg[PG_UNR][3], rgb[PG_UNR][3];
+#pragma unroll
+        for (int u = 0; u < PG_UNR; ++u) {
+          ra[u] = *(const T4*)(pa + 16 * u);
+          if (any_back) rab[u] = *(const T4*)(pab + 16 * u);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) rd[u][v] = pd[(16 * u + v) * PG_M];
+#pragma unroll
+          for (int s = 0; s < 3; ++s) {
+            rg[u][s] = pg[s][16 * u];
+            if (any_back) rgb[u][s] = pgb[s][16 * u];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < PG_UNR; ++u) {
+          // rows past R0 hold finite or non-finite junk in `a`: they only reach rows of dW that are never read
+          const f4 a = widen(ra[u]);
+          const f4 ab = (any_back && ok2b) ? widen(rab[u]) : zero4;
+          bs += (a.x + a.y) + (a.z + a.w);
+          bsb += (ab.x + ab.y) + (ab.z + ab.w);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) accW = mfma4(a[v] + ab[v], widen1(rd[u][v]), accW);
+          if (p.ddist) {
+            f4 dd = zero4;
+#pragma unroll
+            for (int s = 0; s < 3; ++s) {
+              float x = okg[s] ? widen1(rg[u][s]) : 0.0f;
+              if (any_back) x += okgb[s] ? widen1(rgb[u][s]) : 0.0f;
+              dd = mfma4(wA[s], x, dd);
+            }
+            if constexpr (BF) {
+              uint2 w;
+              w.x = pack_bf16(dd.x, dd.y);
+              w.y = pack_bf16(dd.z, dd.w);
+              *(uint2*)(pdd + 16 * u * PG_M) = w;
+            } else {
+              *(f4*)(pdd + 16 * u * PG_M) = dd;
+            }
+          }
+        }
+        const int step = 16 * PG_UNR;
+        pa += ok2 ? step : 0;
+        pab += ok2b ? step : 0;
+        pd += step * PG_M;
+        pdd += step * PG_M;
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+          pg[s] += okg[s] ? step : 0;
+          pgb[s] += okgb[s] ? step : 0;
+        }
+      }
+    } else {
+      // PG_UNR blocks of 16 k per trip: every load of the trip is issued before the first product needs one
+      for (int kb = 0; kb < K; kb += 16 * PG_UNR) {
+        f4 a[PG_UNR], ab[PG_UNR];
+        float dv[PG_UNR][4], gk[PG_UNR][3], gkb[PG_UNR][3];
+  #pragma unroll
+        for (int u = 0; u < PG_UNR; ++u) {
+          const int k0 = kb + 16 * u, kq = k0 + 4 * q;
+          a[u] = load4<BF>(g2, o2 + kq, kq, K, vec, p.W);
+          ab[u] = any_back ? load4<BF>(g2b, o2 + kq, kq, K, vec, p.W) : (f4){0.0f, 0.0f, 0.0f, 0.0f};
+  #pragma unroll
+          for (int v = 0; v < 4; ++v) dv[u][v] = ld1_or0<BF>(p.dist, (t * K + kq + v) * PG_M + i, kq + v < K, p.W);
+  #pragma unroll
+          for (int s = 0; s < 3; ++s) {
+            const bool in = k0 + i < K;
+            gk[u][s] = ld1_or0<BF>(g1[s], o1[s] + k0 + i, in && g1[s] != nullptr, p.W);
+            if (any_back) gkb[u][s] = ld1_or0<BF>(g1b[s], o1[s] + k0 + i, in && g1b[s] != nullptr, p.W);
+            else gkb[u][s] = 0.0f;
+          }
+        }
+  #pragma unroll
+        for (int u = 0; u < PG_UNR; ++u) {
+          const int k0 = kb + 16 * u;
+          bs += (a[u].x + a[u].y) + (a[u].z + a[u].w);
+          bsb += (ab[u].x + ab[u].y) + (ab[u].z + ab[u].w);
+  #pragma unroll
+          for (int v = 0; v < 4; ++v) accW = mfma4(a[u][v] + ab[u][v], dv[u][v], accW);
+          if (p.ddist) {
+            f4 dd = {0.0f, 0.0f, 0.0f, 0.0f};
+  #pragma unroll
+            for (int s = 0; s < 3; ++s) dd = mfma4(wA[s], gk[u][s] + gkb[u][s], dd);
+            if (k0 + i < K) {
+              const long o = (t * K + k0 + i) * PG_M + 4 * q;
+              if (BF) {
+                uint2 w;
+                w.x = (unsigned)f_to_bf16(dd.x) | ((unsigned)f_to_bf16(dd.y) << 16);
+                w.y = (unsigned)f_to_bf16(dd.z) | ((unsigned)f_to_bf16(dd.w) << 16);
+                *(uint2*)((uint16_t*)p.ddist + o) = w;
+              } else {
+                *(f4*)((float*)p.ddist + o) = dd;
+              }
+            }
+          }
+        }
+      }
+    }
+    bs += __shfl_xor(bs, 16, 64);
+    bs += __shfl_xor(bs, 32, 64);
+    bsb += __shfl_xor(bsb, 16, 64);
+    bsb += __shfl_xor(bsb, 32, 64);
+    if (p.dbias && q == 0 && i < R0) {
+      p.dbias[t * R + i] = bs;
+      if (p.has_back && i >= p.H) p.dbias[t * R + R0 + (i - p.H)] = bsb;
+    }
+  }
+  // dW partial of the workgroup: the four waves in order.  Lane (m, q) holds rows 4q .. 4q + 3 of column m.
+#pragma unroll
+  for (int v = 0; v < 4; ++v) wred[wave][(4 * q + v) * PG_M + i] = accW[v];
+  __syncthreads();
+  for (int e = threadIdx.x; e < R0 * PG_M; e += NTHREADS)
+    p.dw_partial[(long)blockIdx.x * R0 * PG_M + e] = (wred[0][e] + wred[1][e]) + (wred[2][e] + wred[3][e]);
+}
+
+// dW = fixed-order sum of the per-workgroup partials: one workgroup per entry of dW
+__global__ __launch_bounds__(NTHREADS) void k_pgen_dw(PGenP p) {
+  __shared__ float red[NTHREADS];
+  const int n = (p.H + 2 * p.G) * PG_M;
+  const int c = blockIdx.x;
+  float a0 = 0.0f, a1 = 0.0f;
+  int b = threadIdx.x;
+  for (; b + NTHREADS < p.nblocks; b += 2 * NTHREADS) {
+    a0 += p.dw_partial[(long)b * n + c];
+    a1 += p.dw_partial[(long)(b + NTHREADS) * n + c];
+  }
+  if (b < p.nblocks) a0 += p.dw_partial[(long)b * n + c];
+  red[threadIdx.x] = a0 + a1;
+  __syncthreads();
+#pragma unroll
+  for (int w = NTHREADS / 2; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) p.dW[c] = red[0];
+}
+
+int pgen_bwd_blocks(long tokens) { return (int)((tokens + PG_TOK - 1) / PG_TOK); }
+
+int launch_pgen_fwd(const PGenP& p, hipStream_t st) {
+  const long kchunks = (p.K + NTHREADS - 1) / NTHREADS;
+  const unsigned blocks = (unsigned)(p.tokens * kchunks);
+  if (p.dtype) hipLaunchKernelGGL(k_pgen_fwd<true>, dim3(blocks), dim3(NTHREADS), 0, st, p);
+  else hipLaunchKernelGGL(k_pgen_fwd<false>, dim3(blocks), dim3(NTHREADS), 0, st, p);
+  return (int)hipGetLastError();
+}
+
+int launch_pgen_bwd(const PGenP& p, hipStream_t st) {
+  const int R0 = p.H + 2 * p.G;
+  const unsigned blocks = (unsigned)p.nblocks;
+  const bool fullk = p.K % (16 * PG_UNR) == 0;
+  if (p.dtype) {
+    if (fullk) hipLaunchKernelGGL((k_pgen_bwd<true, true>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    else hipLaunchKernelGGL((k_pgen_bwd<true, false>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+  } else {
+    if (fullk) hipLaunchKernelGGL((k_pgen_bwd<false, true>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    else hipLaunchKernelGGL((k_pgen_bwd<false, false>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+  }
+  int e = (int)hipGetLastError();
+  if (e) return e;
+  hipLaunchKernelGGL(k_pgen_dw, dim3(R0 * PG_M), dim3(NTHREADS), 0, st, p);
+  return (int)hipGetLastError();
+}
+
+}  // namespace issm

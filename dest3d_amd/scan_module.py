@@ -22,6 +22,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import param_gen
 from .issm_combined import ISSM_biscan_combined, ISSM_chunk_scan_combined
 from .layernorm_gated import RMSNorm as RMSNormGated
 
@@ -96,19 +97,30 @@ class MultiHeadISSMScan(nn.Module):
         h0 = self.query_proj(in_query)                                   # (B, K, H*P)
         out["initial_states"] = h0.unflatten(-1, (H, P)).permute(0, 2, 3, 1)   # (B, H, P, K) view
         out["A"] = (-torch.exp(self.A_log.float()))[:, None].expand(H, self.d_state)
-        # W (G|H, M) @ dist^T (B,L,M,K): the product is written straight into (B,L,G|H,K), K contiguous
-        dist_t = dist.transpose(-1, -2)
-        b_base = torch.matmul(self.bc_proj.weight[:G], dist_t)
-        c_base = torch.matmul(self.bc_proj.weight[G:], dist_t)
-        out["B"] = b_base + b_bias.unsqueeze(-1)
-        out["C"] = c_base + c_bias.unsqueeze(-1)
+        dt_tok_bias = dt_tok + self.dt_bias.to(dt_tok.dtype)
         if self.use_biscan:
             xbc_b = self.key_conv_back(key_xyz, xbc)
             x_b, b_bias_b, c_bias_b = torch.split(xbc_b, [self.d_inner, G, G], dim=-1)
             out["x_back"] = x_b.contiguous().unflatten(-1, (H, P))
-            out["B_back"] = b_base + b_bias_b.unsqueeze(-1)
-            out["C_back"] = c_base + c_bias_b.unsqueeze(-1)
-        dt_raw = torch.matmul(self.dt_proj.weight, dist_t) + (dt_tok + self.dt_bias.to(dt_tok.dtype)).unsqueeze(-1)
+        if param_gen.supported(dist, H, G):
+            # one pass over dist writes every (B,L,H|G,K) operand (dest_module.py:541-553)
+            W = torch.cat([self.dt_proj.weight, self.bc_proj.weight], dim=0)
+            cols = [dt_tok_bias, b_bias, c_bias] + ([b_bias_b, c_bias_b] if self.use_biscan else [])
+            res = param_gen.scan_params(dist, W, torch.cat(cols, dim=-1).float(), H, G, self.use_biscan)
+            dt_raw, out["B"], out["C"] = res[:3]
+            if self.use_biscan:
+                out["B_back"], out["C_back"] = res[3:]
+        else:
+            # W (G|H, M) @ dist^T (B,L,M,K): the product is written straight into (B,L,G|H,K), K contiguous
+            dist_t = dist.transpose(-1, -2)
+            b_base = torch.matmul(self.bc_proj.weight[:G], dist_t)
+            c_base = torch.matmul(self.bc_proj.weight[G:], dist_t)
+            out["B"] = b_base + b_bias.unsqueeze(-1)
+            out["C"] = c_base + c_bias.unsqueeze(-1)
+            if self.use_biscan:
+                out["B_back"] = b_base + b_bias_b.unsqueeze(-1)
+                out["C_back"] = c_base + c_bias_b.unsqueeze(-1)
+            dt_raw = torch.matmul(self.dt_proj.weight, dist_t) + dt_tok_bias.unsqueeze(-1)
         if mask is None:
             out["dt"], out["softplus_in_kernel"] = dt_raw, True
         else:

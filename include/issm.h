@@ -232,6 +232,39 @@ int issm_rmsnorm_bwd_blocks(int64_t rows);
 int issm_gated_rmsnorm_fwd(const issm_norm_args* args);
 int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
 
+/* ---- generation of the scan parameters from the distance encoding -------------------
+ * Replaces the bc_proj / dt_proj Linear layers, their transposes and the broadcast bias
+ * additions of MultiHeadISSMScan.forward (models/dest_module.py:541-553) by one pass:
+ *   base[r][k] = sum_m W[r][m] dist[t][k][m]        r < R0 = H + 2G, rows ordered dt heads, B groups, C groups
+ *   dt[t][h][k] = base[h][k] + bias[t][h]           (pre-softplus; bias = token bias + dt_bias parameter)
+ *   Bm[t][g][k] = base[H+g][k] + bias[t][H+g]       Cm[t][g][k] = base[H+G+g][k] + bias[t][H+G+g]
+ *   Bm_back / Cm_back: the same base rows with bias columns R0+g and R0+G+g (has_back).
+ * t runs over the B*L tokens, M must be 16 and R0 <= 12.  dist, the outputs and their gradients
+ * are contiguous in `dtype`; W (R0, M), bias (tokens, R) with R = R0 + (has_back ? 2G : 0), dbias
+ * (tokens, R) and dW (R0, M) are fp32 contiguous.  dw_partial: issm_param_gen_bwd_blocks(tokens)
+ * * R0 * M floats of scratch.  Absent output gradients may be NULL (treated as zero). */
+typedef struct issm_pgen_args {
+  int64_t tokens;
+  int32_t K, M, H, G;
+  int32_t dtype; /* issm_dtype of dist, dt, Bm, Cm, their gradients and ddist */
+  int32_t has_back;
+  const void* dist;
+  const float* W;
+  const float* bias;
+  void *dt, *Bm, *Cm, *Bm_back, *Cm_back;
+  /* backward */
+  const void *ddt, *dBm, *dCm, *dBm_back, *dCm_back;
+  void* ddist;
+  float* dbias;
+  float* dw_partial;
+  float* dW;
+  void* stream;
+} issm_pgen_args;
+
+int issm_param_gen_bwd_blocks(int64_t tokens);
+int issm_param_gen_fwd(const issm_pgen_args* args);
+int issm_param_gen_bwd(const issm_pgen_args* args);
+
 #ifdef __cplusplus
 }
 #endif
