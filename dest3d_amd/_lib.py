@@ -25,6 +25,7 @@ EXPORTS = [
     "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_stage_bwd_dx", "issm_stage_bwd_reduce",
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
+    "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
 ]
 
 
@@ -90,6 +91,17 @@ class PGenArgs(C.Structure):
     ]
 
 
+class DwConvArgs(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("seqlen", C.c_int32), ("channels", C.c_int32), ("nsets", C.c_int32),
+        ("taps", C.c_int32), ("dtype", C.c_int32),
+        ("u", C.c_void_p), ("u_batch_stride", C.c_int64), ("u_token_stride", C.c_int64),
+        ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("pre", C.c_void_p),
+        ("dy", C.c_void_p * 2), ("du", C.c_void_p), ("partial", C.c_void_p), ("dw", C.c_void_p),
+        ("dbias", C.c_void_p), ("stream", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -122,6 +134,9 @@ def load() -> C.CDLL:
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
+    lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]
+    lib.issm_dwconv_silu_fwd.argtypes = [P(DwConvArgs)]
+    lib.issm_dwconv_silu_bwd.argtypes = [P(DwConvArgs)]
     lib.issm_param_gen_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_param_gen_fwd.argtypes = [P(PGenArgs)]
     lib.issm_param_gen_bwd.argtypes = [P(PGenArgs)]

@@ -25,6 +25,9 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
+int dwconv_partial_rows(int B, int L);
+int launch_dwconv_fwd(const DwConvP& p, hipStream_t st);
+int launch_dwconv_bwd(const DwConvP& p, hipStream_t st);
 int pgen_bwd_blocks(long tokens);
 int launch_pgen_fwd(const PGenP& p, hipStream_t st);
 int launch_pgen_bwd(const PGenP& p, hipStream_t st);
@@ -441,6 +444,45 @@ int issm_param_gen_bwd(const issm_pgen_args* a) {
   if (rc) return rc;
   if (p.tokens == 0) return ISSM_OK;
   return launched(launch_pgen_bwd(p, (hipStream_t)a->stream), "param_gen_bwd");
+}
+
+static int dwconv_params(const issm_dwconv_args* a, DwConvP* p, bool bwd) {
+  if (!a) return fail(ISSM_E_NULL, "dwconv: args is NULL");
+  if (a->batch < 0 || a->seqlen < 0 || a->channels < 1) return fail(ISSM_E_SHAPE, "dwconv: bad shape");
+  if (a->taps != 7) return fail(ISSM_E_UNSUPPORTED, "dwconv: %d taps (only 7 is built)", a->taps);
+  if (a->nsets < 1 || a->nsets > 2) return fail(ISSM_E_UNSUPPORTED, "dwconv: nsets = %d (1 or 2)", a->nsets);
+  if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "dwconv: dtype %d", a->dtype);
+  if (!a->u || !a->w || !a->pre) return fail(ISSM_E_NULL, "dwconv: u/w/pre is NULL");
+  if (a->u_token_stride < a->channels || a->u_batch_stride < 0)
+    return fail(ISSM_E_STRIDE, "dwconv: u strides (%lld, %lld)", (long long)a->u_batch_stride, (long long)a->u_token_stride);
+  if (!bwd && (!a->bias || !a->y)) return fail(ISSM_E_NULL, "dwconv: bias/y is NULL");
+  if (bwd && (!a->partial || !a->dw || !a->dbias)) return fail(ISSM_E_NULL, "dwconv bwd: partial/dw/dbias is NULL");
+  p->B = a->batch; p->L = a->seqlen; p->C = a->channels; p->nsets = a->nsets; p->dtype = a->dtype;
+  p->u = a->u; p->u_bs = a->u_batch_stride; p->u_ls = a->u_token_stride;
+  p->w = a->w; p->bias = a->bias; p->y = a->y; p->pre = a->pre;
+  p->dy[0] = a->dy[0]; p->dy[1] = a->nsets > 1 ? a->dy[1] : nullptr;
+  p->du = a->du; p->partial = a->partial; p->nrows = dwconv_partial_rows(a->batch, a->seqlen);
+  p->dw = a->dw; p->dbias = a->dbias;
+  return ISSM_OK;
+}
+
+int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen) {
+  return (batch > 0 && seqlen > 0) ? dwconv_partial_rows(batch, seqlen) : 0;
+}
+
+int issm_dwconv_silu_fwd(const issm_dwconv_args* a) {
+  DwConvP p;
+  int rc = dwconv_params(a, &p, false);
+  if (rc) return rc;
+  if (p.B == 0 || p.L == 0) return ISSM_OK;
+  return launched(launch_dwconv_fwd(p, (hipStream_t)a->stream), "dwconv_silu_fwd");
+}
+
+int issm_dwconv_silu_bwd(const issm_dwconv_args* a) {
+  DwConvP p;
+  int rc = dwconv_params(a, &p, true);
+  if (rc) return rc;
+  return launched(launch_dwconv_bwd(p, (hipStream_t)a->stream), "dwconv_silu_bwd");
 }
 
 }  // extern "C"

@@ -78,6 +78,23 @@ struct NormP {
   int nblocks;
 };
 
+// parameters of the depthwise conv + SiLU kernels (dwconv_silu.hip)
+struct DwConvP {
+  int B, L, C, nsets, dtype;
+  const void* u;       // (B, L, C) io dtype, element strides u_bs (batch), u_ls (token), channels contiguous
+  long u_bs, u_ls;
+  const float* w;      // (nsets, C, 7) fp32
+  const float* bias;   // (nsets, C) fp32
+  void* y;             // (nsets, B, L, C) io dtype
+  void* pre;           // (nsets, B, L, C) io dtype: convolution output before SiLU (saved for the backward)
+  const void* dy[2];   // (B, L, C) io dtype per set, or NULL
+  void* du;            // (B, L, C) io dtype
+  float* partial;      // (nrows, nsets, 8, C) fp32
+  int nrows;
+  float* dw;           // (nsets, C, 7) fp32
+  float* dbias;        // (nsets, C) fp32
+};
+
 // parameters of the dt / B / C generation kernels (param_gen.hip)
 struct PGenP {
   long tokens;

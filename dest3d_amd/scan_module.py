@@ -23,6 +23,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import param_gen
+from .dwconv import dwconv_silu
 from .issm_combined import ISSM_biscan_combined, ISSM_chunk_scan_combined
 from .layernorm_gated import RMSNorm as RMSNormGated
 
@@ -38,7 +39,7 @@ class PointLiteConv(nn.Module):
         self.act = nn.SiLU()
 
     def forward(self, xyz, feature):
-        return self.act(self.dwconv(feature.transpose(1, 2))).transpose(1, 2)
+        return dwconv_silu(feature, [self.dwconv.weight], [self.dwconv.bias])[0]
 
 
 class MultiHeadISSMScan(nn.Module):
@@ -90,7 +91,12 @@ class MultiHeadISSMScan(nn.Module):
         H, G, P = self.nheads, self.ngroups, self.headdim
         zxbcdt = self.key_proj(in_key)
         z, xbc, dt_tok = torch.split(zxbcdt, [self.d_inner, self.d_inner + 2 * G, H], dim=-1)
-        xbc_f = self.key_conv(key_xyz, xbc)
+        if self.use_biscan:
+            # both convolutions read xbc once (dest_module.py:531,548)
+            convs = (self.key_conv.dwconv, self.key_conv_back.dwconv)
+            xbc_f, xbc_b = dwconv_silu(xbc, [c.weight for c in convs], [c.bias for c in convs])
+        else:
+            xbc_f = self.key_conv(key_xyz, xbc)
         x, b_bias, c_bias = torch.split(xbc_f, [self.d_inner, G, G], dim=-1)
         out = dict(z=z, x=x.contiguous().unflatten(-1, (H, P)))
         # queries become the initial state: one state column per query (dest_module.py:537-538)
@@ -99,7 +105,6 @@ class MultiHeadISSMScan(nn.Module):
         out["A"] = (-torch.exp(self.A_log.float()))[:, None].expand(H, self.d_state)
         dt_tok_bias = dt_tok + self.dt_bias.to(dt_tok.dtype)
         if self.use_biscan:
-            xbc_b = self.key_conv_back(key_xyz, xbc)
             x_b, b_bias_b, c_bias_b = torch.split(xbc_b, [self.d_inner, G, G], dim=-1)
             out["x_back"] = x_b.contiguous().unflatten(-1, (H, P))
         if param_gen.supported(dist, H, G):

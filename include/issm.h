@@ -265,6 +265,39 @@ int issm_param_gen_bwd_blocks(int64_t tokens);
 int issm_param_gen_fwd(const issm_pgen_args* args);
 int issm_param_gen_bwd(const issm_pgen_args* args);
 
+/* ---- depthwise 7-tap convolution along the token order + SiLU -------------------------
+ * PointLiteConv (models/dest_module.py:400-423): nn.Conv1d(C, C, 7, padding=3, groups=C) on
+ * feature.transpose(1, 2), then SiLU, transposed back.  Here on (B, L, C) as it lies, for up to two
+ * weight sets at once (MultiHeadISSMScan applies key_conv and key_conv_back to the same tensor,
+ * dest_module.py:531,548):
+ *   pre[s][b][l][c] = bias[s][c] + sum_j w[s][c][j] u[b][l+j-3][c]   (zero outside [0, L)),  y = silu(pre).
+ * u: `dtype`, channels contiguous, element strides u_batch_stride / u_token_stride.  w (nsets, C, 7) and
+ * bias (nsets, C): fp32 contiguous.  y and pre: (nsets, B, L, C) contiguous in `dtype`; pre is the
+ * convolution output before SiLU, which the backward reads.  Backward: dy[s] (B, L, C) contiguous or NULL
+ * (zero); du (B, L, C) contiguous; dw (nsets, C, 7), dbias (nsets, C) fp32; partial:
+ * issm_dwconv_partial_rows(B, L) * nsets * 8 * C floats of scratch. */
+typedef struct issm_dwconv_args {
+  int32_t batch, seqlen, channels, nsets, taps; /* taps must be 7 */
+  int32_t dtype;
+  const void* u;
+  int64_t u_batch_stride, u_token_stride;
+  const float* w;
+  const float* bias;
+  void* y;
+  void* pre;
+  /* backward */
+  const void* dy[2];
+  void* du;
+  float* partial;
+  float* dw;
+  float* dbias;
+  void* stream;
+} issm_dwconv_args;
+
+int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);
+int issm_dwconv_silu_fwd(const issm_dwconv_args* args);
+int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,88 @@
+"""Depthwise conv7 + SiLU on (B, L, C) (libissm_hip.so) against torch's Conv1d + SiLU in fp64 on the CPU
+(the formulation of models/dest_module.py:400-423).  fp32: rel. error <= 1e-5 forward, 1e-4 gradients;
+bf16: <= 1e-2 / 3e-2 (the convolution output is rounded to bf16 before SiLU, as a bf16 Conv1d module's is)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref(u, ws, bs):
+    C = u.shape[-1]
+    return [F.silu(F.conv1d(u.transpose(1, 2), w.reshape(C, 1, 7), b, padding=3, groups=C)).transpose(1, 2)
+            for w, b in zip(ws, bs)]
+
+
+def _rel(a, b):
+    return ((a.double().cpu() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
+
+
+CASES = [
+    # B, L, C, nsets, dtype, strided input
+    (2, 100, 290, 2, torch.float32, True),
+    (1, 5, 33, 1, torch.float32, False),
+    (3, 16, 64, 2, torch.float32, False),
+    (2, 1, 8, 2, torch.float32, False),
+    (2, 257, 290, 2, torch.bfloat16, True),
+    (1, 40, 130, 1, torch.bfloat16, False),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_L%d_C%d_S%d_%s_%s" % (*c[:4], str(c[4])[6:], "view" if c[5] else "dense"))
+def test_dwconv_silu_matches_fp64(case):
+    from dest3d_amd.dwconv import dwconv_silu
+    B, L, C, S, dtype, strided = case
+    g = torch.Generator().manual_seed(77 + L + C)
+    full = torch.randn(B, L, C + 24, generator=g).to(dtype)
+    base = full.cuda().requires_grad_()
+    u = base[..., 8:8 + C] if strided else base[..., :C].contiguous()
+    ws = [(0.4 * torch.randn(C, 1, 7, generator=g)).cuda().requires_grad_() for _ in range(S)]
+    bs = [(0.2 * torch.randn(C, generator=g)).cuda().requires_grad_() for _ in range(S)]
+    ys = dwconv_silu(u, ws, bs)
+    u64 = (full[..., 8:8 + C] if strided else full[..., :C]).double().requires_grad_()
+    w64 = [w.detach().double().cpu().requires_grad_() for w in ws]
+    b64 = [b.detach().double().cpu().requires_grad_() for b in bs]
+    refs = _ref(u64, w64, b64)
+    ftol, gtol = (1e-5, 1e-4) if dtype == torch.float32 else (1e-2, 3e-2)
+    assert len(ys) == S
+    for y, r in zip(ys, refs):
+        assert y.shape == (B, L, C) and y.dtype == dtype
+        assert _rel(y, r) <= ftol
+    gy = [torch.randn(B, L, C, generator=g).to(dtype) for _ in range(S)]
+    torch.autograd.backward(list(ys), [t.cuda() for t in gy])
+    torch.autograd.backward(refs, [t.double() for t in gy])
+    got_du = base.grad[..., 8:8 + C] if strided else base.grad[..., :C]
+    assert _rel(got_du, u64.grad) <= gtol
+    for s in range(S):
+        assert ws[s].grad.shape == (C, 1, 7)
+        assert _rel(ws[s].grad, w64[s].grad) <= gtol
+        assert _rel(bs[s].grad, b64[s].grad) <= gtol
+
+
+def test_dwconv_one_absent_gradient():
+    from dest3d_amd.dwconv import dwconv_silu
+    g = torch.Generator().manual_seed(5)
+    u = torch.randn(2, 50, 40, generator=g).cuda().requires_grad_()
+    ws = [torch.randn(40, 7, generator=g).cuda().requires_grad_() for _ in range(2)]
+    bs = [torch.randn(40, generator=g).cuda().requires_grad_() for _ in range(2)]
+    y0, y1 = dwconv_silu(u, ws, bs)
+    y0.sum().backward()
+    assert ws[1].grad.abs().max().item() == 0.0 and bs[1].grad.abs().max().item() == 0.0
+    u64 = u.detach().double().cpu().requires_grad_()
+    r = _ref(u64, [ws[0].detach().double().cpu()], [bs[0].detach().double().cpu()])[0]
+    r.sum().backward()
+    assert _rel(u.grad, u64.grad) <= 1e-4
+
+
+def test_dwconv_rejects_unbuilt_shapes():
+    import ctypes as C
+    from dest3d_amd import _lib as L
+    lib = L.load()
+    a = L.DwConvArgs()
+    a.batch, a.seqlen, a.channels, a.nsets, a.taps = 1, 8, 8, 1, 5
+    assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -5
+    a.taps, a.nsets = 7, 3
+    assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -5
+    a.nsets = 1
+    assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -1
