@@ -222,6 +222,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
+    ap.add_argument("--only-layer", action="store_true",
+                    help="time only the whole detector layer (module forward + backward) and print its JSON line")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
     ap.add_argument("--traffic", type=float, default=None,
@@ -235,6 +237,10 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    if args.only_layer:
+        print(json.dumps({"detector_layer_bf16_fwd_bwd_us": round(time_module_layer(torch, args.steps, args.warmup), 2),
+                          "steps": args.steps, "warmup": args.warmup}))
+        return
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
