@@ -192,17 +192,19 @@ def cpu_baseline(torch):
 
 def time_module_layer(torch, steps=10, warmup=3):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
-    keys, batch 8, d_dist 16, bf16), forward + backward through autograd, microseconds.  Includes the PyTorch
-    projections, conv and norms around the scan."""
+    keys, batch 8, d_dist 16, bf16, float locality weights as mask -- what DEST's decoder layer passes,
+    models/dest_module.py:283-290), forward + backward through autograd, microseconds.  Includes the PyTorch
+    projections and norms around the scan."""
     from dest3d_amd.scan_module import MultiHeadISSMScan
     torch.manual_seed(0)
     m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1).cuda().bfloat16()
     key = torch.randn(8, 1024, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
     query = torch.randn(8, 256, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
     dist = (0.5 * torch.randn(8, 1024, 256, 16, device="cuda")).bfloat16().requires_grad_()
+    weights = torch.exp(-15.0 * (torch.rand(8, 1024, 256, device="cuda") - 0.5).clamp_min(0.0))
 
     def step():
-        ok, oq = m(key, query, dist, None)
+        ok, oq = m(key, query, dist, None, weights)
         (ok.float().square().mean() + oq.float().square().mean()).backward()
 
     for _ in range(warmup):

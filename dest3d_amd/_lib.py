@@ -84,9 +84,11 @@ class PGenArgs(C.Structure):
         ("dtype", C.c_int32), ("has_back", C.c_int32),
         ("dist", C.c_void_p), ("W", C.c_void_p), ("bias", C.c_void_p),
         ("dt", C.c_void_p), ("Bm", C.c_void_p), ("Cm", C.c_void_p), ("Bm_back", C.c_void_p), ("Cm_back", C.c_void_p),
+        ("weights", C.c_void_p), ("dt_raw", C.c_void_p),
         ("ddt", C.c_void_p), ("dBm", C.c_void_p), ("dCm", C.c_void_p), ("dBm_back", C.c_void_p),
         ("dCm_back", C.c_void_p),
-        ("ddist", C.c_void_p), ("dbias", C.c_void_p), ("dw_partial", C.c_void_p), ("dW", C.c_void_p),
+        ("ddist", C.c_void_p), ("dbias", C.c_void_p), ("dweights", C.c_void_p),
+        ("dw_partial", C.c_void_p), ("dW", C.c_void_p),
         ("stream", C.c_void_p),
     ]
 

@@ -413,6 +413,7 @@ static int pgen_params(const issm_pgen_args* a, PGenP* p, bool bwd) {
   if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "param_gen: dtype %d", a->dtype);
   if (a->tokens * (int64_t)a->K * 16 >= ((int64_t)1 << 40)) return fail(ISSM_E_SHAPE, "param_gen: too large");
   if (!a->dist || !a->W) return fail(ISSM_E_NULL, "param_gen: dist/W is NULL");
+  if (a->weights && !a->dt_raw) return fail(ISSM_E_NULL, "param_gen: weights given but dt_raw is NULL");
   if (!bwd) {
     if (!a->bias || !a->dt || !a->Bm || !a->Cm) return fail(ISSM_E_NULL, "param_gen: bias/dt/Bm/Cm is NULL");
     if (a->has_back && (!a->Bm_back || !a->Cm_back)) return fail(ISSM_E_NULL, "param_gen: Bm_back/Cm_back is NULL");
@@ -423,6 +424,7 @@ static int pgen_params(const issm_pgen_args* a, PGenP* p, bool bwd) {
   p->dist = a->dist; p->W = a->W; p->bias = a->bias;
   p->dt = a->dt; p->Bm = a->Bm; p->Cm = a->Cm; p->Bb = a->Bm_back; p->Cb = a->Cm_back;
   p->ddt = a->ddt; p->dB = a->dBm; p->dC = a->dCm; p->dBb = a->dBm_back; p->dCb = a->dCm_back;
+  p->weights = a->weights; p->dt_raw = a->dt_raw; p->dweights = a->weights ? a->dweights : nullptr;
   p->ddist = a->ddist; p->dbias = a->dbias; p->dw_partial = a->dw_partial; p->dW = a->dW;
   p->nblocks = pgen_bwd_blocks(a->tokens);
   return ISSM_OK;

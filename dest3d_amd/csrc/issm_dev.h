@@ -103,6 +103,9 @@ struct PGenP {
   const float* W;        // (R0, M) fp32
   const float* bias;     // (tokens, R) fp32, R = R0 + (has_back ? 2G : 0)
   void *dt, *Bm, *Cm, *Bb, *Cb;                    // (tokens, H|G, K) io dtype
+  const float* weights;  // (tokens, K) fp32 or NULL: dt = softplus(raw) * weights instead of raw
+  void* dt_raw;          // (tokens, H, K) io dtype: raw dt, written by the forward when weights is given
+  float* dweights;       // (tokens, K) fp32 or NULL
   const void *ddt, *dB, *dC, *dBb, *dCb;           // gradients of the outputs
   void* ddist;           // (tokens, K, M) io dtype
   float* dbias;          // (tokens, R) fp32

@@ -14,7 +14,6 @@ namespace issm {
 
 constexpr int PG_MAXR0 = 12;  // largest H + 2G built (three 4-row steps of the matrix instruction)
 constexpr int PG_M = 16;      // distance encoding width this kernel is built for
-constexpr int PG_UNR = 4;     // blocks of 16 k whose loads are in flight together in the backward
 constexpr int PG_TOK = 4;     // tokens per workgroup in the backward (one per wave)
 
 template <bool BF>
@@ -86,7 +85,13 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_fwd(PGenP p) {
 #pragma unroll
     for (int m = 0; m < PG_M; ++m) s = fmaf(w[m], d[m], s);
     if (r < p.H) {
-      st1<BF>(p.dt, (t * p.H + r) * p.K + k, s + bias[r]);
+      float v = s + bias[r];
+      if (p.weights) {  // uniform: dt = softplus(raw) * weight, raw kept for the backward
+        if (BF) v = bf16_to_f(f_to_bf16(v));  // the saved value is what the backward differentiates
+        st1<BF>(p.dt_raw, (t * p.H + r) * p.K + k, v);
+        v = softplus_(v) * p.weights[t * p.K + k];
+      }
+      st1<BF>(p.dt, (t * p.H + r) * p.K + k, v);
     } else if (r < p.H + p.G) {
       const int g = r - p.H;
       st1<BF>(p.Bm, (t * p.G + g) * p.K + k, s + bias[r]);
@@ -149,6 +154,9 @@ __device__ __forceinline__ f4 load4(const void* p, long off, int k, int kend, bo
   return r;
 }
 
+// d softplus(x) / dx with torch's threshold: 1 above 20
+__device__ __forceinline__ float dsoftplus_(float x) { return x <= 20.0f ? sigmoidf_(x) : 1.0f; }
+
 // Backward on the matrix cores (v_mfma_f32_16x16x4_f32; lane = (i = lane & 15, q = lane >> 4)).
 // Workgroup = PG_TOK consecutive tokens, a wave owns PG_TOK / 4 of them and walks k in blocks of 16:
 //   ddist^T (m x k) = W^T (m x r) g (r x k)   -- A: lane (m, q) = W[4s + q][m], B: lane (k, q) = g[4s + q][k0 + k];
@@ -157,11 +165,15 @@ __device__ __forceinline__ f4 load4(const void* p, long off, int k, int kend, bo
 //                                                v = 0..3 (the order of k inside the sum is free)
 //   dbias[r]        = sum_k g[r][k]           -- from the second layout, reduced over q at the end of the token.
 // g of a B / C row is the sum of its forward-order and reversed-order gradients wherever the shared base row is
-// differentiated; the two bias gradients stay apart.
-// FULLK: K is a multiple of 16 * PG_UNR, so no load or store needs a bound on k, and every per-lane address is a
-// pointer advanced once per trip plus a compile-time offset.
-template <bool BF, bool FULLK>
+// differentiated; the two bias gradients stay apart.  HASW (dt = softplus(raw) * weight): g of a dt row is
+// ddt * weight * softplus'(raw), and dweight[k] = sum_h ddt[h][k] softplus(raw[h][k]).
+// FULLK: K is a multiple of 64, so no load or store needs a bound on k, and every per-lane address is a
+// pointer advanced once per trip plus a compile-time offset.  UNR blocks of 16 k have their loads in flight together.
+template <bool BF, bool FULLK, bool HASW>
 __global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
+  constexpr int UNR = HASW ? 2 : 4;
+  typedef typename std::conditional<BF, uint16_t, float>::type T;
+  typedef typename std::conditional<BF, uint2, f4>::type T4;
   __shared__ float wred[4][16 * PG_M];
   const int R0 = p.H + 2 * p.G, R = R0 + (p.has_back ? 2 * p.G : 0);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -175,14 +187,83 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
   // row-of-the-lane pointers: layout 2 (row i), layout 1 (rows 4s + q)
   const void* g2 = gr.base(i, false);
   const void* g2b = gr.base(i, true);
+  const bool isdt2 = HASW && i < p.H && g2 != nullptr;
   const void *g1[3], *g1b[3];
+  bool okg[3], okgb[3], isdt1[3];
 #pragma unroll
   for (int s = 0; s < 3; ++s) {
     g1[s] = gr.base(4 * s + q, false);
     g1b[s] = gr.base(4 * s + q, true);
+    okg[s] = g1[s] != nullptr;
+    okgb[s] = g1b[s] != nullptr;
+    isdt1[s] = HASW && 4 * s + q < p.H && okg[s];
   }
+  const bool ok2 = g2 != nullptr, ok2b = g2b != nullptr;
   const bool any_back = gr.dBb != nullptr || gr.dCb != nullptr;  // uniform
-  f4 accW = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+  auto widen = [](T4 w) -> f4 {
+    if constexpr (BF) {
+      return (f4){__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                  __uint_as_float(w.y & 0xffff0000u)};
+    } else {
+      return w;
+    }
+  };
+  auto widen1 = [](T w) -> float {
+    if constexpr (BF) return __uint_as_float((unsigned)w << 16);
+    else return w;
+  };
+  // one block of 16 k, operands already in registers (a / ab / rw2 / ww2: layout 2; x*, raw1, w1: layout 1)
+  f4 accW = zero4;
+  float bs = 0.0f, bsb = 0.0f;
+  auto block = [&](f4 a, f4 ab, f4 rw2, f4 ww2, const float (&dv)[4], const float (&x)[3], const float (&xb)[3],
+                   const float (&raw1)[3], float w1, T* ddst, float* dwdst, bool in_k) {
+    if constexpr (HASW) {
+      if (isdt2) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) a[v] *= ww2[v] * dsoftplus_(rw2[v]);
+      }
+    }
+    bs += (a.x + a.y) + (a.z + a.w);
+    bsb += (ab.x + ab.y) + (ab.z + ab.w);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) accW = mfma4(a[v] + ab[v], dv[v], accW);
+    float gx[3], dws = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      gx[s] = x[s];
+      if constexpr (HASW) {
+        if (isdt1[s]) {
+          dws += x[s] * softplus_(raw1[s]);
+          gx[s] = x[s] * w1 * dsoftplus_(raw1[s]);
+        }
+      }
+      gx[s] += xb[s];
+    }
+    if constexpr (HASW) {
+      if (dwdst != nullptr) {  // uniform
+        dws += __shfl_xor(dws, 16, 64);
+        dws += __shfl_xor(dws, 32, 64);
+        if (q == 0 && in_k) *dwdst = dws;
+      }
+    }
+    if (ddst != nullptr) {  // uniform
+      f4 dd = zero4;
+#pragma unroll
+      for (int s = 0; s < 3; ++s) dd = mfma4(wA[s], gx[s], dd);
+      if (in_k) {
+        if constexpr (BF) {
+          uint2 w;
+          w.x = pack_bf16(dd.x, dd.y);
+          w.y = pack_bf16(dd.z, dd.w);
+          *(uint2*)ddst = w;
+        } else {
+          *(f4*)ddst = dd;
+        }
+      }
+    }
+  };
+
   constexpr int TPW = PG_TOK / 4;
   for (int ti = 0; ti < TPW; ++ti) {
     const long t = (long)blockIdx.x * PG_TOK + wave * TPW + ti;
@@ -191,43 +272,35 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
     long o1[3];
 #pragma unroll
     for (int s = 0; s < 3; ++s) o1[s] = (4 * s + q < R0) ? gr.offset(t, 4 * s + q) : 0;
-    float bs = 0.0f, bsb = 0.0f;
+    bs = 0.0f;
+    bsb = 0.0f;
     if constexpr (FULLK) {
-      typedef typename std::conditional<BF, uint16_t, float>::type T;
-      typedef typename std::conditional<BF, uint2, f4>::type T4;
       const T* nil = (const T*)p.dist;  // what a lane with no row reads (at least 64 * 16 elements long)
-      const bool ok2 = g2 != nullptr, ok2b = g2b != nullptr;
       const T* pa = ok2 ? (const T*)g2 + o2 + 4 * q : nil;
       const T* pab = ok2b ? (const T*)g2b + o2 + 4 * q : nil;
       const T* pd = (const T*)p.dist + (t * K + 4 * q) * PG_M + i;
       const T *pg[3], *pgb[3];
-      bool okg[3], okgb[3];
 #pragma unroll
       for (int s = 0; s < 3; ++s) {
-        okg[s] = g1[s] != nullptr;
-        okgb[s] = g1b[s] != nullptr;
         pg[s] = okg[s] ? (const T*)g1[s] + o1[s] + i : nil;
         pgb[s] = okgb[s] ? (const T*)g1b[s] + o1[s] + i : nil;
       }
-      T* pdd = (T*)p.ddist + (t * K + i) * PG_M + 4 * q;
-      auto widen = [](T4 w) -> f4 {
-        if constexpr (BF) {
-          return (f4){__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
-                      __uint_as_float(w.y & 0xffff0000u)};
-        } else {
-          return w;
-        }
-      };
-      auto widen1 = [](T w) -> float {
-        if constexpr (BF) return __uint_as_float((unsigned)w << 16);
-        else return w;
-      };
-      const f4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-      for (int kb = 0; kb < K; kb += 16 * PG_UNR) {
-        T4 ra[PG_UNR], rab[PG_UNR];
-        T rd[PG_UNR][4], rg[PG_UNR][3], rgb[PG_UNR][3];
+      // HASW: raw in both layouts, weights in both layouts
+      const T* pr2 = isdt2 ? (const T*)p.dt_raw + o2 + 4 * q : nil;
+      const T* pr1[3];
 #pragma unroll
-        for (int u = 0; u < PG_UNR; ++u) {
+      for (int s = 0; s < 3; ++s) pr1[s] = isdt1[s] ? (const T*)p.dt_raw + o1[s] + i : nil;
+      const float* pw2 = HASW ? p.weights + t * K + 4 * q : nullptr;
+      const float* pw1 = HASW ? p.weights + t * K + i : nullptr;
+      T* pdd = p.ddist ? (T*)p.ddist + (t * K + i) * PG_M + 4 * q : nullptr;
+      float* pdw = (HASW && p.dweights) ? p.dweights + t * K + i : nullptr;
+      for (int kb = 0; kb < K; kb += 16 * UNR) {
+        T4 ra[UNR], rab[UNR], rr2[UNR];
+        f4 rw2[UNR];
+        T rd[UNR][4], rg[UNR][3], rgb[UNR][3], rr1[UNR][3];
+        float rw1[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
           ra[u] = *(const T4*)(pa + 16 * u);
           if (any_back) rab[u] = *(const T4*)(pab + 16 * u);
 #pragma unroll
@@ -236,90 +309,73 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
           for (int s = 0; s < 3; ++s) {
             rg[u][s] = pg[s][16 * u];
             if (any_back) rgb[u][s] = pgb[s][16 * u];
+            if constexpr (HASW) rr1[u][s] = pr1[s][16 * u];
+          }
+          if constexpr (HASW) {
+            rr2[u] = *(const T4*)(pr2 + 16 * u);
+            rw2[u] = *(const f4*)(pw2 + 16 * u);
+            rw1[u] = pw1[16 * u];
           }
         }
 #pragma unroll
-        for (int u = 0; u < PG_UNR; ++u) {
-          // rows past R0 hold finite or non-finite junk in `a`: they only reach rows of dW that are never read
-          const f4 a = widen(ra[u]);
-          const f4 ab = (any_back && ok2b) ? widen(rab[u]) : zero4;
-          bs += (a.x + a.y) + (a.z + a.w);
-          bsb += (ab.x + ab.y) + (ab.z + ab.w);
+        for (int u = 0; u < UNR; ++u) {
+          // rows past R0 hold junk in `a`: they only reach rows of dW that are never read
+          float dv[4], x[3], xb[3], raw1[3];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) accW = mfma4(a[v] + ab[v], widen1(rd[u][v]), accW);
-          if (p.ddist) {
-            f4 dd = zero4;
+          for (int v = 0; v < 4; ++v) dv[v] = widen1(rd[u][v]);
 #pragma unroll
-            for (int s = 0; s < 3; ++s) {
-              float x = okg[s] ? widen1(rg[u][s]) : 0.0f;
-              if (any_back) x += okgb[s] ? widen1(rgb[u][s]) : 0.0f;
-              dd = mfma4(wA[s], x, dd);
-            }
-            if constexpr (BF) {
-              uint2 w;
-              w.x = pack_bf16(dd.x, dd.y);
-              w.y = pack_bf16(dd.z, dd.w);
-              *(uint2*)(pdd + 16 * u * PG_M) = w;
-            } else {
-              *(f4*)(pdd + 16 * u * PG_M) = dd;
-            }
+          for (int s = 0; s < 3; ++s) {
+            x[s] = okg[s] ? widen1(rg[u][s]) : 0.0f;
+            xb[s] = (any_back && okgb[s]) ? widen1(rgb[u][s]) : 0.0f;
+            raw1[s] = HASW ? widen1(rr1[u][s]) : 0.0f;
           }
+          block(widen(ra[u]), (any_back && ok2b) ? widen(rab[u]) : zero4, HASW ? widen(rr2[u]) : zero4,
+                HASW ? rw2[u] : zero4, dv, x, xb, raw1, HASW ? rw1[u] : 0.0f,
+                pdd ? pdd + 16 * u * PG_M : nullptr, pdw ? pdw + 16 * u : nullptr, true);
         }
-        const int step = 16 * PG_UNR;
+        const int step = 16 * UNR;
         pa += ok2 ? step : 0;
         pab += ok2b ? step : 0;
         pd += step * PG_M;
-        pdd += step * PG_M;
+        if (pdd) pdd += step * PG_M;
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
           pg[s] += okg[s] ? step : 0;
           pgb[s] += okgb[s] ? step : 0;
+          if constexpr (HASW) pr1[s] += isdt1[s] ? step : 0;
+        }
+        if constexpr (HASW) {
+          pr2 += isdt2 ? step : 0;
+          pw2 += step;
+          pw1 += step;
+          if (pdw) pdw += step;
         }
       }
     } else {
-      // PG_UNR blocks of 16 k per trip: every load of the trip is issued before the first product needs one
-      for (int kb = 0; kb < K; kb += 16 * PG_UNR) {
-        f4 a[PG_UNR], ab[PG_UNR];
-        float dv[PG_UNR][4], gk[PG_UNR][3], gkb[PG_UNR][3];
-  #pragma unroll
-        for (int u = 0; u < PG_UNR; ++u) {
-          const int k0 = kb + 16 * u, kq = k0 + 4 * q;
-          a[u] = load4<BF>(g2, o2 + kq, kq, K, vec, p.W);
-          ab[u] = any_back ? load4<BF>(g2b, o2 + kq, kq, K, vec, p.W) : (f4){0.0f, 0.0f, 0.0f, 0.0f};
-  #pragma unroll
-          for (int v = 0; v < 4; ++v) dv[u][v] = ld1_or0<BF>(p.dist, (t * K + kq + v) * PG_M + i, kq + v < K, p.W);
-  #pragma unroll
-          for (int s = 0; s < 3; ++s) {
-            const bool in = k0 + i < K;
-            gk[u][s] = ld1_or0<BF>(g1[s], o1[s] + k0 + i, in && g1[s] != nullptr, p.W);
-            if (any_back) gkb[u][s] = ld1_or0<BF>(g1b[s], o1[s] + k0 + i, in && g1b[s] != nullptr, p.W);
-            else gkb[u][s] = 0.0f;
-          }
+      const void* safe = p.W;
+      for (int k0 = 0; k0 < K; k0 += 16) {
+        const int kq = k0 + 4 * q;
+        const bool in = k0 + i < K;
+        const f4 a = load4<BF>(g2, o2 + kq, kq, K, vec, safe);
+        const f4 ab = any_back ? load4<BF>(g2b, o2 + kq, kq, K, vec, safe) : zero4;
+        f4 rw2 = zero4, ww2 = zero4;
+        float dv[4], x[3], xb[3], raw1[3], w1 = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dv[v] = ld1_or0<BF>(p.dist, (t * K + kq + v) * PG_M + i, kq + v < K, safe);
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+          x[s] = ld1_or0<BF>(g1[s], o1[s] + k0 + i, in && okg[s], safe);
+          xb[s] = any_back ? ld1_or0<BF>(g1b[s], o1[s] + k0 + i, in && okgb[s], safe) : 0.0f;
+          raw1[s] = HASW ? ld1_or0<BF>(p.dt_raw, o1[s] + k0 + i, in && isdt1[s], safe) : 0.0f;
         }
-  #pragma unroll
-        for (int u = 0; u < PG_UNR; ++u) {
-          const int k0 = kb + 16 * u;
-          bs += (a[u].x + a[u].y) + (a[u].z + a[u].w);
-          bsb += (ab[u].x + ab[u].y) + (ab[u].z + ab[u].w);
-  #pragma unroll
-          for (int v = 0; v < 4; ++v) accW = mfma4(a[u][v] + ab[u][v], dv[u][v], accW);
-          if (p.ddist) {
-            f4 dd = {0.0f, 0.0f, 0.0f, 0.0f};
-  #pragma unroll
-            for (int s = 0; s < 3; ++s) dd = mfma4(wA[s], gk[u][s] + gkb[u][s], dd);
-            if (k0 + i < K) {
-              const long o = (t * K + k0 + i) * PG_M + 4 * q;
-              if (BF) {
-                uint2 w;
-                w.x = (unsigned)f_to_bf16(dd.x) | ((unsigned)f_to_bf16(dd.y) << 16);
-                w.y = (unsigned)f_to_bf16(dd.z) | ((unsigned)f_to_bf16(dd.w) << 16);
-                *(uint2*)((uint16_t*)p.ddist + o) = w;
-              } else {
-                *(f4*)((float*)p.ddist + o) = dd;
-              }
-            }
-          }
+        if constexpr (HASW) {
+          rw2 = load4<BF>(isdt2 ? p.dt_raw : nullptr, o2 + kq, kq, K, vec, safe);
+          ww2 = load4<false>(p.weights, t * K + kq, kq, K, vec, safe);
+          w1 = ld1_or0<false>(p.weights, t * K + k0 + i, in, safe);
         }
+        block(a, ab, rw2, ww2, dv, x, xb, raw1, w1,
+              p.ddist ? (T*)p.ddist + (t * K + k0 + i) * PG_M + 4 * q : nullptr,
+              (HASW && p.dweights) ? p.dweights + t * K + k0 + i : nullptr, in);
       }
     }
     bs += __shfl_xor(bs, 16, 64);
@@ -371,16 +427,21 @@ int launch_pgen_fwd(const PGenP& p, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+template <bool BF, bool HASW>
+static void pgen_bwd_launch(const PGenP& p, hipStream_t st) {
+  const dim3 g((unsigned)p.nblocks), b(NTHREADS);
+  if (p.K % 64 == 0) hipLaunchKernelGGL((k_pgen_bwd<BF, true, HASW>), g, b, 0, st, p);
+  else hipLaunchKernelGGL((k_pgen_bwd<BF, false, HASW>), g, b, 0, st, p);
+}
+
 int launch_pgen_bwd(const PGenP& p, hipStream_t st) {
   const int R0 = p.H + 2 * p.G;
-  const unsigned blocks = (unsigned)p.nblocks;
-  const bool fullk = p.K % (16 * PG_UNR) == 0;
   if (p.dtype) {
-    if (fullk) hipLaunchKernelGGL((k_pgen_bwd<true, true>), dim3(blocks), dim3(NTHREADS), 0, st, p);
-    else hipLaunchKernelGGL((k_pgen_bwd<true, false>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    if (p.weights) pgen_bwd_launch<true, true>(p, st);
+    else pgen_bwd_launch<true, false>(p, st);
   } else {
-    if (fullk) hipLaunchKernelGGL((k_pgen_bwd<false, true>), dim3(blocks), dim3(NTHREADS), 0, st, p);
-    else hipLaunchKernelGGL((k_pgen_bwd<false, false>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    if (p.weights) pgen_bwd_launch<false, true>(p, st);
+    else pgen_bwd_launch<false, false>(p, st);
   }
   int e = (int)hipGetLastError();
   if (e) return e;

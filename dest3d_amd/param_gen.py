@@ -35,7 +35,7 @@ def _args(dist, W, H, G, has_back) -> L.PGenArgs:
 
 class ScanParamsFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, dist, W, bias, nheads, ngroups, has_back):
+    def forward(ctx, dist, W, bias, weights, nheads, ngroups, has_back):
         L.require_gpu(dist, "dist")
         lib = L.load()
         H, G = nheads, ngroups
@@ -46,6 +46,10 @@ class ScanParamsFn(torch.autograd.Function):
         d = dist.detach().contiguous()
         w = W.detach().float().contiguous()
         b = bias.detach().float().contiguous()
+        wt = None
+        if weights is not None:
+            assert weights.shape == (Bsz, Ln, K)
+            wt = weights.detach().float().contiguous()
         with torch.cuda.device(d.device):
             dt = torch.empty((Bsz, Ln, H, K), dtype=d.dtype, device=d.device)
             outs = [torch.empty((Bsz, Ln, G, K), dtype=d.dtype, device=d.device) for _ in range(4 if has_back else 2)]
@@ -54,19 +58,23 @@ class ScanParamsFn(torch.autograd.Function):
             a.dt, a.Bm, a.Cm = dt.data_ptr(), outs[0].data_ptr(), outs[1].data_ptr()
             if has_back:
                 a.Bm_back, a.Cm_back = outs[2].data_ptr(), outs[3].data_ptr()
+            raw = None
+            if wt is not None:
+                raw = torch.empty_like(dt)
+                a.weights, a.dt_raw = wt.data_ptr(), raw.data_ptr()
             L.check(lib.issm_param_gen_fwd(C.byref(a)), "issm_param_gen_fwd")
-        ctx.save_for_backward(d, w)
-        ctx.meta = (H, G, has_back, W.dtype, bias.dtype, R)
+        ctx.save_for_backward(d, w, wt, raw)
+        ctx.meta = (H, G, has_back, W.dtype, bias.dtype, R, None if weights is None else weights.dtype)
         return (dt, *outs)
 
     @staticmethod
     def backward(ctx, *grads):
         lib = L.load()
-        d, w = ctx.saved_tensors
-        H, G, has_back, wdt, bdt, R = ctx.meta
+        d, w, wt, raw = ctx.saved_tensors
+        H, G, has_back, wdt, bdt, R, wtdt = ctx.meta
         Bsz, Ln, K, M = d.shape
         g = [None if t is None else t.to(d.dtype).contiguous() for t in grads]
-        need_dist, need_w, need_bias = ctx.needs_input_grad[:3]
+        need_dist, need_w, need_bias, need_wt = ctx.needs_input_grad[:4]
         with torch.cuda.device(d.device):
             a = _args(d, w, H, G, has_back)
             names = ("ddt", "dBm", "dCm", "dBm_back", "dCm_back")
@@ -83,12 +91,21 @@ class ScanParamsFn(torch.autograd.Function):
             if dbias is not None:
                 a.dbias = dbias.data_ptr()
             a.dw_partial, a.dW = dwp.data_ptr(), dW.data_ptr()
+            dwt = None
+            if wt is not None:
+                a.weights, a.dt_raw = wt.data_ptr(), raw.data_ptr()
+                if need_wt:
+                    dwt = torch.zeros((Bsz, Ln, K), dtype=torch.float32, device=d.device)
+                    a.dweights = dwt.data_ptr()
             L.check(lib.issm_param_gen_bwd(C.byref(a)), "issm_param_gen_bwd")
-        return (ddist, dW.to(wdt) if need_w else None, None if dbias is None else dbias.to(bdt), None, None, None)
+        return (ddist, dW.to(wdt) if need_w else None, None if dbias is None else dbias.to(bdt),
+                None if dwt is None else dwt.to(wtdt), None, None, None)
 
 
-def scan_params(dist, W, bias, nheads: int, ngroups: int, has_back: bool = False):
+def scan_params(dist, W, bias, nheads: int, ngroups: int, has_back: bool = False, weights=None):
     """dist (B, L, K, M=16); W (H+2G, M): rows dt heads, B groups, C groups; bias (B, L, R) with columns
-    [dt heads | B | C | B_back | C_back] (the last two when ``has_back``).  Returns dt (B,L,H,K) -- before
-    softplus -- B, C (B,L,G,K) and, with ``has_back``, B_back, C_back."""
-    return ScanParamsFn.apply(dist, W, bias, nheads, ngroups, has_back)
+    [dt heads | B | C | B_back | C_back] (the last two when ``has_back``).  Returns dt (B,L,H,K), B, C
+    (B,L,G,K) and, with ``has_back``, B_back, C_back.  Without ``weights`` dt is the raw sum (before
+    softplus); with ``weights`` (B, L, K) -- the locality weight, or a 0/1 keep mask --
+    dt = softplus(raw) * weights (dest_module.py:553-559)."""
+    return ScanParamsFn.apply(dist, W, bias, weights, nheads, ngroups, has_back)

@@ -111,10 +111,17 @@ class MultiHeadISSMScan(nn.Module):
             # one pass over dist writes every (B,L,H|G,K) operand (dest_module.py:541-553)
             W = torch.cat([self.dt_proj.weight, self.bc_proj.weight], dim=0)
             cols = [dt_tok_bias, b_bias, c_bias] + ([b_bias_b, c_bias_b] if self.use_biscan else [])
-            res = param_gen.scan_params(dist, W, torch.cat(cols, dim=-1).float(), H, G, self.use_biscan)
+            # a float mask weighs dt, a bool mask drops entries (dest_module.py:555-559): both are a factor on softplus(raw)
+            wts = None
+            if mask is not None:
+                wts = mask.float() if mask.is_floating_point() else (~mask).float()
+            res = param_gen.scan_params(dist, W, torch.cat(cols, dim=-1).float(), H, G, self.use_biscan, wts)
             dt_raw, out["B"], out["C"] = res[:3]
             if self.use_biscan:
                 out["B_back"], out["C_back"] = res[3:]
+            if mask is not None:
+                out["dt"], out["softplus_in_kernel"] = dt_raw, False
+                return out
         else:
             # W (G|H, M) @ dist^T (B,L,M,K): the product is written straight into (B,L,G|H,K), K contiguous
             dist_t = dist.transpose(-1, -2)

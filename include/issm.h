@@ -242,7 +242,12 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
  * t runs over the B*L tokens, M must be 16 and R0 <= 12.  dist, the outputs and their gradients
  * are contiguous in `dtype`; W (R0, M), bias (tokens, R) with R = R0 + (has_back ? 2G : 0), dbias
  * (tokens, R) and dW (R0, M) are fp32 contiguous.  dw_partial: issm_param_gen_bwd_blocks(tokens)
- * * R0 * M floats of scratch.  Absent output gradients may be NULL (treated as zero). */
+ * * R0 * M floats of scratch.  Absent output gradients may be NULL (treated as zero).
+ * weights (tokens, K) fp32, optional -- the per-(token, query) locality weight or 0/1 keep mask that
+ * MultiHeadISSMScan multiplies into dt (dest_module.py:553-559): when given, dt = softplus(raw) * weights
+ * (softplus with torch's threshold 20), the raw values go to dt_raw (tokens, H, K, `dtype`; required then, and
+ * read back by the backward), and dweights (tokens, K) fp32, if not NULL, receives
+ * sum_h ddt[t][h][k] * softplus(raw[t][h][k]). */
 typedef struct issm_pgen_args {
   int64_t tokens;
   int32_t K, M, H, G;
@@ -252,10 +257,13 @@ typedef struct issm_pgen_args {
   const float* W;
   const float* bias;
   void *dt, *Bm, *Cm, *Bm_back, *Cm_back;
+  const float* weights;
+  void* dt_raw;
   /* backward */
   const void *ddt, *dBm, *dCm, *dBm_back, *dCm_back;
   void* ddist;
   float* dbias;
+  float* dweights;
   float* dw_partial;
   float* dW;
   void* stream;
