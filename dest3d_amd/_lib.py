@@ -26,6 +26,7 @@ EXPORTS = [
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
+    "issm_box_dist_workgroups", "issm_box_dist_fwd", "issm_box_dist_bwd",
 ]
 
 
@@ -104,6 +105,18 @@ class DwConvArgs(C.Structure):
     ]
 
 
+class BoxDistArgs(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("seqlen", C.c_int32), ("nquery", C.c_int32),
+        ("D", C.c_int32), ("H", C.c_int32), ("W", C.c_int32), ("dtype", C.c_int32),
+        ("key", C.c_void_p), ("corners", C.c_void_p), ("angle", C.c_void_p), ("table", C.c_void_p),
+        ("log_scale", C.c_float), ("max_value", C.c_float),
+        ("dist", C.c_void_p), ("qcenter", C.c_void_p), ("radius", C.c_void_p),
+        ("weight_dist", C.c_float), ("weights", C.c_void_p),
+        ("ddist", C.c_void_p), ("partial", C.c_void_p), ("dtable", C.c_void_p), ("stream", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -136,6 +149,9 @@ def load() -> C.CDLL:
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
+    lib.issm_box_dist_workgroups.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    lib.issm_box_dist_fwd.argtypes = [P(BoxDistArgs)]
+    lib.issm_box_dist_bwd.argtypes = [P(BoxDistArgs)]
     lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]
     lib.issm_dwconv_silu_fwd.argtypes = [P(DwConvArgs)]
     lib.issm_dwconv_silu_bwd.argtypes = [P(DwConvArgs)]

@@ -1,0 +1,273 @@
+// Box-to-point distance encoding and locality weight: the two (B, L, K) fields DEST computes right before the scan
+// (gfx950).
+//
+// BoxDistFun.forward (models/dest_module.py:174-195): for every (key point l, query box k) and each of the box's 8
+// corners, delta = corner - key, rotated in the x-y plane by the query angle, compressed by a signed log
+// (sign(v) log2(|v| s + 1) / log2 8 / max_value), and used as the sampling position of a trilinear grid_sample
+// (padding zeros, align_corners False) into a small learned table (C = 16 channels over D x H x W = 10^3 nodes); the
+// 8 samples are summed into dist[b][l][k][0..15].  local_weight (dest_module.py:240-249):
+// w[b][l][k] = exp(weight_dist * min(radius_k - |key_l - centre_k|, 0)).
+// As tensor ops this materialises (B, 8K, L, 3) deltas several times and gathers 8 * 8 * 16 table entries per (l, k)
+// from global memory.  Here the table (64 KB, node-major: 16 channels of a node contiguous) lives in LDS, a thread
+// owns one (l, k) pair with its box's corners in registers, and the output row (16 values) leaves as one
+// contiguous store; no intermediate exists.  The backward is the table gradient only (corners are detached in the
+// reference, key positions and angles are inputs): the same walk, scattering weight * ddist into an LDS copy of the
+// table with ds_add_f32, then a fixed-order sum of the per-workgroup copies.
+#include "issm_dev.h"
+
+namespace issm {
+
+constexpr int BD_C = 16;          // channels of the table
+constexpr int BD_MAXCELLS = 1024; // D * H * W nodes that fit the 64 KB LDS copy
+
+struct BoxLane {
+  float cx[8], cy[8], cz[8];  // corners of the lane's box
+  float cs[8], sn[8];         // rotation of flattened corner j = k * 8 + c: angle of query j mod K (as the reference)
+  float qx, qy, qz, radius;
+};
+
+__device__ __forceinline__ void load_box(const BoxDistP& p, int b, int k, BoxLane& bx) {
+  const float* c = p.corners + ((long)b * p.K + k) * 24;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    bx.cx[j] = c[3 * j];
+    bx.cy[j] = c[3 * j + 1];
+    bx.cz[j] = c[3 * j + 2];
+    bx.cs[j] = 1.0f;
+    bx.sn[j] = 0.0f;
+    if (p.angle) {  // uniform
+      const float a = p.angle[(long)b * p.K + (k * 8 + j) % p.K];
+      bx.cs[j] = cosf(a);
+      bx.sn[j] = sinf(a);
+    }
+  }
+  if (p.qcenter) {
+    const float* q = p.qcenter + ((long)b * p.K + k) * 3;
+    bx.qx = q[0]; bx.qy = q[1]; bx.qz = q[2];
+    bx.radius = p.radius[(long)b * p.K + k];
+  }
+}
+
+// corner slot j takes the values of slot j + 1, slot 7 those of slot 0 (after 8 calls the box is as it was)
+__device__ __forceinline__ void rotate_box(BoxLane& bx) {
+  const float x0 = bx.cx[0], y0 = bx.cy[0], z0 = bx.cz[0], c0 = bx.cs[0], s0 = bx.sn[0];
+#pragma unroll
+  for (int j = 0; j < 7; ++j) {
+    bx.cx[j] = bx.cx[j + 1]; bx.cy[j] = bx.cy[j + 1]; bx.cz[j] = bx.cz[j + 1];
+    bx.cs[j] = bx.cs[j + 1]; bx.sn[j] = bx.sn[j + 1];
+  }
+  bx.cx[7] = x0; bx.cy[7] = y0; bx.cz[7] = z0; bx.cs[7] = c0; bx.sn[7] = s0;
+}
+
+// signed log compression and grid_sample's un-normalisation (align_corners False) in one: position in node units
+__device__ __forceinline__ float node_pos(float v, float log_scale, float scale, int n) {
+  const float m = __log2f(fabsf(v) * log_scale + 1.0f) * scale;  // scale = 1 / (log2(8) * max_value)
+  const float g = v < 0.0f ? -m : m;
+  return (g + 1.0f) * (0.5f * n) - 0.5f;
+}
+
+// The 8 neighbours of one sampling position: LDS offset (in floats) of the node and its weight (0 outside).
+struct Tri {
+  int off[8];
+  float w[8];
+};
+__device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, float z, Tri& t) {
+  const float fx = floorf(x), fy = floorf(y), fz = floorf(z);
+  const float ax = x - fx, ay = y - fy, az = z - fz;
+  const int ix = (int)fx, iy = (int)fy, iz = (int)fz;
+#pragma unroll
+  for (int n = 0; n < 8; ++n) {
+    const int dx = n & 1, dy = (n >> 1) & 1, dz = n >> 2;
+    const int jx = ix + dx, jy = iy + dy, jz = iz + dz;
+    const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
+    const float w = (dx ? ax : 1.0f - ax) * (dy ? ay : 1.0f - ay) * (dz ? az : 1.0f - az);
+    t.w[n] = ok ? w : 0.0f;
+    t.off[n] = ok ? ((jz * p.H + jy) * p.W + jx) * BD_C : 0;
+  }
+}
+
+// work split: items = (b, k chunk of 256, l), l fastest; workgroup w takes a contiguous range
+struct Items {
+  long i0, i1;
+  int kchunks;
+};
+__device__ __forceinline__ Items my_items(const BoxDistP& p) {
+  Items it;
+  it.kchunks = (p.K + NTHREADS - 1) / NTHREADS;
+  const long n = (long)p.B * it.kchunks * p.L;
+  it.i0 = n * blockIdx.x / gridDim.x;
+  it.i1 = n * (blockIdx.x + 1) / gridDim.x;
+  return it;
+}
+
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_box_dist_fwd(BoxDistP p) {
+  __shared__ __attribute__((aligned(16))) float tab[BD_MAXCELLS * BD_C];
+  const int cells = p.D * p.H * p.W;
+  if (p.dist) {  // uniform; a weights-only call brings no table
+    for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) {
+      const int ch = e / cells, cell = e - ch * cells;
+      tab[cell * BD_C + ch] = p.table[e];
+    }
+  }
+  __syncthreads();
+  const Items it = my_items(p);
+  const float scale = 1.0f / (3.0f * p.max_value);
+  BoxLane bx;
+  long cur = -1;
+  for (long item = it.i0; item < it.i1; ++item) {
+    const int l = (int)(item % p.L);
+    const long bk = item / p.L;
+    const int b = (int)(bk / it.kchunks), k = (int)(bk % it.kchunks) * NTHREADS + threadIdx.x;
+    if (k >= p.K) continue;
+    if (bk != cur) {
+      load_box(p, b, k, bx);
+      cur = bk;
+    }
+    const float* key = p.key + ((long)b * p.L + l) * 3;  // uniform
+    const float kx = key[0], ky = key[1], kz = key[2];
+    const long o = ((long)b * p.L + l) * p.K + k;
+    if (p.dist) {
+      f4 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+      // A rolled loop that always works on slot 0 and then rotates the box's registers by one corner: fully
+      // unrolled, the compiler issues the LDS reads of all 8 corners first and spills them.
+#pragma unroll 1
+      for (int c = 0; c < 8; ++c) {
+        const float dx = bx.cx[0] - kx, dy = bx.cy[0] - ky, dz = bx.cz[0] - kz;
+        const float rx = dx * bx.cs[0] - dy * bx.sn[0], ry = dx * bx.sn[0] + dy * bx.cs[0];
+        Tri t;
+        trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
+                  node_pos(dz, p.log_scale, scale, p.D), t);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          const f4* src = (const f4*)(tab + t.off[n]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] += t.w[n] * src[j];
+        }
+        rotate_box(bx);
+      }
+      if (BF) {
+        uint4* dst = (uint4*)((uint16_t*)p.dist + o * BD_C);
+        dst[0] = make_uint4(pack_bf16(acc[0].x, acc[0].y), pack_bf16(acc[0].z, acc[0].w), pack_bf16(acc[1].x, acc[1].y),
+                            pack_bf16(acc[1].z, acc[1].w));
+        dst[1] = make_uint4(pack_bf16(acc[2].x, acc[2].y), pack_bf16(acc[2].z, acc[2].w), pack_bf16(acc[3].x, acc[3].y),
+                            pack_bf16(acc[3].z, acc[3].w));
+      } else {
+        f4* dst = (f4*)((float*)p.dist + o * BD_C);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[j] = acc[j];
+      }
+    }
+    if (p.weights) {
+      const float ex = kx - bx.qx, ey = ky - bx.qy, ez = kz - bx.qz;
+      const float d = sqrtf(ex * ex + ey * ey + ez * ez);
+      p.weights[o] = __expf(p.weight_dist * fminf(bx.radius - d, 0.0f));
+    }
+  }
+}
+
+// Table gradient: partial[wg][cell][ch] = sum over the workgroup's (l, k) pairs and corners of weight * ddist.
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
+  __shared__ __attribute__((aligned(16))) float tab[BD_MAXCELLS * BD_C];
+  const int cells = p.D * p.H * p.W;
+  for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) tab[e] = 0.0f;
+  __syncthreads();
+  const Items it = my_items(p);
+  const float scale = 1.0f / (3.0f * p.max_value);
+  BoxLane bx;
+  long cur = -1;
+  for (long item = it.i0; item < it.i1; ++item) {
+    const int l = (int)(item % p.L);
+    const long bk = item / p.L;
+    const int b = (int)(bk / it.kchunks), k = (int)(bk % it.kchunks) * NTHREADS + threadIdx.x;
+    if (k >= p.K) continue;
+    if (bk != cur) {
+      load_box(p, b, k, bx);
+      cur = bk;
+    }
+    const float* key = p.key + ((long)b * p.L + l) * 3;
+    const float kx = key[0], ky = key[1], kz = key[2];
+    const long o = ((long)b * p.L + l) * p.K + k;
+    float g[BD_C];
+    if (BF) {
+      const uint4* src = (const uint4*)((const uint16_t*)p.ddist + o * BD_C);
+      const uint4 a = src[0], c = src[1];
+      const unsigned w[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        g[2 * j] = __uint_as_float(w[j] << 16);
+        g[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    } else {
+      const f4* src = (const f4*)((const float*)p.ddist + o * BD_C);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f4 v = src[j];
+        g[4 * j] = v.x; g[4 * j + 1] = v.y; g[4 * j + 2] = v.z; g[4 * j + 3] = v.w;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const float dx = bx.cx[c] - kx, dy = bx.cy[c] - ky, dz = bx.cz[c] - kz;
+      const float rx = dx * bx.cs[c] - dy * bx.sn[c], ry = dx * bx.sn[c] + dy * bx.cs[c];
+      Tri t;
+      trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
+                node_pos(dz, p.log_scale, scale, p.D), t);
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {
+        if (t.w[n] != 0.0f) {
+          float* dst = tab + t.off[n];
+#pragma unroll
+          for (int j = 0; j < BD_C; ++j) atomicAdd(dst + j, t.w[n] * g[j]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  float* out = p.partial + (long)blockIdx.x * cells * BD_C;
+  for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) out[e] = tab[e];
+}
+
+// dtable[ch][cell] = fixed-order sum over workgroups of partial[wg][cell][ch]
+__global__ __launch_bounds__(NTHREADS) void k_box_dist_dtable(BoxDistP p) {
+  const int cells = p.D * p.H * p.W;
+  const int e = blockIdx.x * NTHREADS + threadIdx.x;  // e = cell * 16 + ch
+  if (e >= cells * BD_C) return;
+  float a0 = 0.0f, a1 = 0.0f;
+  int w = 0;
+  for (; w + 1 < p.nwg; w += 2) {
+    a0 += p.partial[(long)w * cells * BD_C + e];
+    a1 += p.partial[(long)(w + 1) * cells * BD_C + e];
+  }
+  if (w < p.nwg) a0 += p.partial[(long)w * cells * BD_C + e];
+  const int cell = e / BD_C, ch = e % BD_C;
+  p.dtable[(long)ch * cells + cell] = a0 + a1;
+}
+
+int box_dist_workgroups(int B, int L, int K) {
+  const long items = (long)B * ((K + NTHREADS - 1) / NTHREADS) * L;
+  return (int)(items < 512 ? items : 512);  // two 64 KB workgroups per CU
+}
+
+int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st) {
+  const dim3 g(p.nwg), b(NTHREADS);
+  if (p.dtype) hipLaunchKernelGGL(k_box_dist_fwd<true>, g, b, 0, st, p);
+  else hipLaunchKernelGGL(k_box_dist_fwd<false>, g, b, 0, st, p);
+  return (int)hipGetLastError();
+}
+
+int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st) {
+  const dim3 g(p.nwg), b(NTHREADS);
+  if (p.dtype) hipLaunchKernelGGL(k_box_dist_bwd<true>, g, b, 0, st, p);
+  else hipLaunchKernelGGL(k_box_dist_bwd<false>, g, b, 0, st, p);
+  int e = (int)hipGetLastError();
+  if (e) return e;
+  const int n = p.D * p.H * p.W * BD_C;
+  hipLaunchKernelGGL(k_box_dist_dtable, dim3((n + NTHREADS - 1) / NTHREADS), b, 0, st, p);
+  return (int)hipGetLastError();
+}
+
+}  // namespace issm

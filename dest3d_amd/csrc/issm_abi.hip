@@ -25,6 +25,9 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
+int box_dist_workgroups(int B, int L, int K);
+int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st);
+int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st);
 int dwconv_partial_rows(int B, int L);
 int launch_dwconv_fwd(const DwConvP& p, hipStream_t st);
 int launch_dwconv_bwd(const DwConvP& p, hipStream_t st);
@@ -485,6 +488,48 @@ int issm_dwconv_silu_bwd(const issm_dwconv_args* a) {
   int rc = dwconv_params(a, &p, true);
   if (rc) return rc;
   return launched(launch_dwconv_bwd(p, (hipStream_t)a->stream), "dwconv_silu_bwd");
+}
+
+static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
+  if (!a) return fail(ISSM_E_NULL, "box_dist: args is NULL");
+  if (a->batch < 0 || a->seqlen < 0 || a->nquery < 0 || a->D < 1 || a->H < 1 || a->W < 1)
+    return fail(ISSM_E_SHAPE, "box_dist: bad shape");
+  if ((int64_t)a->D * a->H * a->W > 1024)
+    return fail(ISSM_E_UNSUPPORTED, "box_dist: table of %d x %d x %d nodes (at most 1024 fit)", a->D, a->H, a->W);
+  if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "box_dist: dtype %d", a->dtype);
+  if (!a->key || !a->corners) return fail(ISSM_E_NULL, "box_dist: key/corners is NULL");
+  if (!bwd) {
+    if (a->dist && !a->table) return fail(ISSM_E_NULL, "box_dist: table is NULL");
+    if (a->weights && (!a->qcenter || !a->radius)) return fail(ISSM_E_NULL, "box_dist: qcenter/radius is NULL");
+  } else if (!a->ddist || !a->partial || !a->dtable) {
+    return fail(ISSM_E_NULL, "box_dist bwd: ddist/partial/dtable is NULL");
+  }
+  p->B = a->batch; p->L = a->seqlen; p->K = a->nquery; p->D = a->D; p->H = a->H; p->W = a->W; p->dtype = a->dtype;
+  p->nwg = box_dist_workgroups(a->batch, a->seqlen, a->nquery);
+  p->key = a->key; p->corners = a->corners; p->angle = a->angle; p->table = a->table;
+  p->log_scale = a->log_scale; p->max_value = a->max_value; p->dist = a->dist;
+  p->qcenter = a->qcenter; p->radius = a->radius; p->weight_dist = a->weight_dist; p->weights = a->weights;
+  p->ddist = a->ddist; p->partial = a->partial; p->dtable = a->dtable;
+  return ISSM_OK;
+}
+
+int issm_box_dist_workgroups(int32_t batch, int32_t seqlen, int32_t nquery) {
+  return (batch > 0 && seqlen > 0 && nquery > 0) ? box_dist_workgroups(batch, seqlen, nquery) : 0;
+}
+
+int issm_box_dist_fwd(const issm_box_dist_args* a) {
+  BoxDistP p;
+  int rc = box_dist_params(a, &p, false);
+  if (rc) return rc;
+  if (p.nwg == 0 || (!p.dist && !p.weights)) return ISSM_OK;
+  return launched(launch_box_dist_fwd(p, (hipStream_t)a->stream), "box_dist_fwd");
+}
+
+int issm_box_dist_bwd(const issm_box_dist_args* a) {
+  BoxDistP p;
+  int rc = box_dist_params(a, &p, true);
+  if (rc) return rc;
+  return launched(launch_box_dist_bwd(p, (hipStream_t)a->stream), "box_dist_bwd");
 }
 
 }  // extern "C"

@@ -78,6 +78,24 @@ struct NormP {
   int nblocks;
 };
 
+// parameters of the box-to-point distance encoding kernels (box_dist.hip)
+struct BoxDistP {
+  int B, L, K, D, H, W, dtype, nwg;
+  const float* key;      // (B, L, 3)
+  const float* corners;  // (B, K, 8, 3)
+  const float* angle;    // (B, K) or NULL (zero)
+  const float* table;    // (16, D, H, W)
+  float log_scale, max_value;
+  void* dist;            // (B, L, K, 16) io dtype, or NULL
+  const float* qcenter;  // (B, K, 3), with radius (B, K): inputs of the locality weight
+  const float* radius;
+  float weight_dist;
+  float* weights;        // (B, L, K) fp32, or NULL
+  const void* ddist;     // (B, L, K, 16) io dtype
+  float* partial;        // (nwg, D*H*W, 16) fp32
+  float* dtable;         // (16, D, H, W) fp32
+};
+
 // parameters of the depthwise conv + SiLU kernels (dwconv_silu.hip)
 struct DwConvP {
   int B, L, C, nsets, dtype;
@@ -113,6 +131,14 @@ struct PGenP {
   float* dW;             // (R0, M) fp32
   int nblocks;
 };
+
+// two floats -> two bf16 (round to nearest even) in one dword
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  typedef float fl2 __attribute__((ext_vector_type(2)));
+  const bf2 h = __builtin_convertvector((fl2){lo, hi}, bf2);
+  return __builtin_bit_cast(unsigned, h);
+}
 
 __device__ __forceinline__ float bf16_to_f(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float f) {

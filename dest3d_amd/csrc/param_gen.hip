@@ -60,14 +60,6 @@ __device__ __forceinline__ void st1(void* p, long i, float v) {
   if (BF) ((uint16_t*)p)[i] = f_to_bf16(v); else ((float*)p)[i] = v;
 }
 
-// two floats -> two bf16 (round to nearest even) in one dword
-__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
-  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-  typedef float fl2 __attribute__((ext_vector_type(2)));
-  const bf2 h = __builtin_convertvector((fl2){lo, hi}, bf2);
-  return __builtin_bit_cast(unsigned, h);
-}
-
 // Forward: thread = (token, k).  W and the token's biases are uniform across the workgroup's lanes of a token.
 template <bool BF>
 __global__ __launch_bounds__(NTHREADS) void k_pgen_fwd(PGenP p) {

@@ -306,6 +306,44 @@ int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);
 int issm_dwconv_silu_fwd(const issm_dwconv_args* args);
 int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
 
+/* ---- box-to-point distance encoding and locality weight ----------------------------------
+ * BoxDistFun.forward (models/dest_module.py:174-195) and ISSMDecoderLayer.local_weight (:240-249), the two
+ * (B, L, K) fields computed right before MultiHeadISSMScan:
+ *   dist[b][l][k][0..15] = sum over the 8 corners c of box k of trilinear(table, f(R_j (corner - key_l)))
+ *     f(v) = sign(v) log2(|v| log_scale + 1) / log2(8) / max_value per component, R_j the x-y rotation by
+ *     angle[b][(8k + c) mod K] (the reference tiles the angles that way; NULL = no rotation), trilinear =
+ *     grid_sample(mode bilinear, padding zeros, align_corners False) with x indexing W, y H, z D;
+ *   weights[b][l][k] = exp(weight_dist * min(radius[b][k] - |key_l - qcenter[b][k]|, 0)).
+ * key (B, L, 3), corners (B, K, 8, 3), angle (B, K), table (16, D, H, W) with D*H*W <= 1024, qcenter (B, K, 3),
+ * radius (B, K), weights (B, L, K), dtable (16, D, H, W): fp32 contiguous.  dist and ddist: (B, L, K, 16)
+ * contiguous in `dtype`.  Either output of the forward may be NULL (skipped).  The backward produces the table
+ * gradient only (the reference detaches the corners; key positions and angles are inputs); partial:
+ * issm_box_dist_workgroups(B, L, K) * D*H*W * 16 floats of scratch.  The per-workgroup accumulation uses LDS
+ * float atomics, so dtable can differ in the last bits between runs. */
+typedef struct issm_box_dist_args {
+  int32_t batch, seqlen, nquery, D, H, W;
+  int32_t dtype;
+  const float* key;
+  const float* corners;
+  const float* angle;
+  const float* table;
+  float log_scale, max_value;
+  void* dist;
+  const float* qcenter;
+  const float* radius;
+  float weight_dist;
+  float* weights;
+  /* backward */
+  const void* ddist;
+  float* partial;
+  float* dtable;
+  void* stream;
+} issm_box_dist_args;
+
+int issm_box_dist_workgroups(int32_t batch, int32_t seqlen, int32_t nquery);
+int issm_box_dist_fwd(const issm_box_dist_args* args);
+int issm_box_dist_bwd(const issm_box_dist_args* args);
+
 #ifdef __cplusplus
 }
 #endif
