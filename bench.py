@@ -190,6 +190,41 @@ def cpu_baseline(torch):
             "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional"}
 
 
+def time_box_dist_layer(torch, steps=10, warmup=3):
+    """BoxDistFun + local_weight + MultiHeadISSMScan as ISSMDecoderLayer chains them (models/dest_module.py:283-290)
+    at the configs[2] shape, bf16 module, forward + backward, microseconds.  Returns (whole, box_dist forward only)."""
+    from dest3d_amd.box_dist import BoxDistFun
+    from dest3d_amd.scan_module import MultiHeadISSMScan
+    torch.manual_seed(0)
+    m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1).cuda().bfloat16()
+    bd = BoxDistFun(out_dim=16).cuda().bfloat16()
+    key = torch.randn(8, 1024, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    query = torch.randn(8, 256, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    key_pos = 8.0 * torch.rand(8, 1024, 3, device="cuda")
+    query_pos = torch.cat([8.0 * torch.rand(8, 256, 3, device="cuda"), 0.2 + 2.0 * torch.rand(8, 256, 3, device="cuda")], -1)
+    zero_angle = torch.zeros(8, 256, device="cuda")
+
+    def encode():
+        return bd(key_pos, query_pos[..., :3], query_pos[..., 3:], zero_angle, weight_query_pos=query_pos)
+
+    def step():
+        dist, weights = encode()
+        ok, oq = m(key, query, dist, key_pos, weights)
+        (ok.float().square().mean() + oq.float().square().mean()).backward()
+
+    out = []
+    for fn in (step, encode):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        out.append((time.perf_counter() - t0) / steps * 1e6)
+    return out
+
+
 def time_module_layer(torch, steps=10, warmup=3):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16, float locality weights as mask -- what DEST's decoder layer passes,
@@ -240,8 +275,10 @@ def main():
         sys.exit(2)
 
     if args.only_layer:
+        whole, enc = time_box_dist_layer(torch, args.steps, args.warmup)
         print(json.dumps({"detector_layer_bf16_fwd_bwd_us": round(time_module_layer(torch, args.steps, args.warmup), 2),
-                          "steps": args.steps, "warmup": args.warmup}))
+                          "box_dist_plus_layer_bf16_fwd_bwd_us": round(whole, 2),
+                          "box_dist_and_weight_fwd_us": round(enc, 2), "steps": args.steps, "warmup": args.warmup}))
         return
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
@@ -280,6 +317,7 @@ def main():
             del r
         SHAPE["P"] = 32
         variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
+        variants["box_dist_plus_layer_bf16_fwd_bwd"] = round(time_box_dist_layer(torch)[0], 2)
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),

@@ -86,6 +86,73 @@ __device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, f
   }
 }
 
+// The 8 corners of a box usually fall into the same or adjacent table cells (a box is small next to the spacing
+// of the log-compressed lattice), so their 8 x 8 node weights are first merged, in registers, over a 3 x 3 x 3 window
+// of nodes anchored at the smallest base node: up to 27 -- typically 8 to 12 non-zero -- table accesses per
+// (point, box) pair instead of 64.  Possible when the corners' base nodes differ by at most one along every axis;
+// otherwise the caller walks the corners one by one.
+struct Window {
+  int mx, my, mz;
+  float w[27];  // [dz][dy][dx]
+};
+__device__ __forceinline__ bool corner_window(const BoxDistP& p, const BoxLane& bx, float kx, float ky, float kz,
+                                              float scale, Window& win) {
+  float fx[8], fy[8], fz[8];
+  int ix[8], iy[8], iz[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float dx = bx.cx[c] - kx, dy = bx.cy[c] - ky, dz = bx.cz[c] - kz;
+    const float rx = dx * bx.cs[c] - dy * bx.sn[c], ry = dx * bx.sn[c] + dy * bx.cs[c];
+    const float x = node_pos(rx, p.log_scale, scale, p.W), y = node_pos(ry, p.log_scale, scale, p.H),
+                z = node_pos(dz, p.log_scale, scale, p.D);
+    const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
+    fx[c] = x - gx; fy[c] = y - gy; fz[c] = z - gz;
+    ix[c] = (int)gx; iy[c] = (int)gy; iz[c] = (int)gz;
+  }
+  int mx = ix[0], my = iy[0], mz = iz[0], Mx = ix[0], My = iy[0], Mz = iz[0];
+#pragma unroll
+  for (int c = 1; c < 8; ++c) {
+    mx = min(mx, ix[c]); Mx = max(Mx, ix[c]);
+    my = min(my, iy[c]); My = max(My, iy[c]);
+    mz = min(mz, iz[c]); Mz = max(Mz, iz[c]);
+  }
+  if (Mx - mx > 1 || My - my > 1 || Mz - mz > 1) return false;
+  win.mx = mx; win.my = my; win.mz = mz;
+#pragma unroll
+  for (int e = 0; e < 27; ++e) win.w[e] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const bool sx = ix[c] != mx, sy = iy[c] != my, sz = iz[c] != mz;
+    const float ax[3] = {sx ? 0.0f : 1.0f - fx[c], sx ? 1.0f - fx[c] : fx[c], sx ? fx[c] : 0.0f};
+    const float ay[3] = {sy ? 0.0f : 1.0f - fy[c], sy ? 1.0f - fy[c] : fy[c], sy ? fy[c] : 0.0f};
+    const float az[3] = {sz ? 0.0f : 1.0f - fz[c], sz ? 1.0f - fz[c] : fz[c], sz ? fz[c] : 0.0f};
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const float yx = ay[i] * ax[j];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) win.w[k * 9 + i * 3 + j] = fmaf(az[k], yx, win.w[k * 9 + i * 3 + j]);
+      }
+  }
+  return true;
+}
+// visit the window's nodes that lie inside the table and carry weight: f(LDS offset in floats, weight)
+template <class F>
+__device__ __forceinline__ void for_window(const BoxDistP& p, const Window& win, F f) {
+#pragma unroll
+  for (int k = 0; k < 3; ++k)
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int jx = win.mx + j, jy = win.my + i, jz = win.mz + k;
+        const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
+        const float w = win.w[k * 9 + i * 3 + j];
+        if (ok && w != 0.0f) f(((jz * p.H + jy) * p.W + jx) * BD_C, w);
+      }
+}
+
 // work split: items = (b, k chunk of 256, l), l fastest; workgroup w takes a contiguous range
 struct Items {
   long i0, i1;
@@ -131,22 +198,31 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_fwd(BoxDistP p) {
       f4 acc[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[j] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
-      // A rolled loop that always works on slot 0 and then rotates the box's registers by one corner: fully
-      // unrolled, the compiler issues the LDS reads of all 8 corners first and spills them.
+      Window win;
+      if (corner_window(p, bx, kx, ky, kz, scale, win)) {
+        for_window(p, win, [&](int off, float w) {
+          const f4* src = (const f4*)(tab + off);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] += w * src[j];
+        });
+      } else {
+        // A rolled loop that always works on slot 0 and then rotates the box's registers by one corner: fully
+        // unrolled, the compiler issues the LDS reads of all 8 corners first and spills them.
 #pragma unroll 1
-      for (int c = 0; c < 8; ++c) {
-        const float dx = bx.cx[0] - kx, dy = bx.cy[0] - ky, dz = bx.cz[0] - kz;
-        const float rx = dx * bx.cs[0] - dy * bx.sn[0], ry = dx * bx.sn[0] + dy * bx.cs[0];
-        Tri t;
-        trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
-                  node_pos(dz, p.log_scale, scale, p.D), t);
+        for (int c = 0; c < 8; ++c) {
+          const float dx = bx.cx[0] - kx, dy = bx.cy[0] - ky, dz = bx.cz[0] - kz;
+          const float rx = dx * bx.cs[0] - dy * bx.sn[0], ry = dx * bx.sn[0] + dy * bx.cs[0];
+          Tri t;
+          trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
+                    node_pos(dz, p.log_scale, scale, p.D), t);
 #pragma unroll
-        for (int n = 0; n < 8; ++n) {
-          const f4* src = (const f4*)(tab + t.off[n]);
+          for (int n = 0; n < 8; ++n) {
+            const f4* src = (const f4*)(tab + t.off[n]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[j] += t.w[n] * src[j];
+            for (int j = 0; j < 4; ++j) acc[j] += t.w[n] * src[j];
+          }
+          rotate_box(bx);
         }
-        rotate_box(bx);
       }
       if (BF) {
         uint4* dst = (uint4*)((uint16_t*)p.dist + o * BD_C);
@@ -177,6 +253,9 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
   __syncthreads();
   const Items it = my_items(p);
   const float scale = 1.0f / (3.0f * p.max_value);
+  int rot[BD_C];
+#pragma unroll
+  for (int j = 0; j < BD_C; ++j) rot[j] = (j + threadIdx.x) & 15;
   BoxLane bx;
   long cur = -1;
   for (long item = it.i0; item < it.i1; ++item) {
@@ -209,20 +288,42 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
         g[4 * j] = v.x; g[4 * j + 1] = v.y; g[4 * j + 2] = v.z; g[4 * j + 3] = v.w;
       }
     }
+    // Lane r adds channel (j + r) mod 16 at step j.  Samples crowd into few nodes (the signed log maps most
+    // distances near +-1), so many lanes of a wave hit the same node at once: with every lane on channel j that is
+    // one LDS address and the adds serialise; rotated, the lanes of a node spread over its 16 channels.
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const float dx = bx.cx[c] - kx, dy = bx.cy[c] - ky, dz = bx.cz[c] - kz;
-      const float rx = dx * bx.cs[c] - dy * bx.sn[c], ry = dx * bx.sn[c] + dy * bx.cs[c];
-      Tri t;
-      trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
-                node_pos(dz, p.log_scale, scale, p.D), t);
+    for (int bit = 8; bit >= 1; bit >>= 1) {
+      const bool on = (threadIdx.x & bit) != 0;
+      float t[BD_C];
 #pragma unroll
-      for (int n = 0; n < 8; ++n) {
-        if (t.w[n] != 0.0f) {
-          float* dst = tab + t.off[n];
+      for (int j = 0; j < BD_C; ++j) t[j] = on ? g[(j + bit) & 15] : g[j];
 #pragma unroll
-          for (int j = 0; j < BD_C; ++j) atomicAdd(dst + j, t.w[n] * g[j]);
+      for (int j = 0; j < BD_C; ++j) g[j] = t[j];
+    }
+    Window win;
+    if (corner_window(p, bx, kx, ky, kz, scale, win)) {
+      for_window(p, win, [&](int off, float w) {
+        float* dst = tab + off;
+#pragma unroll
+        for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], w * g[j]);
+      });
+    } else {
+#pragma unroll 1
+      for (int c = 0; c < 8; ++c) {
+        const float dx = bx.cx[0] - kx, dy = bx.cy[0] - ky, dz = bx.cz[0] - kz;
+        const float rx = dx * bx.cs[0] - dy * bx.sn[0], ry = dx * bx.sn[0] + dy * bx.cs[0];
+        Tri t;
+        trilinear(p, node_pos(rx, p.log_scale, scale, p.W), node_pos(ry, p.log_scale, scale, p.H),
+                  node_pos(dz, p.log_scale, scale, p.D), t);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          if (t.w[n] != 0.0f) {
+            float* dst = tab + t.off[n];
+#pragma unroll
+            for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], t.w[n] * g[j]);
+          }
         }
+        rotate_box(bx);
       }
     }
   }
