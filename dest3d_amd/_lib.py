@@ -26,7 +26,7 @@ EXPORTS = [
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
-    "issm_box_dist_workgroups", "issm_box_dist_fwd", "issm_box_dist_bwd",
+    "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
 ]
 
 
@@ -149,7 +149,7 @@ def load() -> C.CDLL:
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
-    lib.issm_box_dist_workgroups.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
     lib.issm_box_dist_fwd.argtypes = [P(BoxDistArgs)]
     lib.issm_box_dist_bwd.argtypes = [P(BoxDistArgs)]
     lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]
@@ -161,6 +161,7 @@ def load() -> C.CDLL:
     for name in EXPORTS:
         if name != "issm_last_error":
             getattr(lib, name).restype = C.c_int
+    lib.issm_box_dist_bwd_scratch_bytes.restype = C.c_int64
     _lib = lib
     return lib
 

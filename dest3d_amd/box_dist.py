@@ -98,8 +98,8 @@ class BoxDistFn(torch.autograd.Function):
                 a.key, a.corners = key.data_ptr(), cor.data_ptr()
                 a.angle = None if ang is None else ang.data_ptr()
                 a.log_scale, a.max_value = float(log_scale), float(max_value)
-                nwg = lib.issm_box_dist_workgroups(Bsz, nP, nQ)
-                partial = torch.empty((max(nwg, 1), D * H * W, CHANNELS), dtype=torch.float32, device=key.device)
+                nbytes = lib.issm_box_dist_bwd_scratch_bytes(Bsz, nP, nQ, D, H, W)
+                partial = torch.empty(nbytes // 8, dtype=torch.int64, device=key.device)
                 out = torch.zeros((Cn, D, H, W), dtype=torch.float32, device=key.device)
                 a.ddist, a.partial, a.dtable = g.data_ptr(), partial.data_ptr(), out.data_ptr()
                 a.stream = L.current_stream_ptr(key.device)

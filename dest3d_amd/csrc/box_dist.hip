@@ -12,7 +12,9 @@
 // owns one (l, k) pair with its box's corners in registers, and the output row (16 values) leaves as one
 // contiguous store; no intermediate exists.  The backward is the table gradient only (corners are detached in the
 // reference, key positions and angles are inputs): the same walk, scattering weight * ddist into an LDS copy of the
-// table with ds_add_f32, then a fixed-order sum of the per-workgroup copies.
+// table, then a sum of the per-workgroup copies.  The LDS copy is 64-bit fixed point (terms scaled by
+// 2^34 / max|ddist|, found by a first pass): LDS integer atomics run about twice as fast as ds_add_f32 here, and
+// integer sums do not depend on the order of the adds, so the gradient is reproducible bit for bit.
 #include "issm_dev.h"
 
 namespace issm {
@@ -244,13 +246,48 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_fwd(BoxDistP p) {
   }
 }
 
+// Fixed-point scale of the table gradient.  A pair's node weights sum to 8 (one per corner), so a node of one
+// workgroup's copy collects at most 8 * pairs-per-workgroup * max|ddist|; with 2^34 / max|ddist| that stays below
+// 2^63 for 2^26 pairs per workgroup, and the sum over all workgroups is taken in 64 bits as well (2^26 pairs in total
+// is the bound the launcher checks).
+__device__ __forceinline__ float bd_scale(const unsigned* scal) {
+  const float gmax = __uint_as_float(scal[0]);
+  return gmax > 0.0f ? 17179869184.0f / gmax : 1.0f;
+}
+
+__global__ void k_box_dist_clear(unsigned* scal) { scal[0] = 0u; }
+
+// max |ddist| (bit pattern of a non-negative float orders like the unsigned integer)
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_box_dist_gmax(BoxDistP p, unsigned* scal) {
+  const long n = (long)p.B * p.L * p.K * BD_C;
+  float m = 0.0f;
+  for (long e = ((long)blockIdx.x * NTHREADS + threadIdx.x) * 8; e < n; e += (long)gridDim.x * NTHREADS * 8) {
+    if (BF) {
+      const uint4 v = *(const uint4*)((const uint16_t*)p.ddist + e);
+      const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        m = fmaxf(m, fmaxf(fabsf(__uint_as_float(w[j] << 16)), fabsf(__uint_as_float(w[j] & 0xffff0000u))));
+    } else {
+      const f4 a = *(const f4*)((const float*)p.ddist + e), c = *(const f4*)((const float*)p.ddist + e + 4);
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0 && m > 0.0f && m == m) atomicMax(scal, __float_as_uint(m));
+}
+
 // Table gradient: partial[wg][cell][ch] = sum over the workgroup's (l, k) pairs and corners of weight * ddist.
 template <bool BF>
 __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
-  __shared__ __attribute__((aligned(16))) float tab[BD_MAXCELLS * BD_C];
+  __shared__ __attribute__((aligned(16))) unsigned long long tab[BD_MAXCELLS * BD_C];  // 128 KB: one workgroup per CU
   const int cells = p.D * p.H * p.W;
-  for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) tab[e] = 0.0f;
+  for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) tab[e] = 0ull;
   __syncthreads();
+  const float fx_scale = bd_scale((const unsigned*)p.partial);
   const Items it = my_items(p);
   const float scale = 1.0f / (3.0f * p.max_value);
   int rot[BD_C];
@@ -288,6 +325,8 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
         g[4 * j] = v.x; g[4 * j + 1] = v.y; g[4 * j + 2] = v.z; g[4 * j + 3] = v.w;
       }
     }
+#pragma unroll
+    for (int j = 0; j < BD_C; ++j) g[j] *= fx_scale;
     // Lane r adds channel (j + r) mod 16 at step j.  Samples crowd into few nodes (the signed log maps most
     // distances near +-1), so many lanes of a wave hit the same node at once: with every lane on channel j that is
     // one LDS address and the adds serialise; rotated, the lanes of a node spread over its 16 channels.
@@ -303,9 +342,9 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
     Window win;
     if (corner_window(p, bx, kx, ky, kz, scale, win)) {
       for_window(p, win, [&](int off, float w) {
-        float* dst = tab + off;
+        unsigned long long* dst = tab + off;
 #pragma unroll
-        for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], w * g[j]);
+        for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], (unsigned long long)__float2ll_rn(w * g[j]));
       });
     } else {
 #pragma unroll 1
@@ -318,9 +357,9 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
           if (t.w[n] != 0.0f) {
-            float* dst = tab + t.off[n];
+            unsigned long long* dst = tab + t.off[n];
 #pragma unroll
-            for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], t.w[n] * g[j]);
+            for (int j = 0; j < BD_C; ++j) atomicAdd(dst + rot[j], (unsigned long long)__float2ll_rn(t.w[n] * g[j]));
           }
         }
         rotate_box(bx);
@@ -328,29 +367,29 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_bwd(BoxDistP p) {
     }
   }
   __syncthreads();
-  float* out = p.partial + (long)blockIdx.x * cells * BD_C;
+  unsigned long long* out = (unsigned long long*)p.partial + 2 + (long)blockIdx.x * cells * BD_C;
   for (int e = threadIdx.x; e < cells * BD_C; e += NTHREADS) out[e] = tab[e];
 }
 
-// dtable[ch][cell] = fixed-order sum over workgroups of partial[wg][cell][ch]
+// dtable[ch][cell] = (sum over workgroups of partial[wg][cell][ch], exact in 64 bits) / scale
 __global__ __launch_bounds__(NTHREADS) void k_box_dist_dtable(BoxDistP p) {
   const int cells = p.D * p.H * p.W;
   const int e = blockIdx.x * NTHREADS + threadIdx.x;  // e = cell * 16 + ch
   if (e >= cells * BD_C) return;
-  float a0 = 0.0f, a1 = 0.0f;
-  int w = 0;
-  for (; w + 1 < p.nwg; w += 2) {
-    a0 += p.partial[(long)w * cells * BD_C + e];
-    a1 += p.partial[(long)(w + 1) * cells * BD_C + e];
-  }
-  if (w < p.nwg) a0 += p.partial[(long)w * cells * BD_C + e];
+  const long long* part = (const long long*)p.partial + 2;
+  long long a = 0;
+  for (int w = 0; w < p.nwg_bwd; ++w) a += part[(long)w * cells * BD_C + e];
   const int cell = e / BD_C, ch = e % BD_C;
-  p.dtable[(long)ch * cells + cell] = a0 + a1;
+  p.dtable[(long)ch * cells + cell] = (float)((double)a / (double)bd_scale((const unsigned*)p.partial));
 }
 
 int box_dist_workgroups(int B, int L, int K) {
   const long items = (long)B * ((K + NTHREADS - 1) / NTHREADS) * L;
-  return (int)(items < 512 ? items : 512);  // two 64 KB workgroups per CU
+  return (int)(items < 512 ? items : 512);  // forward: two 64 KB workgroups per CU
+}
+int box_dist_bwd_workgroups(int B, int L, int K) {
+  const long items = (long)B * ((K + NTHREADS - 1) / NTHREADS) * L;
+  return (int)(items < 256 ? items : 256);  // backward: one 128 KB workgroup per CU
 }
 
 int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st) {
@@ -361,7 +400,11 @@ int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st) {
 }
 
 int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st) {
-  const dim3 g(p.nwg), b(NTHREADS);
+  const dim3 g(p.nwg_bwd), b(NTHREADS);
+  unsigned* scal = (unsigned*)p.partial;
+  hipLaunchKernelGGL(k_box_dist_clear, dim3(1), dim3(1), 0, st, scal);
+  if (p.dtype) hipLaunchKernelGGL(k_box_dist_gmax<true>, dim3(512), b, 0, st, p, scal);
+  else hipLaunchKernelGGL(k_box_dist_gmax<false>, dim3(512), b, 0, st, p, scal);
   if (p.dtype) hipLaunchKernelGGL(k_box_dist_bwd<true>, g, b, 0, st, p);
   else hipLaunchKernelGGL(k_box_dist_bwd<false>, g, b, 0, st, p);
   int e = (int)hipGetLastError();

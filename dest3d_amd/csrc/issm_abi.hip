@@ -26,6 +26,7 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
 int box_dist_workgroups(int B, int L, int K);
+int box_dist_bwd_workgroups(int B, int L, int K);
 int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st);
 int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st);
 int dwconv_partial_rows(int B, int L);
@@ -506,6 +507,9 @@ static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
   }
   p->B = a->batch; p->L = a->seqlen; p->K = a->nquery; p->D = a->D; p->H = a->H; p->W = a->W; p->dtype = a->dtype;
   p->nwg = box_dist_workgroups(a->batch, a->seqlen, a->nquery);
+  p->nwg_bwd = box_dist_bwd_workgroups(a->batch, a->seqlen, a->nquery);
+  if (bwd && (int64_t)a->batch * a->seqlen * a->nquery > ((int64_t)1 << 26))
+    return fail(ISSM_E_UNSUPPORTED, "box_dist bwd: more than 2^26 (point, box) pairs");
   p->key = a->key; p->corners = a->corners; p->angle = a->angle; p->table = a->table;
   p->log_scale = a->log_scale; p->max_value = a->max_value; p->dist = a->dist;
   p->qcenter = a->qcenter; p->radius = a->radius; p->weight_dist = a->weight_dist; p->weights = a->weights;
@@ -513,8 +517,9 @@ static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
   return ISSM_OK;
 }
 
-int issm_box_dist_workgroups(int32_t batch, int32_t seqlen, int32_t nquery) {
-  return (batch > 0 && seqlen > 0 && nquery > 0) ? box_dist_workgroups(batch, seqlen, nquery) : 0;
+int64_t issm_box_dist_bwd_scratch_bytes(int32_t batch, int32_t seqlen, int32_t nquery, int32_t D, int32_t H, int32_t W) {
+  if (batch <= 0 || seqlen <= 0 || nquery <= 0 || D <= 0 || H <= 0 || W <= 0) return 16;
+  return 16 + (int64_t)box_dist_bwd_workgroups(batch, seqlen, nquery) * D * H * W * 16 * 8;
 }
 
 int issm_box_dist_fwd(const issm_box_dist_args* a) {
@@ -529,6 +534,7 @@ int issm_box_dist_bwd(const issm_box_dist_args* a) {
   BoxDistP p;
   int rc = box_dist_params(a, &p, true);
   if (rc) return rc;
+  if (p.nwg_bwd == 0) return ISSM_OK;
   return launched(launch_box_dist_bwd(p, (hipStream_t)a->stream), "box_dist_bwd");
 }
 

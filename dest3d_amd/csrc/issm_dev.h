@@ -80,7 +80,7 @@ struct NormP {
 
 // parameters of the box-to-point distance encoding kernels (box_dist.hip)
 struct BoxDistP {
-  int B, L, K, D, H, W, dtype, nwg;
+  int B, L, K, D, H, W, dtype, nwg, nwg_bwd;
   const float* key;      // (B, L, 3)
   const float* corners;  // (B, K, 8, 3)
   const float* angle;    // (B, K) or NULL (zero)
@@ -92,7 +92,7 @@ struct BoxDistP {
   float weight_dist;
   float* weights;        // (B, L, K) fp32, or NULL
   const void* ddist;     // (B, L, K, 16) io dtype
-  float* partial;        // (nwg, D*H*W, 16) fp32
+  void* partial;         // 2 words (scale) + (nwg_bwd, D*H*W, 16) 64-bit fixed-point words
   float* dtable;         // (16, D, H, W) fp32
 };
 

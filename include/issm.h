@@ -318,8 +318,9 @@ int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
  * radius (B, K), weights (B, L, K), dtable (16, D, H, W): fp32 contiguous.  dist and ddist: (B, L, K, 16)
  * contiguous in `dtype`.  Either output of the forward may be NULL (skipped).  The backward produces the table
  * gradient only (the reference detaches the corners; key positions and angles are inputs); partial:
- * issm_box_dist_workgroups(B, L, K) * D*H*W * 16 floats of scratch.  The per-workgroup accumulation uses LDS
- * float atomics, so dtable can differ in the last bits between runs. */
+ * issm_box_dist_bwd_scratch_bytes(...) bytes of scratch, 16-byte aligned.  The gradient is accumulated in 64-bit
+ * fixed point scaled by 2^34 / max|ddist|, so it does not depend on the order of the adds (reproducible bit for
+ * bit; absolute resolution 2^-34 max|ddist| per term); at most 2^26 (point, box) pairs per call. */
 typedef struct issm_box_dist_args {
   int32_t batch, seqlen, nquery, D, H, W;
   int32_t dtype;
@@ -335,12 +336,12 @@ typedef struct issm_box_dist_args {
   float* weights;
   /* backward */
   const void* ddist;
-  float* partial;
+  void* partial;
   float* dtable;
   void* stream;
 } issm_box_dist_args;
 
-int issm_box_dist_workgroups(int32_t batch, int32_t seqlen, int32_t nquery);
+int64_t issm_box_dist_bwd_scratch_bytes(int32_t batch, int32_t seqlen, int32_t nquery, int32_t D, int32_t H, int32_t W);
 int issm_box_dist_fwd(const issm_box_dist_args* args);
 int issm_box_dist_bwd(const issm_box_dist_args* args);
 

@@ -82,6 +82,25 @@ def test_local_weight_and_fused_module_call():
         assert _rel(p.grad.cpu().numpy(), p2.grad.numpy()) <= 2e-3, n
 
 
+def test_table_gradient_is_bit_reproducible():
+    """The gradient is accumulated in 64-bit fixed point: the order of the adds cannot change it."""
+    from dest3d_amd.box_dist import box_dist, box_parametrization_to_corners
+    key, qxyz, qsize, ang = _inputs(2, 200, 256, 21, False)
+    tk, tq, ts, ta = (torch.from_numpy(x).cuda() for x in (key, qxyz, qsize, ang))
+    corners = box_parametrization_to_corners(tq, ts, ta)
+    g = torch.randn(2, 200, 256, 16, generator=torch.Generator().manual_seed(1)).cuda()
+    grads = []
+    for _ in range(3):
+        t = torch.randn(16, 10, 10, 10, generator=torch.Generator().manual_seed(2)).cuda().requires_grad_()
+        box_dist(t, tk, corners).backward(g)
+        grads.append(t.grad.clone())
+    assert torch.equal(grads[0], grads[1]) and torch.equal(grads[0], grads[2])
+    # a zero upstream gradient gives an exactly zero table gradient
+    t = torch.randn(16, 10, 10, 10, generator=torch.Generator().manual_seed(2)).cuda().requires_grad_()
+    box_dist(t, tk, corners).backward(torch.zeros_like(g))
+    assert t.grad.abs().max().item() == 0.0
+
+
 def test_box_dist_rejects_unbuilt_shapes():
     import ctypes as C
     from dest3d_amd import _lib as L
