@@ -103,6 +103,20 @@ class Runner:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e6
 
+    def step_percentiles(self, steps):
+        """p10 / p50 / p90 of single steps, each bracketed by HIP events on the launch stream (caches not flushed
+        between steps: consecutive steps reuse the same buffers, as a training loop does)."""
+        torch = self.torch
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for e0, e1 in ev:
+            e0.record()
+            self.step()
+            e1.record()
+        torch.cuda.synchronize()
+        t = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in ev)
+        pick = lambda q: round(t[min(len(t) - 1, int(q * len(t)))], 2)
+        return {"p10": pick(0.10), "p50": pick(0.50), "p90": pick(0.90)}
+
     def stage_times(self, reps=20):
         """Average duration of each kernel, HIP events on the launch stream around `reps`
         back-to-back launches of that kernel."""
@@ -288,6 +302,7 @@ def main():
         torch.cuda.synchronize()
     run = Runner(torch, 2, torch.float32)
     us = run.time_steps(args.steps, args.warmup)
+    pct = run.step_percentiles(max(args.steps, 20))
     stages = run.stage_times()
     work = stage_work(2)
     dom = max((k for k in stages if k in work), key=lambda k: stages[k])
@@ -325,6 +340,7 @@ def main():
         "config": {"workload": "configs[1]: B=8 L=1024 H=8 P=32 N=256 G=1 chunk=64, fwd+bwd, bidirectional pair "
                                "(fused), fp32 I/O, fp32 MFMA accumulate"},
         "roofline": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in roof.items()},
+        "step_us_percentiles": pct,
         "stages_us": {k: round(v, 2) for k, v in stages.items()},
         "stage_roofline": per_stage,
         "variants_us": variants,

@@ -49,6 +49,171 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd(NormP p) {
   }
 }
 
+// ---- fast paths: one group per row, ncols a multiple of 4 and at most 1024 ---------------------------------
+// A lane owns vectors lane, lane + 64, ... of 4 consecutive columns; the row stays in registers between the
+// reduction and the second use, loads and stores are as wide as each tensor's row alignment allows (8 bytes for
+// bf16, 16 for fp32 when aligned), and the backward keeps its dw partial in registers instead of
+// read-modify-writing LDS.
+// `al` (uniform per tensor): 0 = the 4 elements are aligned for one load, 1 = for two half loads, 2 = element loads
+template <bool BF>
+__device__ __forceinline__ f4 ld4(const void* p, long off, bool ok, int al) {
+  f4 r = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (!ok) return r;
+  if (BF) {
+    const uint16_t* q = (const uint16_t*)p + off;
+    uint2 w;
+    if (al == 0) w = *(const uint2*)q;
+    else if (al == 1) w = make_uint2(*(const unsigned*)q, *(const unsigned*)(q + 2));
+    else w = make_uint2((unsigned)q[0] | ((unsigned)q[1] << 16), (unsigned)q[2] | ((unsigned)q[3] << 16));
+    r.x = __uint_as_float(w.x << 16); r.y = __uint_as_float(w.x & 0xffff0000u);
+    r.z = __uint_as_float(w.y << 16); r.w = __uint_as_float(w.y & 0xffff0000u);
+  } else {
+    const float* q = (const float*)p + off;
+    if (al == 0) r = *(const f4*)q;
+    else if (al == 1) {
+      const float2 a = *(const float2*)q, b = *(const float2*)(q + 2);
+      r = (f4){a.x, a.y, b.x, b.y};
+    } else r = (f4){q[0], q[1], q[2], q[3]};
+  }
+  return r;
+}
+template <bool BF>
+__device__ __forceinline__ void st4(void* p, long off, f4 v, int al) {
+  if (BF) {
+    uint16_t* q = (uint16_t*)p + off;
+    const unsigned lo = pack_bf16(v.x, v.y), hi = pack_bf16(v.z, v.w);
+    if (al == 0) *(uint2*)q = make_uint2(lo, hi);
+    else if (al == 1) { *(unsigned*)q = lo; *(unsigned*)(q + 2) = hi; }
+    else { q[0] = (uint16_t)lo; q[1] = (uint16_t)(lo >> 16); q[2] = (uint16_t)hi; q[3] = (uint16_t)(hi >> 16); }
+  } else {
+    float* q = (float*)p + off;
+    if (al == 0) *(f4*)q = v;
+    else if (al == 1) { *(float2*)q = make_float2(v.x, v.y); *(float2*)(q + 2) = make_float2(v.z, v.w); }
+    else { q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w; }
+  }
+}
+// alignment class of rows starting at q with `stride` elements between them
+__device__ __forceinline__ int al_of(const void* q, long stride, bool bf) {
+  const uintptr_t a = (uintptr_t)q | ((uintptr_t)(stride < 0 ? -stride : stride) * (bf ? 2 : 4));
+  const uintptr_t full = bf ? 7 : 15;
+  return (a & full) == 0 ? 0 : ((a & (full >> 1)) == 0 ? 1 : 2);
+}
+__device__ __forceinline__ f4 silu4(f4 z, f4& sg) {
+  f4 g;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { sg[i] = sigmoidf_(z[i]); g[i] = z[i] * sg[i]; }
+  return g;
+}
+
+template <bool BF, int NV>
+__global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= p.rows) return;
+  const int nvec = p.ncols >> 2;
+  const int ax = al_of(p.x, p.xs, BF), az = al_of(p.z, p.zs, BF), ay = al_of(p.y, p.ys, BF);
+  f4 x[NV], gate[NV];
+  float ss = 0.0f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int vi = lane + 64 * v;
+    const bool ok = vi < nvec;
+    x[v] = ld4<BF>(p.x, row * p.xs + 4 * vi, ok, ax);
+    gate[v] = (f4){1.0f, 1.0f, 1.0f, 1.0f};
+    if (p.z) {
+      f4 sg;
+      gate[v] = silu4(ld4<BF>(p.z, row * p.zs + 4 * vi, ok, az), sg);
+      if (!p.nbg) x[v] *= gate[v];
+    }
+    ss += (x[v].x * x[v].x + x[v].y * x[v].y) + (x[v].z * x[v].z + x[v].w * x[v].w);
+  }
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)p.ncols + p.eps);
+  if (lane == 0 && p.rstd) p.rstd[row] = rstd;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int vi = lane + 64 * v;
+    if (vi < nvec) {
+      f4 w;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = ldv(p.w, 4 * vi + i, p.wdt);
+      f4 y = x[v] * rstd * w;
+      if (p.z && p.nbg) y *= gate[v];
+      st4<BF>(p.y, row * p.ys + 4 * vi, y, ay);
+    }
+  }
+}
+
+template <bool BF, int NV>
+__global__ __launch_bounds__(64) void k_rmsnorm_bwd_fast(NormP p) {
+  const int lane = threadIdx.x;
+  const int nvec = p.ncols >> 2;
+  const int ax = al_of(p.x, p.xs, BF), az = al_of(p.z, p.zs, BF), ady = al_of(p.dy, p.dys, BF);
+  const int adx = al_of(p.dx, p.dxs, BF), adz = al_of(p.dz, p.dzs, BF);
+  f4 w[NV], dwacc[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int vi = lane + 64 * v;
+    dwacc[v] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+    w[v] = dwacc[v];
+    if (vi < nvec) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[v][i] = ldv(p.w, 4 * vi + i, p.wdt);
+    }
+  }
+  for (long row = blockIdx.x; row < p.rows; row += p.nblocks) {
+    const float rstd = p.rstd[row];
+    f4 xo[NV], dyo[NV], z[NV], sg[NV], gate[NV];
+    float c1 = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int vi = lane + 64 * v;
+      const bool ok = vi < nvec;
+      xo[v] = ld4<BF>(p.x, row * p.xs + 4 * vi, ok, ax);
+      dyo[v] = ld4<BF>(p.dy, row * p.dys + 4 * vi, ok, ady);
+      gate[v] = (f4){1.0f, 1.0f, 1.0f, 1.0f};
+      if (p.z) {
+        z[v] = ld4<BF>(p.z, row * p.zs + 4 * vi, ok, az);
+        gate[v] = silu4(z[v], sg[v]);
+      }
+      const f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+      const f4 d = (p.z && p.nbg) ? dyo[v] * gate[v] : dyo[v];
+      const f4 t = vv * rstd * d * w[v];
+      c1 += (t.x + t.y) + (t.z + t.w);
+    }
+    c1 = wave_sum(c1) / (float)p.ncols;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int vi = lane + 64 * v;
+      if (vi < nvec) {
+        const f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+        const f4 d = (p.z && p.nbg) ? dyo[v] * gate[v] : dyo[v];
+        const f4 xhat = vv * rstd;
+        f4 dxv = (w[v] * d - xhat * c1) * rstd;
+        dwacc[v] += d * xhat;
+        if (p.z) {
+          f4 dzv;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float ds = sg[v][i] * (1.0f + z[v][i] * (1.0f - sg[v][i]));  // d silu / dz
+            dzv[i] = p.nbg ? dyo[v][i] * (xhat[i] * w[v][i]) * ds : dxv[i] * xo[v][i] * ds;
+          }
+          if (!p.nbg) dxv *= gate[v];
+          if (p.dz) st4<BF>(p.dz, row * p.dzs + 4 * vi, dzv, adz);
+        }
+        st4<BF>(p.dx, row * p.dxs + 4 * vi, dxv, adx);
+      }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int vi = lane + 64 * v;
+    if (vi < nvec) *(f4*)(p.dw_partial + (long)blockIdx.x * p.ncols + 4 * vi) = dwacc[v];
+  }
+}
+
+static bool norm_fast_ok(const NormP& p) { return p.ngroups == 1 && (p.ncols & 3) == 0 && p.ncols <= 1024; }
+
 // One wavefront per block; block b walks rows b, b+nblocks, ... and keeps its dw partial in LDS.
 __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
   extern __shared__ float dws[];
@@ -101,43 +266,60 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
   for (int c = lane; c < p.ncols; c += 64) p.dw_partial[(long)blockIdx.x * p.ncols + c] = dws[c];
 }
 
-// dw[c] = sum over the per-block partials, in a fixed order: block = 32 columns x 8 row groups, row group g
-// adds partials g, g+8, ... with four independent accumulators, then the 8 group sums are combined in order.
+// dw[c] = sum over the per-block partials, in a fixed order: block = 8 columns x 32 row groups, row group g adds
+// partials g, g+32, ... with two independent accumulators, then the 32 group sums are combined in order.
 __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_dw(NormP p) {
   __shared__ float red[NTHREADS];
-  const int c = blockIdx.x * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
-  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  const int c = blockIdx.x * 8 + (threadIdx.x & 7), g = threadIdx.x >> 3;
+  float a0 = 0.0f, a1 = 0.0f;
   if (c < p.ncols) {
     int b = g;
-    for (; b + 24 < p.nblocks; b += 32) {
+    for (; b + 32 < p.nblocks; b += 64) {
       a0 += p.dw_partial[(long)b * p.ncols + c];
-      a1 += p.dw_partial[(long)(b + 8) * p.ncols + c];
-      a2 += p.dw_partial[(long)(b + 16) * p.ncols + c];
-      a3 += p.dw_partial[(long)(b + 24) * p.ncols + c];
+      a1 += p.dw_partial[(long)(b + 32) * p.ncols + c];
     }
-    for (; b < p.nblocks; b += 8) a0 += p.dw_partial[(long)b * p.ncols + c];
+    if (b < p.nblocks) a0 += p.dw_partial[(long)b * p.ncols + c];
   }
-  red[threadIdx.x] = (a0 + a1) + (a2 + a3);
+  red[threadIdx.x] = a0 + a1;
   __syncthreads();
   if (g == 0 && c < p.ncols) {
     float t = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) t += red[k * 32 + (threadIdx.x & 31)];
+    for (int k = 0; k < 32; ++k) t += red[k * 8 + (threadIdx.x & 7)];
     p.dw[c] = t;
   }
 }
 
+#define NORM_FAST(KERNEL, GRID, BLOCK)                                                            \
+  do {                                                                                           \
+    const int nv = (p.ncols / 4 + 63) / 64;                                                      \
+    if (p.dt) {                                                                                  \
+      if (nv <= 1) hipLaunchKernelGGL((KERNEL<true, 1>), GRID, BLOCK, 0, st, p);                 \
+      else if (nv == 2) hipLaunchKernelGGL((KERNEL<true, 2>), GRID, BLOCK, 0, st, p);            \
+      else hipLaunchKernelGGL((KERNEL<true, 4>), GRID, BLOCK, 0, st, p);                         \
+    } else {                                                                                     \
+      if (nv <= 1) hipLaunchKernelGGL((KERNEL<false, 1>), GRID, BLOCK, 0, st, p);                \
+      else if (nv == 2) hipLaunchKernelGGL((KERNEL<false, 2>), GRID, BLOCK, 0, st, p);           \
+      else hipLaunchKernelGGL((KERNEL<false, 4>), GRID, BLOCK, 0, st, p);                        \
+    }                                                                                            \
+  } while (0)
+
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st) {
+  if (norm_fast_ok(p)) {
+    NORM_FAST(k_rmsnorm_fwd_fast, dim3((unsigned)((p.rows + 3) / 4)), dim3(NTHREADS));
+    return (int)hipGetLastError();
+  }
   const long items = p.rows * p.ngroups;
   hipLaunchKernelGGL(k_rmsnorm_fwd, dim3((unsigned)((items + 3) / 4)), dim3(NTHREADS), 0, st, p);
   return (int)hipGetLastError();
 }
 
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st) {
-  hipLaunchKernelGGL(k_rmsnorm_bwd, dim3(p.nblocks), dim3(64), (size_t)p.ncols * sizeof(float), st, p);
+  if (norm_fast_ok(p)) NORM_FAST(k_rmsnorm_bwd_fast, dim3(p.nblocks), dim3(64));
+  else hipLaunchKernelGGL(k_rmsnorm_bwd, dim3(p.nblocks), dim3(64), (size_t)p.ncols * sizeof(float), st, p);
   int e = (int)hipGetLastError();
   if (e) return e;
-  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 31) / 32), dim3(NTHREADS), 0, st, p);
+  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 7) / 8), dim3(NTHREADS), 0, st, p);
   return (int)hipGetLastError();
 }
 
