@@ -103,6 +103,36 @@ class Runner:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e6
 
+    def capture(self):
+        """Record one step (forward + backward, 9 kernel launches, no allocation, no memset) into a HIP graph on a side
+        stream of default priority and return the graph."""
+        torch = self.torch
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        keep = self.a.stream
+        self.a.stream = side.cuda_stream
+        with torch.cuda.stream(side):
+            self.step()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            self.step()
+        self.a.stream = keep
+        torch.cuda.current_stream().wait_stream(side)
+        return graph
+
+    def time_graph_replays(self, steps, warmup):
+        torch = self.torch
+        graph = self.capture()
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e6
+
     def step_percentiles(self, steps):
         """p10 / p50 / p90 of single steps, each bracketed by HIP events on the launch stream (caches not flushed
         between steps: consecutive steps reuse the same buffers, as a training loop does)."""
@@ -323,6 +353,7 @@ def main():
                         "frac": round(rate / (PEAK_FP32_MFMA_TFLOPS * 1e12 if b == "mfma" else PEAK_HBM_GBS * 1e9), 4)}
     variants = {}
     if not args.no_variants:
+        variants["headline_as_hip_graph_replay"] = round(run.time_graph_replays(args.steps, 5), 2)
         for name, nd, dt, pdim in (("uni_fp32", 1, torch.float32, 32), ("uni_bf16", 1, torch.bfloat16, 32),
                                    ("bidir_bf16", 2, torch.bfloat16, 32),
                                    ("bidir_bf16_headdim36", 2, torch.bfloat16, 36)):  # the detector's head size
