@@ -15,159 +15,9 @@
 // table, then a sum of the per-workgroup copies.  The LDS copy is 64-bit fixed point (terms scaled by
 // 2^34 / max|ddist|, found by a first pass): LDS integer atomics run about twice as fast as ds_add_f32 here, and
 // integer sums do not depend on the order of the adds, so the gradient is reproducible bit for bit.
-#include "issm_dev.h"
+#include "box_dist_dev.h"
 
 namespace issm {
-
-constexpr int BD_C = 16;          // channels of the table
-constexpr int BD_MAXCELLS = 1024; // D * H * W nodes that fit the 64 KB LDS copy
-
-struct BoxLane {
-  float cx[8], cy[8], cz[8];  // corners of the lane's box
-  float cs[8], sn[8];         // rotation of flattened corner j = k * 8 + c: angle of query j mod K (as the reference)
-  float qx, qy, qz, radius;
-};
-
-__device__ __forceinline__ void load_box(const BoxDistP& p, int b, int k, BoxLane& bx) {
-  const float* c = p.corners + ((long)b * p.K + k) * 24;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    bx.cx[j] = c[3 * j];
-    bx.cy[j] = c[3 * j + 1];
-    bx.cz[j] = c[3 * j + 2];
-    bx.cs[j] = 1.0f;
-    bx.sn[j] = 0.0f;
-    if (p.angle) {  // uniform
-      const float a = p.angle[(long)b * p.K + (k * 8 + j) % p.K];
-      bx.cs[j] = cosf(a);
-      bx.sn[j] = sinf(a);
-    }
-  }
-  if (p.qcenter) {
-    const float* q = p.qcenter + ((long)b * p.K + k) * 3;
-    bx.qx = q[0]; bx.qy = q[1]; bx.qz = q[2];
-    bx.radius = p.radius[(long)b * p.K + k];
-  }
-}
-
-// corner slot j takes the values of slot j + 1, slot 7 those of slot 0 (after 8 calls the box is as it was)
-__device__ __forceinline__ void rotate_box(BoxLane& bx) {
-  const float x0 = bx.cx[0], y0 = bx.cy[0], z0 = bx.cz[0], c0 = bx.cs[0], s0 = bx.sn[0];
-#pragma unroll
-  for (int j = 0; j < 7; ++j) {
-    bx.cx[j] = bx.cx[j + 1]; bx.cy[j] = bx.cy[j + 1]; bx.cz[j] = bx.cz[j + 1];
-    bx.cs[j] = bx.cs[j + 1]; bx.sn[j] = bx.sn[j + 1];
-  }
-  bx.cx[7] = x0; bx.cy[7] = y0; bx.cz[7] = z0; bx.cs[7] = c0; bx.sn[7] = s0;
-}
-
-// signed log compression and grid_sample's un-normalisation (align_corners False) in one: position in node units
-__device__ __forceinline__ float node_pos(float v, float log_scale, float scale, int n) {
-  const float m = __log2f(fabsf(v) * log_scale + 1.0f) * scale;  // scale = 1 / (log2(8) * max_value)
-  const float g = v < 0.0f ? -m : m;
-  return (g + 1.0f) * (0.5f * n) - 0.5f;
-}
-
-// The 8 neighbours of one sampling position: LDS offset (in floats) of the node and its weight (0 outside).
-struct Tri {
-  int off[8];
-  float w[8];
-};
-__device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, float z, Tri& t) {
-  const float fx = floorf(x), fy = floorf(y), fz = floorf(z);
-  const float ax = x - fx, ay = y - fy, az = z - fz;
-  const int ix = (int)fx, iy = (int)fy, iz = (int)fz;
-#pragma unroll
-  for (int n = 0; n < 8; ++n) {
-    const int dx = n & 1, dy = (n >> 1) & 1, dz = n >> 2;
-    const int jx = ix + dx, jy = iy + dy, jz = iz + dz;
-    const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
-    const float w = (dx ? ax : 1.0f - ax) * (dy ? ay : 1.0f - ay) * (dz ? az : 1.0f - az);
-    t.w[n] = ok ? w : 0.0f;
-    t.off[n] = ok ? ((jz * p.H + jy) * p.W + jx) * BD_C : 0;
-  }
-}
-
-// The 8 corners of a box usually fall into the same or adjacent table cells (a box is small next to the spacing
-// of the log-compressed lattice), so their 8 x 8 node weights are first merged, in registers, over a 3 x 3 x 3 window
-// of nodes anchored at the smallest base node: up to 27 -- typically 8 to 12 non-zero -- table accesses per
-// (point, box) pair instead of 64.  Possible when the corners' base nodes differ by at most one along every axis;
-// otherwise the caller walks the corners one by one.
-struct Window {
-  int mx, my, mz;
-  float w[27];  // [dz][dy][dx]
-};
-__device__ __forceinline__ bool corner_window(const BoxDistP& p, const BoxLane& bx, float kx, float ky, float kz,
-                                              float scale, Window& win) {
-  float fx[8], fy[8], fz[8];
-  int ix[8], iy[8], iz[8];
-#pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    const float dx = bx.cx[c] - kx, dy = bx.cy[c] - ky, dz = bx.cz[c] - kz;
-    const float rx = dx * bx.cs[c] - dy * bx.sn[c], ry = dx * bx.sn[c] + dy * bx.cs[c];
-    const float x = node_pos(rx, p.log_scale, scale, p.W), y = node_pos(ry, p.log_scale, scale, p.H),
-                z = node_pos(dz, p.log_scale, scale, p.D);
-    const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
-    fx[c] = x - gx; fy[c] = y - gy; fz[c] = z - gz;
-    ix[c] = (int)gx; iy[c] = (int)gy; iz[c] = (int)gz;
-  }
-  int mx = ix[0], my = iy[0], mz = iz[0], Mx = ix[0], My = iy[0], Mz = iz[0];
-#pragma unroll
-  for (int c = 1; c < 8; ++c) {
-    mx = min(mx, ix[c]); Mx = max(Mx, ix[c]);
-    my = min(my, iy[c]); My = max(My, iy[c]);
-    mz = min(mz, iz[c]); Mz = max(Mz, iz[c]);
-  }
-  if (Mx - mx > 1 || My - my > 1 || Mz - mz > 1) return false;
-  win.mx = mx; win.my = my; win.mz = mz;
-#pragma unroll
-  for (int e = 0; e < 27; ++e) win.w[e] = 0.0f;
-#pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    const bool sx = ix[c] != mx, sy = iy[c] != my, sz = iz[c] != mz;
-    const float ax[3] = {sx ? 0.0f : 1.0f - fx[c], sx ? 1.0f - fx[c] : fx[c], sx ? fx[c] : 0.0f};
-    const float ay[3] = {sy ? 0.0f : 1.0f - fy[c], sy ? 1.0f - fy[c] : fy[c], sy ? fy[c] : 0.0f};
-    const float az[3] = {sz ? 0.0f : 1.0f - fz[c], sz ? 1.0f - fz[c] : fz[c], sz ? fz[c] : 0.0f};
-#pragma unroll
-    for (int i = 0; i < 3; ++i)
-#pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        const float yx = ay[i] * ax[j];
-#pragma unroll
-        for (int k = 0; k < 3; ++k) win.w[k * 9 + i * 3 + j] = fmaf(az[k], yx, win.w[k * 9 + i * 3 + j]);
-      }
-  }
-  return true;
-}
-// visit the window's nodes that lie inside the table and carry weight: f(LDS offset in floats, weight)
-template <class F>
-__device__ __forceinline__ void for_window(const BoxDistP& p, const Window& win, F f) {
-#pragma unroll
-  for (int k = 0; k < 3; ++k)
-#pragma unroll
-    for (int i = 0; i < 3; ++i)
-#pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        const int jx = win.mx + j, jy = win.my + i, jz = win.mz + k;
-        const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
-        const float w = win.w[k * 9 + i * 3 + j];
-        if (ok && w != 0.0f) f(((jz * p.H + jy) * p.W + jx) * BD_C, w);
-      }
-}
-
-// work split: items = (b, k chunk of 256, l), l fastest; workgroup w takes a contiguous range
-struct Items {
-  long i0, i1;
-  int kchunks;
-};
-__device__ __forceinline__ Items my_items(const BoxDistP& p) {
-  Items it;
-  it.kchunks = (p.K + NTHREADS - 1) / NTHREADS;
-  const long n = (long)p.B * it.kchunks * p.L;
-  it.i0 = n * blockIdx.x / gridDim.x;
-  it.i1 = n * (blockIdx.x + 1) / gridDim.x;
-  return it;
-}
 
 template <bool BF>
 __global__ __launch_bounds__(NTHREADS) void k_box_dist_fwd(BoxDistP p) {
@@ -244,15 +94,6 @@ __global__ __launch_bounds__(NTHREADS) void k_box_dist_fwd(BoxDistP p) {
       p.weights[o] = __expf(p.weight_dist * fminf(bx.radius - d, 0.0f));
     }
   }
-}
-
-// Fixed-point scale of the table gradient.  A pair's node weights sum to 8 (one per corner), so a node of one
-// workgroup's copy collects at most 8 * pairs-per-workgroup * max|ddist|; with 2^34 / max|ddist| that stays below
-// 2^63 for 2^26 pairs per workgroup, and the sum over all workgroups is taken in 64 bits as well (2^26 pairs in total
-// is the bound the launcher checks).
-__device__ __forceinline__ float bd_scale(const unsigned* scal) {
-  const float gmax = __uint_as_float(scal[0]);
-  return gmax > 0.0f ? 17179869184.0f / gmax : 1.0f;
 }
 
 __global__ void k_box_dist_clear(unsigned* scal) { scal[0] = 0u; }
@@ -399,7 +240,21 @@ int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+int launch_box_dist_bwd_sorted(const BoxDistP& p, hipStream_t st);
+long box_dist_sorted_scratch_bytes(int B, int L, int K, int D, int H, int W);
+
+// few pairs: scatter with LDS atomics (one launch of work); many pairs: sort by window, then dense sums
+constexpr long BD_SORT_MIN_PAIRS = 1 << 16;
+
+long box_dist_bwd_scratch_bytes(int B, int L, int K, int D, int H, int W) {
+  const long atomic_path = 16 + (long)box_dist_bwd_workgroups(B, L, K) * D * H * W * BD_C * 8;
+  if ((long)B * L * K < BD_SORT_MIN_PAIRS) return atomic_path;
+  const long sorted_path = box_dist_sorted_scratch_bytes(B, L, K, D, H, W);
+  return sorted_path > atomic_path ? sorted_path : atomic_path;
+}
+
 int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st) {
+  if ((long)p.B * p.L * p.K >= BD_SORT_MIN_PAIRS) return launch_box_dist_bwd_sorted(p, st);
   const dim3 g(p.nwg_bwd), b(NTHREADS);
   unsigned* scal = (unsigned*)p.partial;
   hipLaunchKernelGGL(k_box_dist_clear, dim3(1), dim3(1), 0, st, scal);

@@ -1,0 +1,389 @@
+// Table gradient of the box-to-point distance encoding without a scatter (gfx950).
+//
+// dtable[node][ch] = sum over (point, box) pairs of weight[pair][node] * ddist[pair][ch].  Scattering that into an
+// LDS copy of the table is bound by the LDS atomic rate (about one add per three cycles per CU).  Here the pairs are
+// first sorted by where they land: a pair contributes one *entry* per window of 3 x 3 x 3 nodes it touches (one if
+// its corners are on one side of the point, two if it straddles the point along one axis, ...), entries are binned
+// by window anchor with a counting sort, and then all entries of a bin share their 27 nodes, so the gradient of a
+// bin is a dense (27 x entries) . (entries x 16) product accumulated in registers.  Passes:
+//   count   workgroup histograms of the entries' bins (LDS integer atomics, one per entry)
+//   plan    bin offsets and the list of work items (bin, range of at most BDS_SEG entries); then each counting
+//           workgroup's base inside each bin (a scan over workgroups, so the ranges do not depend on timing)
+//   fill    the same walk again, writing each entry's record (pair index, corner mask) into its bin
+//   accum   one workgroup per work item: 256 entries at a time, lane = entry recomputes the window weights of its
+//           corners and stages them with ddist in LDS; then thread = (node of the window, channel) adds
+//           weight * ddist over the entries, in 64-bit fixed point (order-independent, hence reproducible)
+//   scatter / finish   work-item results into the table (integer atomics in global memory, a few 10^5), then float.
+#include "box_dist_dev.h"
+
+namespace issm {
+
+constexpr int BDS_SEG = 2048;      // entries per work item
+constexpr int BDS_MAXBINS = 9280;  // (D + 2)(H + 2)(W + 2) for D*H*W <= 1024 is at most 1026 * 3 * 3
+constexpr int BDS_NWG = 512;       // workgroups of the count and fill passes (they must walk identically)
+constexpr int BDS_OUT = 27 * BD_C; // results per work item
+
+struct SortP {
+  unsigned* scal;               // [0] bits of max|ddist|, [1] number of work items
+  int* counts;                  // [nbins] entries per bin
+  int* binoff;                  // [nbins] first entry of each bin
+  int* wgbase;                  // [BDS_NWG][nbins] counts per workgroup, turned into base positions by the plan
+  int* items;                   // [maxitems][3] bin, first entry, one past the last entry
+  unsigned long long* records;  // [maxrecords] pair index | corner mask << 32
+  long long* item_out;          // [maxitems][BDS_OUT]
+  long long* dtab;              // [cells][16]
+  int nbins, maxitems;
+  long maxrecords;
+};
+
+// Fixed-point scale: a term weight * ddist is at most 8 max|ddist|, so with 2^27 / max|ddist| it converts to a 32-bit
+// integer (one instruction); the sums are kept in 64 bits (2^26 pairs * 8 * 2^27 < 2^63).
+__device__ __forceinline__ float bds_scale(const unsigned* scal) {
+  const float gmax = __uint_as_float(scal[0]);
+  return gmax > 0.0f ? 134217728.0f / gmax : 1.0f;
+}
+
+__device__ __forceinline__ int bds_bin(const BoxDistP& p, int mx, int my, int mz) {
+  if (mx < -2 || mx > p.W - 1 || my < -2 || my > p.H - 1 || mz < -2 || mz > p.D - 1) return -1;  // no node inside
+  return ((mz + 2) * (p.H + 2) + (my + 2)) * (p.W + 2) + (mx + 2);
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_clear(BoxDistP p, SortP s) {
+  const int cells = p.D * p.H * p.W;
+  const int i = blockIdx.x * NTHREADS + threadIdx.x;
+  if (i < 4) s.scal[i] = 0u;
+  if (i < s.nbins) s.counts[i] = 0;
+  if (i < cells * BD_C) s.dtab[i] = 0;
+}
+
+// The walk shared by count and fill: thread = (b, l, k) as in the forward, f(bin, pair index, corner mask).
+template <class F>
+__device__ __forceinline__ void bds_walk(const BoxDistP& p, F f) {
+  const Items it = my_items(p);
+  const float scale = 1.0f / (3.0f * p.max_value);
+  BoxLane bx;
+  long cur = -1;
+  for (long item = it.i0; item < it.i1; ++item) {
+    const int l = (int)(item % p.L);
+    const long bk = item / p.L;
+    const int b = (int)(bk / it.kchunks), k = (int)(bk % it.kchunks) * NTHREADS + threadIdx.x;
+    if (k >= p.K) continue;
+    if (bk != cur) {
+      load_box(p, b, k, bx);
+      cur = bk;
+    }
+    const float* key = p.key + ((long)b * p.L + l) * 3;
+    CornerGrid cg;
+    corner_grid(p, bx, key[0], key[1], key[2], scale, cg);
+    const unsigned pid = (unsigned)(((long)b * p.L + l) * p.K + k);
+    for_entries(cg, [&](int mx, int my, int mz, unsigned mask) {
+      const int bin = bds_bin(p, mx, my, mz);
+      if (bin >= 0) f(bin, pid, mask);
+    });
+  }
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_count(BoxDistP p, SortP s) {
+  __shared__ int hist[BDS_MAXBINS];
+  for (int e = threadIdx.x; e < s.nbins; e += NTHREADS) hist[e] = 0;
+  __syncthreads();
+  bds_walk(p, [&](int bin, unsigned, unsigned) { atomicAdd(&hist[bin], 1); });
+  __syncthreads();
+  for (int e = threadIdx.x; e < s.nbins; e += NTHREADS) {
+    const int c = hist[e];
+    s.wgbase[(long)blockIdx.x * s.nbins + e] = c;
+    if (c) atomicAdd(&s.counts[e], c);
+  }
+}
+
+// exclusive scan of v[0..n) into out (one workgroup; v and out may alias); returns the total to every thread
+__device__ int bds_scan(const int* v, int* out, int n, int* part) {
+  const int per = (n + NTHREADS - 1) / NTHREADS;
+  const int e0 = min(threadIdx.x * per, n), e1 = min(e0 + per, n);
+  int sum = 0;
+  for (int e = e0; e < e1; ++e) sum += v[e];
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int t = 0; t < NTHREADS; ++t) {
+      const int c = part[t];
+      part[t] = run;
+      run += c;
+    }
+    part[NTHREADS] = run;
+  }
+  __syncthreads();
+  int run = part[threadIdx.x];
+  for (int e = e0; e < e1; ++e) {
+    const int c = v[e];
+    out[e] = run;
+    run += c;
+  }
+  const int total = part[NTHREADS];
+  __syncthreads();
+  return total;
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_plan(SortP s) {
+  __shared__ int off[BDS_MAXBINS];
+  __shared__ int ibase[BDS_MAXBINS];
+  __shared__ int part[NTHREADS + 1];
+  bds_scan(s.counts, off, s.nbins, part);
+  for (int e = threadIdx.x; e < s.nbins; e += NTHREADS) {
+    s.binoff[e] = off[e];
+    ibase[e] = (s.counts[e] + BDS_SEG - 1) / BDS_SEG;
+  }
+  __syncthreads();
+  // work items: ranges of at most BDS_SEG entries of one bin
+  const int nitems = bds_scan(ibase, ibase, s.nbins, part);
+  for (int e = threadIdx.x; e < s.nbins; e += NTHREADS) {
+    const int c = s.counts[e], first = off[e];
+    int it = ibase[e];
+    for (int a = 0; a < c; a += BDS_SEG, ++it) {
+      if (it < s.maxitems) {
+        s.items[3 * it] = e;
+        s.items[3 * it + 1] = first + a;
+        s.items[3 * it + 2] = first + min(a + BDS_SEG, c);
+      }
+    }
+  }
+  if (threadIdx.x == 0) s.scal[1] = (unsigned)min(nitems, s.maxitems);
+}
+
+// Base position of every counting workgroup inside every bin: a running sum over the workgroups, in order (thread
+// = bin; 16 loads in flight at a time).
+__global__ __launch_bounds__(64) void k_bds_wgbase(SortP s) {
+  const int e = blockIdx.x * 64 + threadIdx.x;
+  if (e >= s.nbins) return;
+  int run = s.binoff[e];
+  for (int w0 = 0; w0 < BDS_NWG; w0 += 16) {
+    int c[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) c[j] = s.wgbase[(long)(w0 + j) * s.nbins + e];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      s.wgbase[(long)(w0 + j) * s.nbins + e] = run;
+      run += c[j];
+    }
+  }
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_fill(BoxDistP p, SortP s) {
+  __shared__ int cur[BDS_MAXBINS];
+  for (int e = threadIdx.x; e < s.nbins; e += NTHREADS) cur[e] = s.wgbase[(long)blockIdx.x * s.nbins + e];
+  __syncthreads();
+  bds_walk(p, [&](int bin, unsigned pid, unsigned mask) {
+    const int pos = atomicAdd(&cur[bin], 1);
+    if (pos >= 0 && pos < s.maxrecords) s.records[pos] = (unsigned long long)pid | ((unsigned long long)mask << 32);
+  });
+}
+
+// weights of one axis over the window's three nodes: the corner's base node is `i`, its fraction `f`, the window
+// starts at `m`.  A base node outside [m, m + 1] can only come from a position within rounding of a node, where the
+// weight it would carry is ~0: such parts are dropped.
+__device__ __forceinline__ void axis3(int i, float f, int m, float (&a)[3]) {
+  const int s0 = i - m;
+#pragma unroll
+  for (int j = 0; j < 3; ++j) a[j] = (s0 == j ? 1.0f - f : 0.0f) + (s0 + 1 == j ? f : 0.0f);
+}
+
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
+  __shared__ float Wl[NTHREADS][27];  // odd row length: the lanes' rows start in different banks
+  __shared__ __attribute__((aligned(16))) float Gl[NTHREADS][BD_C];
+  const int item = blockIdx.x;
+  if (item >= (int)s.scal[1]) return;  // uniform
+  const int bin = s.items[3 * item], first = s.items[3 * item + 1], last = s.items[3 * item + 2];
+  const int mx = bin % (p.W + 2) - 2, my = (bin / (p.W + 2)) % (p.H + 2) - 2, mz = bin / ((p.W + 2) * (p.H + 2)) - 2;
+  const float scale = 1.0f / (3.0f * p.max_value);
+  const float fx_scale = bds_scale(s.scal);
+  const int t0 = threadIdx.x, t1 = threadIdx.x + NTHREADS;  // the thread's (node, channel) results
+  const int slot0 = t0 >> 4, slot1 = t1 >> 4, ch = t0 & 15;
+  const bool has1 = t1 < BDS_OUT;
+  long long acc0 = 0, acc1 = 0;
+  for (int base = first; base < last; base += NTHREADS) {
+    const int e = base + threadIdx.x;
+    float w[27];
+#pragma unroll
+    for (int j = 0; j < 27; ++j) w[j] = 0.0f;
+    f4 g[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) g[j] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+    if (e < last) {
+      const unsigned long long rec = s.records[e];
+      unsigned pid = (unsigned)rec, mask = (unsigned)(rec >> 32);
+      if (pid >= (unsigned)((long)p.B * p.L * p.K) || mask > 255u) { pid = 0u; mask = 0u; }  // never index with a stray record
+      const int k = (int)(pid % (unsigned)p.K);
+      const unsigned bl = pid / (unsigned)p.K;
+      const int l = (int)(bl % (unsigned)p.L), b = (int)(bl / (unsigned)p.L);
+      const float* key = p.key + ((long)b * p.L + l) * 3;
+      const float kx = key[0], ky = key[1], kz = key[2];
+      const float* cor = p.corners + ((long)b * p.K + k) * 24;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (mask & (1u << c)) {
+          float cs = 1.0f, sn = 0.0f;
+          if (p.angle) {  // uniform
+            const float a = p.angle[(long)b * p.K + (k * 8 + c) % p.K];
+            cs = cosf(a);
+            sn = sinf(a);
+          }
+          float x, y, z;
+          corner_pos(p, cor[3 * c], cor[3 * c + 1], cor[3 * c + 2], cs, sn, kx, ky, kz, scale, x, y, z);
+          const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
+          float ax[3], ay[3], az[3];
+          axis3((int)gx, x - gx, mx, ax);
+          axis3((int)gy, y - gy, my, ay);
+          axis3((int)gz, z - gz, mz, az);
+#pragma unroll
+          for (int i = 0; i < 3; ++i)
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+              const float yx = ay[i] * ax[j];
+#pragma unroll
+              for (int kk = 0; kk < 3; ++kk) w[kk * 9 + i * 3 + j] = fmaf(az[kk], yx, w[kk * 9 + i * 3 + j]);
+            }
+        }
+      }
+      if (BF) {
+        const uint4* src = (const uint4*)((const uint16_t*)p.ddist + (long)pid * BD_C);
+        const uint4 a = src[0], c = src[1];
+        g[0] = (f4){__uint_as_float(a.x << 16), __uint_as_float(a.x & 0xffff0000u), __uint_as_float(a.y << 16),
+                    __uint_as_float(a.y & 0xffff0000u)};
+        g[1] = (f4){__uint_as_float(a.z << 16), __uint_as_float(a.z & 0xffff0000u), __uint_as_float(a.w << 16),
+                    __uint_as_float(a.w & 0xffff0000u)};
+        g[2] = (f4){__uint_as_float(c.x << 16), __uint_as_float(c.x & 0xffff0000u), __uint_as_float(c.y << 16),
+                    __uint_as_float(c.y & 0xffff0000u)};
+        g[3] = (f4){__uint_as_float(c.z << 16), __uint_as_float(c.z & 0xffff0000u), __uint_as_float(c.w << 16),
+                    __uint_as_float(c.w & 0xffff0000u)};
+      } else {
+        const f4* src = (const f4*)((const float*)p.ddist + (long)pid * BD_C);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) g[j] = src[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 27; ++j) Wl[threadIdx.x][j] = w[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *(f4*)&Gl[threadIdx.x][4 * j] = g[j] * fx_scale;
+    __syncthreads();
+    const int nb = min(NTHREADS, last - base);  // rows nb .. 255 hold zeros: the loop may run past nb in steps of 4
+#pragma unroll 4
+    for (int ee = 0; ee < ((nb + 3) & ~3); ++ee) {
+      const float gv = Gl[ee][ch];
+      acc0 += (long long)__float2int_rn(Wl[ee][slot0] * gv);  // |weight * ddist * scale| <= 8 * 2^27: fits 32 bits
+      if (has1) acc1 += (long long)__float2int_rn(Wl[ee][slot1] * gv);
+    }
+    __syncthreads();
+  }
+  s.item_out[(long)item * BDS_OUT + t0] = acc0;
+  if (has1) s.item_out[(long)item * BDS_OUT + t1] = acc1;
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_scatter(BoxDistP p, SortP s) {
+  const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  const int item = (int)(id / BDS_OUT);
+  if (item >= (int)s.scal[1]) return;
+  const int r = (int)(id % BDS_OUT), slot = r >> 4, ch = r & 15;
+  const int bin = s.items[3 * item];
+  const int jx = bin % (p.W + 2) - 2 + slot % 3, jy = (bin / (p.W + 2)) % (p.H + 2) - 2 + (slot / 3) % 3,
+            jz = bin / ((p.W + 2) * (p.H + 2)) - 2 + slot / 9;
+  if (jx < 0 || jx >= p.W || jy < 0 || jy >= p.H || jz < 0 || jz >= p.D) return;
+  const long long v = s.item_out[id];
+  if (v != 0) atomicAdd((unsigned long long*)&s.dtab[((long)(jz * p.H + jy) * p.W + jx) * BD_C + ch], (unsigned long long)v);
+}
+
+__global__ __launch_bounds__(NTHREADS) void k_bds_finish(BoxDistP p, SortP s) {
+  const int cells = p.D * p.H * p.W;
+  const int e = blockIdx.x * NTHREADS + threadIdx.x;  // e = cell * 16 + ch
+  if (e >= cells * BD_C) return;
+  p.dtable[(long)(e % BD_C) * cells + e / BD_C] = (float)((double)s.dtab[e] / (double)bds_scale(s.scal));
+}
+
+template <bool BF>
+__global__ __launch_bounds__(NTHREADS) void k_bds_gmax(BoxDistP p, unsigned* scal) {
+  const long n = (long)p.B * p.L * p.K * BD_C;
+  float m = 0.0f;
+  for (long e = ((long)blockIdx.x * NTHREADS + threadIdx.x) * 8; e < n; e += (long)gridDim.x * NTHREADS * 8) {
+    if (BF) {
+      const uint4 v = *(const uint4*)((const uint16_t*)p.ddist + e);
+      const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        m = fmaxf(m, fmaxf(fabsf(__uint_as_float(w[j] << 16)), fabsf(__uint_as_float(w[j] & 0xffff0000u))));
+    } else {
+      const f4 a = *(const f4*)((const float*)p.ddist + e), c = *(const f4*)((const float*)p.ddist + e + 4);
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0 && m > 0.0f && m == m) atomicMax(scal, __float_as_uint(m));
+}
+
+static long bds_align(long v) { return (v + 15) & ~15L; }
+
+struct BdsLayout {
+  long scal, counts, binoff, wgbase, items, records, item_out, dtab, total;
+  int nbins, maxitems;
+  long maxrecords;
+};
+static BdsLayout bds_layout(int B, int L, int K, int D, int H, int W) {
+  BdsLayout y;
+  const long pairs = (long)B * L * K, maxrec = pairs * 8;
+  y.nbins = (D + 2) * (H + 2) * (W + 2);
+  y.maxitems = (int)(y.nbins + maxrec / BDS_SEG + 1);
+  long o = 0;
+  y.scal = o; o = bds_align(o + 16);
+  y.counts = o; o = bds_align(o + (long)y.nbins * 4);
+  y.binoff = o; o = bds_align(o + (long)y.nbins * 4);
+  y.wgbase = o; o = bds_align(o + (long)BDS_NWG * y.nbins * 4);
+  y.items = o; o = bds_align(o + (long)y.maxitems * 12);
+  y.records = o; o = bds_align(o + maxrec * 8);
+  y.item_out = o; o = bds_align(o + (long)y.maxitems * BDS_OUT * 8);
+  y.dtab = o; o = bds_align(o + (long)D * H * W * BD_C * 8);
+  y.total = o;
+  return y;
+}
+
+long box_dist_sorted_scratch_bytes(int B, int L, int K, int D, int H, int W) { return bds_layout(B, L, K, D, H, W).total; }
+
+int launch_box_dist_bwd_sorted(const BoxDistP& p, hipStream_t st) {
+  const BdsLayout y = bds_layout(p.B, p.L, p.K, p.D, p.H, p.W);
+  if (y.nbins > BDS_MAXBINS) return (int)hipErrorInvalidValue;
+  char* base = (char*)p.partial;
+  SortP s;
+  s.scal = (unsigned*)(base + y.scal);
+  s.counts = (int*)(base + y.counts);
+  s.binoff = (int*)(base + y.binoff);
+  s.wgbase = (int*)(base + y.wgbase);
+  s.items = (int*)(base + y.items);
+  s.records = (unsigned long long*)(base + y.records);
+  s.item_out = (long long*)(base + y.item_out);
+  s.dtab = (long long*)(base + y.dtab);
+  s.nbins = y.nbins;
+  s.maxitems = y.maxitems;
+  s.maxrecords = (long)p.B * p.L * p.K * 8;
+  const dim3 b(NTHREADS);
+  const int cells16 = p.D * p.H * p.W * BD_C;
+  const int nclear = cells16 > y.nbins ? cells16 : y.nbins;
+  hipLaunchKernelGGL(k_bds_clear, dim3((nclear + NTHREADS - 1) / NTHREADS), b, 0, st, p, s);
+  if (p.dtype) hipLaunchKernelGGL(k_bds_gmax<true>, dim3(512), b, 0, st, p, s.scal);
+  else hipLaunchKernelGGL(k_bds_gmax<false>, dim3(512), b, 0, st, p, s.scal);
+  hipLaunchKernelGGL(k_bds_count, dim3(BDS_NWG), b, 0, st, p, s);
+  hipLaunchKernelGGL(k_bds_plan, dim3(1), b, 0, st, s);
+  hipLaunchKernelGGL(k_bds_wgbase, dim3((y.nbins + 63) / 64), dim3(64), 0, st, s);
+  hipLaunchKernelGGL(k_bds_fill, dim3(BDS_NWG), b, 0, st, p, s);
+  int e = (int)hipGetLastError();
+  if (e) return e;
+  if (p.dtype) hipLaunchKernelGGL(k_bds_accum<true>, dim3(y.maxitems), b, 0, st, p, s);
+  else hipLaunchKernelGGL(k_bds_accum<false>, dim3(y.maxitems), b, 0, st, p, s);
+  const long nscat = (long)y.maxitems * BDS_OUT;
+  hipLaunchKernelGGL(k_bds_scatter, dim3((unsigned)((nscat + NTHREADS - 1) / NTHREADS)), b, 0, st, p, s);
+  hipLaunchKernelGGL(k_bds_finish, dim3((cells16 + NTHREADS - 1) / NTHREADS), b, 0, st, p, s);
+  return (int)hipGetLastError();
+}
+
+}  // namespace issm

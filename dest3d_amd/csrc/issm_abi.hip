@@ -27,6 +27,7 @@ int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
 int box_dist_workgroups(int B, int L, int K);
 int box_dist_bwd_workgroups(int B, int L, int K);
+long box_dist_bwd_scratch_bytes(int B, int L, int K, int D, int H, int W);
 int launch_box_dist_fwd(const BoxDistP& p, hipStream_t st);
 int launch_box_dist_bwd(const BoxDistP& p, hipStream_t st);
 int dwconv_partial_rows(int B, int L);
@@ -519,7 +520,7 @@ static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
 
 int64_t issm_box_dist_bwd_scratch_bytes(int32_t batch, int32_t seqlen, int32_t nquery, int32_t D, int32_t H, int32_t W) {
   if (batch <= 0 || seqlen <= 0 || nquery <= 0 || D <= 0 || H <= 0 || W <= 0) return 16;
-  return 16 + (int64_t)box_dist_bwd_workgroups(batch, seqlen, nquery) * D * H * W * 16 * 8;
+  return box_dist_bwd_scratch_bytes(batch, seqlen, nquery, D, H, W);
 }
 
 int issm_box_dist_fwd(const issm_box_dist_args* a) {
