@@ -252,6 +252,9 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
         return bd(key_pos, query_pos[..., :3], query_pos[..., 3:], zero_angle, weight_query_pos=query_pos)
 
     def step():
+        for mod in (m, bd):
+            mod.zero_grad(set_to_none=True)   # as an optimizer step would: no accumulation into old gradients
+        key.grad = query.grad = None
         dist, weights = encode()
         ok, oq = m(key, query, dist, key_pos, weights)
         (ok.float().square().mean() + oq.float().square().mean()).backward()
@@ -283,6 +286,8 @@ def time_module_layer(torch, steps=10, warmup=3):
     weights = torch.exp(-15.0 * (torch.rand(8, 1024, 256, device="cuda") - 0.5).clamp_min(0.0))
 
     def step():
+        m.zero_grad(set_to_none=True)   # as an optimizer step would: no accumulation into old gradients
+        key.grad = query.grad = dist.grad = None
         ok, oq = m(key, query, dist, None, weights)
         (ok.float().square().mean() + oq.float().square().mean()).backward()
 
