@@ -272,17 +272,18 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
     return out
 
 
-def time_module_layer(torch, steps=10, warmup=3):
+def time_module_layer(torch, steps=10, warmup=3, dtype=None):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
-    keys, batch 8, d_dist 16, bf16, float locality weights as mask -- what DEST's decoder layer passes,
+    keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
     models/dest_module.py:283-290), forward + backward through autograd, microseconds.  Includes the PyTorch
     projections and norms around the scan."""
     from dest3d_amd.scan_module import MultiHeadISSMScan
     torch.manual_seed(0)
-    m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1).cuda().bfloat16()
-    key = torch.randn(8, 1024, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
-    query = torch.randn(8, 256, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
-    dist = (0.5 * torch.randn(8, 1024, 256, 16, device="cuda")).bfloat16().requires_grad_()
+    dtype = dtype or torch.bfloat16
+    m = MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8, expand=1).cuda().to(dtype)
+    key = torch.randn(8, 1024, 288, device="cuda", dtype=dtype, requires_grad=True)
+    query = torch.randn(8, 256, 288, device="cuda", dtype=dtype, requires_grad=True)
+    dist = (0.5 * torch.randn(8, 1024, 256, 16, device="cuda")).to(dtype).requires_grad_()
     weights = torch.exp(-15.0 * (torch.rand(8, 1024, 256, device="cuda") - 0.5).clamp_min(0.0))
 
     def step():
@@ -368,6 +369,7 @@ def main():
             del r
         SHAPE["P"] = 32
         variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
+        variants["detector_layer_fp32_fwd_bwd"] = round(time_module_layer(torch, dtype=torch.float32), 2)
         variants["box_dist_plus_layer_bf16_fwd_bwd"] = round(time_box_dist_layer(torch)[0], 2)
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
