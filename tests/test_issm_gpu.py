@@ -491,3 +491,28 @@ def test_hip_graph_replays_match_eager():
     finally:
         bench.SHAPE.clear()
         bench.SHAPE.update(keep)
+
+
+def test_randomised_shapes_fp32_match_oracle():
+    """Twelve seeded draws of every dimension and option (ragged lengths, head and state sizes that are not
+    multiples of the tile sizes, grouped B / C, each optional input present or absent) against the fp64 oracle."""
+    rng = torch.Generator().manual_seed(2024)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    flip = lambda: bool(torch.randint(0, 2, (1,), generator=rng))
+    for trial in range(12):
+        G = pick(1, 2)
+        H = G * pick(1, 3)
+        Bsz, L, P, N = pick(1, 3), pick(1, 210), pick(1, 64), pick(1, 280)
+        kw = dict(h0=flip(), softplus=flip(), D=[None, "h", "hp"][pick(0, 2)], z=flip(), bias=flip())
+        case = (Bsz, L, H, P, N, G, kw)
+        _say(f"randomised fp32 {trial}: {case}")
+        d = _problem(Bsz, L, H, P, N, G, seed=500 + trial, **kw)
+        y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+        y, fin, g, _ = _run_operator(d, torch.float32, chunk_size=[64, 128, 256][trial % 3])
+        _check(f"out {case}", y, y_ref, FWD32)
+        _check(f"final_states {case}", fin, fin_ref, FWD32)
+        for k in GRAD_NAMES:
+            if d[k] is None:
+                assert g[k] is None
+                continue
+            _check(f"d{k} {case}", g[k], g_ref[k], BWD32)
