@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ISSM chunked scan on one MI355X.
 
-Workload (BASELINE.json configs[1]): B=8, L=1024, H=8, P=32, N=256, G=1, chunk=64, forward +
+Workload (the configuration the headline metric is quoted on): B=8, L=1024, H=8, P=32, N=256, G=1, chunk=64, forward +
 backward of the bidirectional pair of scans (second direction = reversed token order, same dt /
 A / D / initial states), fp32 inputs, synthetic seeded data already resident in HBM.
 One "step" = one forward + backward call of the operator.  `value` is microseconds per step.
