@@ -27,6 +27,7 @@ EXPORTS = [
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
     "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
+    "issm_hilbert_codes",
 ]
 
 
@@ -117,6 +118,14 @@ class BoxDistArgs(C.Structure):
     ]
 
 
+class HilbertArgs(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("npoint", C.c_int32), ("bits", C.c_int32), ("order", C.c_int32 * 3),
+        ("cell", C.c_float), ("points", C.c_void_p), ("mins", C.c_void_p), ("codes", C.c_void_p),
+        ("stream", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -150,6 +159,7 @@ def load() -> C.CDLL:
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
     lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
+    lib.issm_hilbert_codes.argtypes = [P(HilbertArgs)]
     lib.issm_box_dist_fwd.argtypes = [P(BoxDistArgs)]
     lib.issm_box_dist_bwd.argtypes = [P(BoxDistArgs)]
     lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]

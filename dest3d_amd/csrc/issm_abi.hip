@@ -25,6 +25,7 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
+int launch_hilbert_codes(const HilbertP& p, hipStream_t st);
 int box_dist_workgroups(int B, int L, int K);
 int box_dist_bwd_workgroups(int B, int L, int K);
 long box_dist_bwd_scratch_bytes(int B, int L, int K, int D, int H, int W);
@@ -537,6 +538,26 @@ int issm_box_dist_bwd(const issm_box_dist_args* a) {
   if (rc) return rc;
   if (p.nwg_bwd == 0) return ISSM_OK;
   return launched(launch_box_dist_bwd(p, (hipStream_t)a->stream), "box_dist_bwd");
+}
+
+int issm_hilbert_codes(const issm_hilbert_args* a) {
+  if (!a) return fail(ISSM_E_NULL, "hilbert: args is NULL");
+  if (a->batch < 0 || a->npoint < 0) return fail(ISSM_E_SHAPE, "hilbert: bad shape");
+  if (a->bits < 1 || a->bits > 20) return fail(ISSM_E_UNSUPPORTED, "hilbert: bits = %d (1..20)", a->bits);
+  if (!(a->cell > 0.0f)) return fail(ISSM_E_SHAPE, "hilbert: cell must be positive");
+  int seen = 0;
+  for (int i = 0; i < 3; ++i) {
+    if (a->order[i] < 0 || a->order[i] > 2) return fail(ISSM_E_SHAPE, "hilbert: order[%d] = %d", i, a->order[i]);
+    seen |= 1 << a->order[i];
+  }
+  if (seen != 7) return fail(ISSM_E_SHAPE, "hilbert: order is not a permutation of 0, 1, 2");
+  if ((int64_t)a->batch * a->npoint == 0) return ISSM_OK;
+  if (!a->points || !a->mins || !a->codes) return fail(ISSM_E_NULL, "hilbert: points/mins/codes is NULL");
+  HilbertP p;
+  p.B = a->batch; p.N = a->npoint; p.bits = a->bits; p.cell = a->cell;
+  for (int i = 0; i < 3; ++i) p.perm[i] = a->order[i];
+  p.points = a->points; p.mins = a->mins; p.codes = (long*)a->codes;
+  return launched(launch_hilbert_codes(p, (hipStream_t)a->stream), "hilbert_codes");
 }
 
 }  // extern "C"

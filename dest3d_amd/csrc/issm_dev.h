@@ -78,6 +78,16 @@ struct NormP {
   int nblocks;
 };
 
+// parameters of the serialization-code kernel (hilbert.hip)
+struct HilbertP {
+  int B, N, bits;
+  int perm[3];          // grid coordinate used as first / second / third curve coordinate
+  float cell;
+  const float* points;  // (B, N, 3)
+  const float* mins;    // (B, 3) per-sample minimum corner
+  long* codes;          // (B, N)
+};
+
 // parameters of the box-to-point distance encoding kernels (box_dist.hip)
 struct BoxDistP {
   int B, L, K, D, H, W, dtype, nwg, nwg_bwd;

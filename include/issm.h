@@ -346,6 +346,25 @@ int64_t issm_box_dist_bwd_scratch_bytes(int32_t batch, int32_t seqlen, int32_t n
 int issm_box_dist_fwd(const issm_box_dist_args* args);
 int issm_box_dist_bwd(const issm_box_dist_args* args);
 
+/* ---- serialization codes of the key points ------------------------------------------------
+ * Serialization.forward / encode (models/dest_module.py:307-356): grid = trunc((point - min of the sample) / cell)
+ * clamped to 2^bits - 1, coordinates permuted by `order` (order[i] = which of x, y, z is the i-th curve
+ * coordinate: "yxz" is {1, 0, 2}), mapped to its position on the 3-D Hilbert curve.  The reference looks the
+ * position up in a table file it does not ship; this entry point computes it (Skilling's algorithm), so the curve's
+ * orientation may differ from that table's.  points (B, N, 3), mins (B, 3): fp32 contiguous; codes (B, N) int64.
+ * 1 <= bits <= 20. */
+typedef struct issm_hilbert_args {
+  int32_t batch, npoint, bits;
+  int32_t order[3];
+  float cell;
+  const float* points;
+  const float* mins;
+  int64_t* codes;
+  void* stream;
+} issm_hilbert_args;
+
+int issm_hilbert_codes(const issm_hilbert_args* args);
+
 #ifdef __cplusplus
 }
 #endif
