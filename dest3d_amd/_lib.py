@@ -28,6 +28,9 @@ EXPORTS = [
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
     "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
     "issm_hilbert_codes",
+    "issm_pn2_furthest_point_sampling", "issm_pn2_ball_query", "issm_pn2_group_points", "issm_pn2_group_points_grad",
+    "issm_pn2_gather_points", "issm_pn2_gather_points_grad", "issm_pn2_three_nn", "issm_pn2_three_interpolate",
+    "issm_pn2_three_interpolate_grad",
 ]
 
 
@@ -160,6 +163,16 @@ def load() -> C.CDLL:
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
     lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
     lib.issm_hilbert_codes.argtypes = [P(HilbertArgs)]
+    i32, f32 = C.c_int32, C.c_float
+    lib.issm_pn2_furthest_point_sampling.argtypes = [i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_ball_query.argtypes = [i32, i32, i32, f32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_group_points.argtypes = [i32, i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_group_points_grad.argtypes = [i32, i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_gather_points.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_gather_points_grad.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_three_nn.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp]
+    lib.issm_pn2_three_interpolate.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, vp]
+    lib.issm_pn2_three_interpolate_grad.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.issm_box_dist_fwd.argtypes = [P(BoxDistArgs)]
     lib.issm_box_dist_bwd.argtypes = [P(BoxDistArgs)]
     lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]

@@ -26,6 +26,17 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
 int launch_hilbert_codes(const HilbertP& p, hipStream_t st);
+int launch_fps(int b, int n, int npoint, const float* xyz, float* temp, int* idxs, hipStream_t st);
+int launch_ball_query(int b, int n, int m, float radius, int nsample, const float* new_xyz, const float* xyz, int* idx,
+                      hipStream_t st);
+int launch_group_points(int b, int c, int n, int ms, const float* points, const int* idx, float* out, hipStream_t st);
+int launch_group_points_grad(int b, int c, int n, int ms, const float* grad_out, const int* idx, float* grad_points,
+                             hipStream_t st);
+int launch_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2, int* idx, hipStream_t st);
+int launch_three_interpolate(int b, int c, int m, int n, const float* points, const int* idx, const float* weight, float* out,
+                             hipStream_t st);
+int launch_three_interpolate_grad(int b, int c, int n, int m, const float* grad_out, const int* idx, const float* weight,
+                                  float* grad_points, hipStream_t st);
 int box_dist_workgroups(int B, int L, int K);
 int box_dist_bwd_workgroups(int B, int L, int K);
 long box_dist_bwd_scratch_bytes(int B, int L, int K, int D, int H, int W);
@@ -558,6 +569,101 @@ int issm_hilbert_codes(const issm_hilbert_args* a) {
   for (int i = 0; i < 3; ++i) p.perm[i] = a->order[i];
   p.points = a->points; p.mins = a->mins; p.codes = (long*)a->codes;
   return launched(launch_hilbert_codes(p, (hipStream_t)a->stream), "hilbert_codes");
+}
+
+// shared checks of the point-set operators: non-negative sizes, work present, pointers given
+#define PN2_SIZES(what, ...)                                                              \
+  do {                                                                                    \
+    const long long dims_[] = {__VA_ARGS__};                                              \
+    for (long long d_ : dims_)                                                            \
+      if (d_ < 0) return fail(ISSM_E_SHAPE, what ": negative size");                      \
+  } while (0)
+#define PN2_PTRS(what, ...)                                                               \
+  do {                                                                                    \
+    const void* ptrs_[] = {__VA_ARGS__};                                                  \
+    for (const void* q_ : ptrs_)                                                          \
+      if (!q_) return fail(ISSM_E_NULL, what ": NULL pointer");                           \
+  } while (0)
+
+int issm_pn2_furthest_point_sampling(int32_t b, int32_t n, int32_t npoint, const float* xyz, float* temp, int32_t* idxs,
+                                     void* stream) {
+  PN2_SIZES("furthest_point_sampling", b, n, npoint);
+  if (b == 0 || npoint == 0) return ISSM_OK;
+  if (n == 0) return fail(ISSM_E_SHAPE, "furthest_point_sampling: no points to draw from");
+  if (b > 65535) return fail(ISSM_E_UNSUPPORTED, "furthest_point_sampling: batch %d > 65535", b);
+  PN2_PTRS("furthest_point_sampling", xyz, idxs);
+  if (n > 49152 && !temp) return fail(ISSM_E_NULL, "furthest_point_sampling: temp is NULL (needed above 49152 points)");
+  return launched(launch_fps(b, n, npoint, xyz, temp, idxs, (hipStream_t)stream), "furthest_point_sampling");
+}
+
+int issm_pn2_ball_query(int32_t b, int32_t n, int32_t m, float radius, int32_t nsample, const float* new_xyz,
+                        const float* xyz, int32_t* idx, void* stream) {
+  PN2_SIZES("ball_query", b, n, m, nsample);
+  if (b == 0 || m == 0 || nsample == 0) return ISSM_OK;
+  if (b > 65535) return fail(ISSM_E_UNSUPPORTED, "ball_query: batch %d > 65535", b);
+  PN2_PTRS("ball_query", new_xyz, idx);
+  if (n > 0 && !xyz) return fail(ISSM_E_NULL, "ball_query: xyz is NULL");
+  return launched(launch_ball_query(b, n, m, radius, nsample, new_xyz, xyz, idx, (hipStream_t)stream), "ball_query");
+}
+
+int issm_pn2_group_points(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* points,
+                          const int32_t* idx, float* out, void* stream) {
+  PN2_SIZES("group_points", b, c, n, npoints, nsample);
+  if ((int64_t)b * c * npoints * nsample == 0) return ISSM_OK;
+  if (n == 0) return fail(ISSM_E_SHAPE, "group_points: no points to index");
+  if ((int64_t)npoints * nsample > 0x7fffffff) return fail(ISSM_E_SHAPE, "group_points: too many indices per sample");
+  PN2_PTRS("group_points", points, idx, out);
+  return launched(launch_group_points(b, c, n, npoints * nsample, points, idx, out, (hipStream_t)stream), "group_points");
+}
+
+int issm_pn2_group_points_grad(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* grad_out,
+                               const int32_t* idx, float* grad_points, void* stream) {
+  PN2_SIZES("group_points_grad", b, c, n, npoints, nsample);
+  if ((int64_t)b * c * npoints * nsample == 0) return ISSM_OK;
+  if (n == 0) return fail(ISSM_E_SHAPE, "group_points_grad: no points to index");
+  if ((int64_t)npoints * nsample > 0x7fffffff) return fail(ISSM_E_SHAPE, "group_points_grad: too many indices per sample");
+  PN2_PTRS("group_points_grad", grad_out, idx, grad_points);
+  return launched(launch_group_points_grad(b, c, n, npoints * nsample, grad_out, idx, grad_points, (hipStream_t)stream),
+                  "group_points_grad");
+}
+
+int issm_pn2_gather_points(int32_t b, int32_t c, int32_t n, int32_t npoints, const float* points, const int32_t* idx,
+                           float* out, void* stream) {
+  return issm_pn2_group_points(b, c, n, npoints, 1, points, idx, out, stream);
+}
+
+int issm_pn2_gather_points_grad(int32_t b, int32_t c, int32_t n, int32_t npoints, const float* grad_out,
+                                const int32_t* idx, float* grad_points, void* stream) {
+  return issm_pn2_group_points_grad(b, c, n, npoints, 1, grad_out, idx, grad_points, stream);
+}
+
+int issm_pn2_three_nn(int32_t b, int32_t n, int32_t m, const float* unknown, const float* known, float* dist2,
+                      int32_t* idx, void* stream) {
+  PN2_SIZES("three_nn", b, n, m);
+  if (b == 0 || n == 0) return ISSM_OK;
+  if (b > 65535) return fail(ISSM_E_UNSUPPORTED, "three_nn: batch %d > 65535", b);
+  PN2_PTRS("three_nn", unknown, dist2, idx);
+  if (m > 0 && !known) return fail(ISSM_E_NULL, "three_nn: known is NULL");
+  return launched(launch_three_nn(b, n, m, unknown, known, dist2, idx, (hipStream_t)stream), "three_nn");
+}
+
+int issm_pn2_three_interpolate(int32_t b, int32_t c, int32_t m, int32_t n, const float* points, const int32_t* idx,
+                               const float* weight, float* out, void* stream) {
+  PN2_SIZES("three_interpolate", b, c, m, n);
+  if ((int64_t)b * c * n == 0) return ISSM_OK;
+  if (m == 0) return fail(ISSM_E_SHAPE, "three_interpolate: no points to index");
+  PN2_PTRS("three_interpolate", points, idx, weight, out);
+  return launched(launch_three_interpolate(b, c, m, n, points, idx, weight, out, (hipStream_t)stream), "three_interpolate");
+}
+
+int issm_pn2_three_interpolate_grad(int32_t b, int32_t c, int32_t n, int32_t m, const float* grad_out, const int32_t* idx,
+                                    const float* weight, float* grad_points, void* stream) {
+  PN2_SIZES("three_interpolate_grad", b, c, n, m);
+  if ((int64_t)b * c * n == 0) return ISSM_OK;
+  if (m == 0) return fail(ISSM_E_SHAPE, "three_interpolate_grad: no points to index");
+  PN2_PTRS("three_interpolate_grad", grad_out, idx, weight, grad_points);
+  return launched(launch_three_interpolate_grad(b, c, n, m, grad_out, idx, weight, grad_points, (hipStream_t)stream),
+                  "three_interpolate_grad");
 }
 
 }  // extern "C"

@@ -1,0 +1,273 @@
+// Point-set operators of the PointNet++ backbone for gfx950: furthest point sampling, ball query, grouping,
+// gathering, 3-nearest-neighbour search and interpolation (the functions of the reference's `pointnet2._ext`,
+// pointnet2/_ext_src/src/*.cpp).  Index arithmetic is exact; all tensors fp32 / int32, contiguous.
+//
+//  * furthest point sampling: one 512-thread workgroup per sample; a thread owns points tid, tid + 512, ... and keeps
+//    their running minimum distance in registers (up to 49152 points; beyond that in the caller's `temp`); per
+//    sample drawn: one pass over the thread's points, an argmax over the wave with shuffles, over the 8 waves
+//    through LDS.  Ties go to the smaller index.
+//  * ball query: one wave per query centre; 64 points are tested per step and compacted in index order with a
+//    ballot, so the first `nsample` hits are found without a serial scan; the wave stops as soon as it has them.
+//  * 3-NN: one thread per unknown point, known points staged through LDS 256 at a time.
+//  * group / gather / interpolate: one thread per output element, innermost index fastest; the gradients scatter
+//    with hardware float atomics (duplicates in idx are the rule), as the reference does.
+#include "issm_dev.h"
+
+namespace issm {
+
+constexpr int FPS_T = 512;    // threads of the sampling workgroup (two waves per SIMD: 256 registers each)
+constexpr int FPS_REG = 96;   // points per thread whose running distance lives in registers
+
+// Squared distance in plain fp32 steps (three subtractions, three products, two additions, each rounded): no fused
+// multiply-add and no reordering, so the comparisons that pick indices agree with a straightforward fp32 evaluation.
+__device__ __forceinline__ float sqdist(float ax, float ay, float az, float bx, float by, float bz) {
+#pragma clang fp contract(off) reassociate(off)
+  const float dx = ax - bx, dy = ay - by, dz = az - bz;
+  const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+  return (xx + yy) + zz;
+}
+
+struct ArgMax {
+  float v;
+  int i;
+};
+__device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {  // larger value, then smaller index
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+
+// idxs[b][0] = 0; then repeatedly the point farthest from the chosen set.  Points with |p|^2 <= 1e-3 (padding at the
+// origin) are never chosen and keep their distance, as in the reference (sampling_gpu.cu:105-106).
+__global__ __launch_bounds__(FPS_T) void k_fps(int n, int npoint, const float* __restrict__ xyz, float* __restrict__ temp,
+                                                int* __restrict__ idxs) {
+  __shared__ float sv[FPS_T / 64];
+  __shared__ int si[FPS_T / 64];
+  __shared__ int chosen;
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* p = xyz + (long)b * n * 3;
+  float* tmp = temp + (long)b * n;
+  int* out = idxs + (long)b * npoint;
+  const bool inreg = n <= FPS_T * FPS_REG;
+  float dreg[FPS_REG];
+#pragma unroll
+  for (int j = 0; j < FPS_REG; ++j) dreg[j] = 1e10f;
+  if (!inreg)
+    for (int k = tid; k < n; k += FPS_T) tmp[k] = 1e10f;
+  if (tid == 0) out[0] = 0;
+  int old = 0;
+  for (int s = 1; s < npoint; ++s) {
+    const float ox = p[old * 3], oy = p[old * 3 + 1], oz = p[old * 3 + 2];
+    float bv = -1.0f;
+    int bi = 0;
+    // new running distance of point k (old one d); updates the thread's best candidate
+#define FPS_VISIT(k, d)                                                         \
+    do {                                                                          \
+      const float x = p[(k) * 3], y = p[(k) * 3 + 1], z = p[(k) * 3 + 2];         \
+      if (sqdist(x, y, z, 0.0f, 0.0f, 0.0f) > 1e-3f) {                            \
+        d = fminf(d, sqdist(x, y, z, ox, oy, oz));                                \
+        if (d > bv) { bv = d; bi = (k); } /* k ascends: the first maximum stays */ \
+      }                                                                           \
+    } while (0)
+    if (inreg) {
+#pragma unroll
+      for (int j = 0; j < FPS_REG; ++j) {
+        int first = j * FPS_T;
+        asm volatile("" : "+s"(first));  // keeps 96 loop-invariant addresses from being held in registers
+        const int k = tid + first;
+        if (k < n) FPS_VISIT(k, dreg[j]);
+      }
+    } else {
+      for (int k = tid; k < n; k += FPS_T) {
+        float d = tmp[k];
+        FPS_VISIT(k, d);
+        tmp[k] = d;
+      }
+    }
+#undef FPS_VISIT
+    ArgMax best = {bv, bi};
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      ArgMax other = {__shfl_xor(best.v, o, 64), __shfl_xor(best.i, o, 64)};
+      best = better(best, other);
+    }
+    if (lane == 0) { sv[wave] = best.v; si[wave] = best.i; }
+    __syncthreads();
+    if (tid == 0) {
+      ArgMax a = {sv[0], si[0]};
+      for (int w = 1; w < FPS_T / 64; ++w) a = better(a, ArgMax{sv[w], si[w]});
+      chosen = a.i;
+      out[s] = a.i;
+    }
+    __syncthreads();
+    old = chosen;
+  }
+}
+
+// idx[b][j][0..nsample): the first nsample points (in index order) closer than radius to new_xyz[b][j]; missing
+// slots repeat the first hit; no hit at all leaves zeros (ball_query_gpu.cu:20-44).
+__global__ __launch_bounds__(NTHREADS) void k_ball_query(int n, int m, float radius2, int nsample,
+                                                         const float* __restrict__ new_xyz, const float* __restrict__ xyz,
+                                                         int* __restrict__ idx) {
+  const int b = blockIdx.y, lane = threadIdx.x & 63;
+  const int j = blockIdx.x * (NTHREADS / 64) + (threadIdx.x >> 6);
+  if (j >= m) return;  // whole wave
+  const float* q = new_xyz + ((long)b * m + j) * 3;
+  const float qx = q[0], qy = q[1], qz = q[2];
+  const float* p = xyz + (long)b * n * 3;
+  int* out = idx + ((long)b * m + j) * nsample;
+  int cnt = 0, first = 0;
+  for (int k0 = 0; k0 < n && cnt < nsample; k0 += 64) {
+    const int k = k0 + lane;
+    bool hit = false;
+    if (k < n) {
+      hit = sqdist(qx, qy, qz, p[k * 3], p[k * 3 + 1], p[k * 3 + 2]) < radius2;
+    }
+    const unsigned long long mask = __ballot(hit);
+    if (mask == 0) continue;
+    if (cnt == 0) first = k0 + __builtin_ctzll(mask);
+    const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+    if (hit && slot < nsample) out[slot] = k;
+    cnt += __popcll(mask);
+  }
+  if (cnt > nsample) cnt = nsample;
+  for (int s = cnt + lane; s < nsample; s += 64) out[s] = first;  // first == 0 when nothing was found
+}
+
+// out[b][c][j][s] = points[b][c][idx[b][j][s]]   (one thread per output element)
+__global__ __launch_bounds__(NTHREADS) void k_group_points(long total, int c, int n, int ms, const float* __restrict__ points,
+                                                           const int* __restrict__ idx, float* __restrict__ out) {
+  const long e = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (e >= total) return;
+  const int r = (int)(e % ms);
+  const long bc = e / ms;
+  const int b = (int)(bc / c);
+  const int k = min(max(idx[(long)b * ms + r], 0), n - 1);  // a stray index must not leave the tensor
+  out[e] = points[bc * n + k];
+}
+__global__ __launch_bounds__(NTHREADS) void k_group_points_grad(long total, int c, int n, int ms,
+                                                                const float* __restrict__ grad_out,
+                                                                const int* __restrict__ idx, float* __restrict__ grad_points) {
+  const long e = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (e >= total) return;
+  const int r = (int)(e % ms);
+  const long bc = e / ms;
+  const int b = (int)(bc / c);
+  const int k = min(max(idx[(long)b * ms + r], 0), n - 1);
+  unsafeAtomicAdd(grad_points + bc * n + k, grad_out[e]);
+}
+
+// 3 nearest known points of every unknown point: squared distances ascending, ties to the smaller index
+__global__ __launch_bounds__(NTHREADS) void k_three_nn(int n, int m, const float* __restrict__ unknown,
+                                                       const float* __restrict__ known, float* __restrict__ dist2,
+                                                       int* __restrict__ idx) {
+  __shared__ float kx[NTHREADS], ky[NTHREADS], kz[NTHREADS];
+  const int b = blockIdx.y;
+  const int j = blockIdx.x * NTHREADS + threadIdx.x;
+  const bool live = j < n;
+  float ux = 0.0f, uy = 0.0f, uz = 0.0f;
+  if (live) {
+    const float* u = unknown + ((long)b * n + j) * 3;
+    ux = u[0]; uy = u[1]; uz = u[2];
+  }
+  float b1 = __builtin_huge_valf(), b2 = b1, b3 = b1;  // fewer than 3 known points leave +inf (the reference's 1e40)
+  int i1 = 0, i2 = 0, i3 = 0;
+  const float* kp = known + (long)b * m * 3;
+  for (int k0 = 0; k0 < m; k0 += NTHREADS) {
+    const int kk = k0 + threadIdx.x;
+    if (kk < m) { kx[threadIdx.x] = kp[kk * 3]; ky[threadIdx.x] = kp[kk * 3 + 1]; kz[threadIdx.x] = kp[kk * 3 + 2]; }
+    __syncthreads();
+    const int lim = min(NTHREADS, m - k0);
+    for (int t = 0; t < lim; ++t) {
+      const float d = sqdist(ux, uy, uz, kx[t], ky[t], kz[t]);
+      const int k = k0 + t;
+      if (d < b1) { b3 = b2; i3 = i2; b2 = b1; i2 = i1; b1 = d; i1 = k; }
+      else if (d < b2) { b3 = b2; i3 = i2; b2 = d; i2 = k; }
+      else if (d < b3) { b3 = d; i3 = k; }
+    }
+    __syncthreads();
+  }
+  if (live) {
+    float* dd = dist2 + ((long)b * n + j) * 3;
+    int* ii = idx + ((long)b * n + j) * 3;
+    dd[0] = b1; dd[1] = b2; dd[2] = b3;
+    ii[0] = i1; ii[1] = i2; ii[2] = i3;
+  }
+}
+
+// out[b][c][j] = sum_k weight[b][j][k] * points[b][c][idx[b][j][k]]
+__global__ __launch_bounds__(NTHREADS) void k_three_interpolate(long total, int c, int m, int n, const float* __restrict__ points,
+                                                                const int* __restrict__ idx, const float* __restrict__ weight,
+                                                                float* __restrict__ out) {
+  const long e = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % n);
+  const long bc = e / n;
+  const int b = (int)(bc / c);
+  const long o = ((long)b * n + j) * 3;
+  const float* src = points + bc * m;
+  float acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) acc += weight[o + k] * src[min(max(idx[o + k], 0), m - 1)];
+  out[e] = acc;
+}
+__global__ __launch_bounds__(NTHREADS) void k_three_interpolate_grad(long total, int c, int n, int m,
+                                                                     const float* __restrict__ grad_out,
+                                                                     const int* __restrict__ idx,
+                                                                     const float* __restrict__ weight,
+                                                                     float* __restrict__ grad_points) {
+  const long e = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % n);
+  const long bc = e / n;
+  const int b = (int)(bc / c);
+  const long o = ((long)b * n + j) * 3;
+  float* dst = grad_points + bc * m;
+  const float g = grad_out[e];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) unsafeAtomicAdd(dst + min(max(idx[o + k], 0), m - 1), g * weight[o + k]);
+}
+
+static unsigned blocks_for(long total) { return (unsigned)((total + NTHREADS - 1) / NTHREADS); }
+
+int launch_fps(int b, int n, int npoint, const float* xyz, float* temp, int* idxs, hipStream_t st) {
+  hipLaunchKernelGGL(k_fps, dim3(b), dim3(FPS_T), 0, st, n, npoint, xyz, temp, idxs);
+  return (int)hipGetLastError();
+}
+int launch_ball_query(int b, int n, int m, float radius, int nsample, const float* new_xyz, const float* xyz, int* idx,
+                      hipStream_t st) {
+  hipLaunchKernelGGL(k_ball_query, dim3((m + 3) / 4, b), dim3(NTHREADS), 0, st, n, m, radius * radius, nsample, new_xyz, xyz,
+                     idx);
+  return (int)hipGetLastError();
+}
+int launch_group_points(int b, int c, int n, int ms, const float* points, const int* idx, float* out, hipStream_t st) {
+  const long total = (long)b * c * ms;
+  hipLaunchKernelGGL(k_group_points, dim3(blocks_for(total)), dim3(NTHREADS), 0, st, total, c, n, ms, points, idx, out);
+  return (int)hipGetLastError();
+}
+int launch_group_points_grad(int b, int c, int n, int ms, const float* grad_out, const int* idx, float* grad_points,
+                             hipStream_t st) {
+  const long total = (long)b * c * ms;
+  hipLaunchKernelGGL(k_group_points_grad, dim3(blocks_for(total)), dim3(NTHREADS), 0, st, total, c, n, ms, grad_out, idx,
+                     grad_points);
+  return (int)hipGetLastError();
+}
+int launch_three_nn(int b, int n, int m, const float* unknown, const float* known, float* dist2, int* idx, hipStream_t st) {
+  hipLaunchKernelGGL(k_three_nn, dim3((n + NTHREADS - 1) / NTHREADS, b), dim3(NTHREADS), 0, st, n, m, unknown, known, dist2,
+                     idx);
+  return (int)hipGetLastError();
+}
+int launch_three_interpolate(int b, int c, int m, int n, const float* points, const int* idx, const float* weight, float* out,
+                             hipStream_t st) {
+  const long total = (long)b * c * n;
+  hipLaunchKernelGGL(k_three_interpolate, dim3(blocks_for(total)), dim3(NTHREADS), 0, st, total, c, m, n, points, idx, weight,
+                     out);
+  return (int)hipGetLastError();
+}
+int launch_three_interpolate_grad(int b, int c, int n, int m, const float* grad_out, const int* idx, const float* weight,
+                                  float* grad_points, hipStream_t st) {
+  const long total = (long)b * c * n;
+  hipLaunchKernelGGL(k_three_interpolate_grad, dim3(blocks_for(total)), dim3(NTHREADS), 0, st, total, c, n, m, grad_out, idx,
+                     weight, grad_points);
+  return (int)hipGetLastError();
+}
+
+}  // namespace issm

@@ -365,6 +365,39 @@ typedef struct issm_hilbert_args {
 
 int issm_hilbert_codes(const issm_hilbert_args* args);
 
+/* ---- point-set operators of the PointNet++ backbone ---------------------------------------
+ * The functions of the reference's `pointnet2._ext` (pointnet2/_ext_src/src/bindings.cpp:8-24), same argument
+ * meaning as its C++ wrappers; fp32 / int32, contiguous, device pointers.  Outputs that the reference allocates
+ * with torch::zeros and then accumulates into (the *_grad functions) must be zeroed by the caller.
+ *   furthest_point_sampling  sampling.cpp:70-91     xyz (b, n, 3) -> idxs (b, npoint); temp (b, n) scratch, used
+ *                            only when n > 49152.  Starts at point 0; points with |p|^2 <= 1e-3 are never drawn;
+ *                            equal distances go to the smaller index.
+ *   ball_query               ball_query.cpp:13-37   new_xyz (b, m, 3), xyz (b, n, 3) -> idx (b, m, nsample)
+ *   group_points(_grad)      group_points.cpp:17-65 points (b, c, n), idx (b, npoints, nsample) -> (b, c, npoints, nsample)
+ *   gather_points(_grad)     sampling.cpp:20-68     points (b, c, n), idx (b, npoints) -> (b, c, npoints)
+ *   three_nn                 interpolate.cpp:19-45  unknown (b, n, 3), known (b, m, 3) -> dist2, idx (b, n, 3)
+ *   three_interpolate(_grad) interpolate.cpp:47-104 points (b, c, m), idx, weight (b, n, 3) -> (b, c, n)
+ * Distances are evaluated in plain fp32 steps (no fused multiply-add), so index choices follow a straightforward
+ * fp32 evaluation. */
+int issm_pn2_furthest_point_sampling(int32_t b, int32_t n, int32_t npoint, const float* xyz, float* temp, int32_t* idxs,
+                                     void* stream);
+int issm_pn2_ball_query(int32_t b, int32_t n, int32_t m, float radius, int32_t nsample, const float* new_xyz,
+                        const float* xyz, int32_t* idx, void* stream);
+int issm_pn2_group_points(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* points,
+                          const int32_t* idx, float* out, void* stream);
+int issm_pn2_group_points_grad(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* grad_out,
+                               const int32_t* idx, float* grad_points, void* stream);
+int issm_pn2_gather_points(int32_t b, int32_t c, int32_t n, int32_t npoints, const float* points, const int32_t* idx,
+                           float* out, void* stream);
+int issm_pn2_gather_points_grad(int32_t b, int32_t c, int32_t n, int32_t npoints, const float* grad_out,
+                                const int32_t* idx, float* grad_points, void* stream);
+int issm_pn2_three_nn(int32_t b, int32_t n, int32_t m, const float* unknown, const float* known, float* dist2,
+                      int32_t* idx, void* stream);
+int issm_pn2_three_interpolate(int32_t b, int32_t c, int32_t m, int32_t n, const float* points, const int32_t* idx,
+                               const float* weight, float* out, void* stream);
+int issm_pn2_three_interpolate_grad(int32_t b, int32_t c, int32_t n, int32_t m, const float* grad_out, const int32_t* idx,
+                                    const float* weight, float* grad_points, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
