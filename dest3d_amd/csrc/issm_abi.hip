@@ -592,7 +592,7 @@ int issm_pn2_furthest_point_sampling(int32_t b, int32_t n, int32_t npoint, const
   if (n == 0) return fail(ISSM_E_SHAPE, "furthest_point_sampling: no points to draw from");
   if (b > 65535) return fail(ISSM_E_UNSUPPORTED, "furthest_point_sampling: batch %d > 65535", b);
   PN2_PTRS("furthest_point_sampling", xyz, idxs);
-  if (n > 49152 && !temp) return fail(ISSM_E_NULL, "furthest_point_sampling: temp is NULL (needed above 49152 points)");
+  if (n > 24576 && !temp) return fail(ISSM_E_NULL, "furthest_point_sampling: temp is NULL (needed above 24576 points)");
   return launched(launch_fps(b, n, npoint, xyz, temp, idxs, (hipStream_t)stream), "furthest_point_sampling");
 }
 

@@ -3,9 +3,9 @@
 // pointnet2/_ext_src/src/*.cpp).  Index arithmetic is exact; all tensors fp32 / int32, contiguous.
 //
 //  * furthest point sampling: one 512-thread workgroup per sample; a thread owns points tid, tid + 512, ... and keeps
-//    their running minimum distance in registers (up to 49152 points; beyond that in the caller's `temp`); per
-//    sample drawn: one pass over the thread's points, an argmax over the wave with shuffles, over the 8 waves
-//    through LDS.  Ties go to the smaller index.
+//    their coordinates and running minimum distance in registers (up to 24576 points; beyond that coordinates are
+//    re-read and distances kept in the caller's `temp`); per sample drawn: one pass over the thread's points, an
+//    argmax over the wave with shuffles, over the 8 waves through LDS.  Ties go to the smaller index.
 //  * ball query: one wave per query centre; 64 points are tested per step and compacted in index order with a
 //    ballot, so the first `nsample` hits are found without a serial scan; the wave stops as soon as it has them.
 //  * 3-NN: one thread per unknown point, known points staged through LDS 256 at a time.
@@ -16,7 +16,6 @@
 namespace issm {
 
 constexpr int FPS_T = 512;    // threads of the sampling workgroup (two waves per SIMD: 256 registers each)
-constexpr int FPS_REG = 96;   // points per thread whose running distance lives in registers
 
 // Squared distance in plain fp32 steps (three subtractions, three products, two additions, each rounded): no fused
 // multiply-add and no reordering, so the comparisons that pick indices agree with a straightforward fp32 evaluation.
@@ -37,6 +36,9 @@ __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {  // larger value,
 
 // idxs[b][0] = 0; then repeatedly the point farthest from the chosen set.  Points with |p|^2 <= 1e-3 (padding at the
 // origin) are never chosen and keep their distance, as in the reference (sampling_gpu.cu:105-106).
+// PPT > 0: the thread's PPT points -- coordinates and running distance -- live in registers for the whole kernel
+// (n <= 512 * PPT); PPT == 0: any n, coordinates re-read from memory (L2) and distances kept in `temp`.
+template <int PPT>
 __global__ __launch_bounds__(FPS_T) void k_fps(int n, int npoint, const float* __restrict__ xyz, float* __restrict__ temp,
                                                 int* __restrict__ idxs) {
   __shared__ float sv[FPS_T / 64];
@@ -44,45 +46,46 @@ __global__ __launch_bounds__(FPS_T) void k_fps(int n, int npoint, const float* _
   __shared__ int chosen;
   const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* p = xyz + (long)b * n * 3;
-  float* tmp = temp + (long)b * n;
   int* out = idxs + (long)b * npoint;
-  const bool inreg = n <= FPS_T * FPS_REG;
-  float dreg[FPS_REG];
+  constexpr int R = PPT > 0 ? PPT : 1;
+  float px[R], py[R], pz[R], dreg[R];
+  float* tmp = nullptr;
+  if (PPT > 0) {
 #pragma unroll
-  for (int j = 0; j < FPS_REG; ++j) dreg[j] = 1e10f;
-  if (!inreg)
+    for (int j = 0; j < R; ++j) {
+      const int k = tid + j * FPS_T;
+      px[j] = py[j] = pz[j] = 0.0f;  // a slot past n looks like a padding point: skipped
+      if (k < n) { px[j] = p[k * 3]; py[j] = p[k * 3 + 1]; pz[j] = p[k * 3 + 2]; }
+      // padding points get a distance that never wins; the others start at 1e10
+      dreg[j] = sqdist(px[j], py[j], pz[j], 0.0f, 0.0f, 0.0f) > 1e-3f ? 1e10f : -2.0f;
+    }
+  } else {
+    tmp = temp + (long)b * n;
     for (int k = tid; k < n; k += FPS_T) tmp[k] = 1e10f;
+  }
   if (tid == 0) out[0] = 0;
   int old = 0;
   for (int s = 1; s < npoint; ++s) {
     const float ox = p[old * 3], oy = p[old * 3 + 1], oz = p[old * 3 + 2];
     float bv = -1.0f;
     int bi = 0;
-    // new running distance of point k (old one d); updates the thread's best candidate
-#define FPS_VISIT(k, d)                                                         \
-    do {                                                                          \
-      const float x = p[(k) * 3], y = p[(k) * 3 + 1], z = p[(k) * 3 + 2];         \
-      if (sqdist(x, y, z, 0.0f, 0.0f, 0.0f) > 1e-3f) {                            \
-        d = fminf(d, sqdist(x, y, z, ox, oy, oz));                                \
-        if (d > bv) { bv = d; bi = (k); } /* k ascends: the first maximum stays */ \
-      }                                                                           \
-    } while (0)
-    if (inreg) {
+    if (PPT > 0) {
 #pragma unroll
-      for (int j = 0; j < FPS_REG; ++j) {
-        int first = j * FPS_T;
-        asm volatile("" : "+s"(first));  // keeps 96 loop-invariant addresses from being held in registers
-        const int k = tid + first;
-        if (k < n) FPS_VISIT(k, dreg[j]);
+      for (int j = 0; j < R; ++j) {
+        const float d = fminf(dreg[j], sqdist(px[j], py[j], pz[j], ox, oy, oz));
+        dreg[j] = d;
+        if (d > bv) { bv = d; bi = tid + j * FPS_T; }  // indices ascend with j: the first maximum stays
       }
     } else {
       for (int k = tid; k < n; k += FPS_T) {
-        float d = tmp[k];
-        FPS_VISIT(k, d);
-        tmp[k] = d;
+        const float x = p[k * 3], y = p[k * 3 + 1], z = p[k * 3 + 2];
+        if (sqdist(x, y, z, 0.0f, 0.0f, 0.0f) > 1e-3f) {
+          const float d = fminf(tmp[k], sqdist(x, y, z, ox, oy, oz));
+          tmp[k] = d;
+          if (d > bv) { bv = d; bi = k; }
+        }
       }
     }
-#undef FPS_VISIT
     ArgMax best = {bv, bi};
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -94,8 +97,8 @@ __global__ __launch_bounds__(FPS_T) void k_fps(int n, int npoint, const float* _
     if (tid == 0) {
       ArgMax a = {sv[0], si[0]};
       for (int w = 1; w < FPS_T / 64; ++w) a = better(a, ArgMax{sv[w], si[w]});
-      chosen = a.i;
-      out[s] = a.i;
+      chosen = a.v > -1.0f ? a.i : 0;  // nothing but padding points: index 0, as the reference
+      out[s] = chosen;
     }
     __syncthreads();
     old = chosen;
@@ -229,7 +232,11 @@ __global__ __launch_bounds__(NTHREADS) void k_three_interpolate_grad(long total,
 static unsigned blocks_for(long total) { return (unsigned)((total + NTHREADS - 1) / NTHREADS); }
 
 int launch_fps(int b, int n, int npoint, const float* xyz, float* temp, int* idxs, hipStream_t st) {
-  hipLaunchKernelGGL(k_fps, dim3(b), dim3(FPS_T), 0, st, n, npoint, xyz, temp, idxs);
+  const dim3 g(b), t(FPS_T);
+  if (n <= FPS_T * 8) hipLaunchKernelGGL(k_fps<8>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 24) hipLaunchKernelGGL(k_fps<24>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 48) hipLaunchKernelGGL(k_fps<48>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else hipLaunchKernelGGL(k_fps<0>, g, t, 0, st, n, npoint, xyz, temp, idxs);
   return (int)hipGetLastError();
 }
 int launch_ball_query(int b, int n, int m, float radius, int nsample, const float* new_xyz, const float* xyz, int* idx,

@@ -35,7 +35,7 @@ class FurthestPointSampling(Function):
         Bsz, N, _ = x.shape
         with torch.cuda.device(x.device):
             out = torch.zeros((Bsz, npoint), dtype=torch.int32, device=x.device)
-            temp = torch.empty((Bsz, N), dtype=torch.float32, device=x.device) if N > 49152 else None
+            temp = torch.empty((Bsz, N), dtype=torch.float32, device=x.device) if N > 24576 else None
             L.check(lib.issm_pn2_furthest_point_sampling(Bsz, N, npoint, x.data_ptr(), None if temp is None else temp.data_ptr(),
                                                          out.data_ptr(), _st(x)), "issm_pn2_furthest_point_sampling")
         ctx.mark_non_differentiable(out)

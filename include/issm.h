@@ -370,7 +370,7 @@ int issm_hilbert_codes(const issm_hilbert_args* args);
  * meaning as its C++ wrappers; fp32 / int32, contiguous, device pointers.  Outputs that the reference allocates
  * with torch::zeros and then accumulates into (the *_grad functions) must be zeroed by the caller.
  *   furthest_point_sampling  sampling.cpp:70-91     xyz (b, n, 3) -> idxs (b, npoint); temp (b, n) scratch, used
- *                            only when n > 49152.  Starts at point 0; points with |p|^2 <= 1e-3 are never drawn;
+ *                            only when n > 24576.  Starts at point 0; points with |p|^2 <= 1e-3 are never drawn;
  *                            equal distances go to the smaller index.
  *   ball_query               ball_query.cpp:13-37   new_xyz (b, m, 3), xyz (b, n, 3) -> idx (b, m, nsample)
  *   group_points(_grad)      group_points.cpp:17-65 points (b, c, n), idx (b, npoints, nsample) -> (b, c, npoints, nsample)
