@@ -30,7 +30,7 @@ EXPORTS = [
     "issm_hilbert_codes",
     "issm_pn2_furthest_point_sampling", "issm_pn2_ball_query", "issm_pn2_group_points", "issm_pn2_group_points_grad",
     "issm_pn2_gather_points", "issm_pn2_gather_points_grad", "issm_pn2_three_nn", "issm_pn2_three_interpolate",
-    "issm_pn2_three_interpolate_grad",
+    "issm_pn2_three_interpolate_grad", "issm_pn2_group_points_grad_cl", "issm_pn2_three_interpolate_grad_cl",
 ]
 
 
@@ -173,6 +173,8 @@ def load() -> C.CDLL:
     lib.issm_pn2_three_nn.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp]
     lib.issm_pn2_three_interpolate.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.issm_pn2_three_interpolate_grad.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, vp]
+    lib.issm_pn2_group_points_grad_cl.argtypes = [i32, i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.issm_pn2_three_interpolate_grad_cl.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.issm_box_dist_fwd.argtypes = [P(BoxDistArgs)]
     lib.issm_box_dist_bwd.argtypes = [P(BoxDistArgs)]
     lib.issm_dwconv_partial_rows.argtypes = [C.c_int32, C.c_int32]

@@ -37,6 +37,8 @@ int launch_three_interpolate(int b, int c, int m, int n, const float* points, co
                              hipStream_t st);
 int launch_three_interpolate_grad(int b, int c, int n, int m, const float* grad_out, const int* idx, const float* weight,
                                   float* grad_points, hipStream_t st);
+int launch_scatter_channel_last(bool k3, int b, int c, int n, int ne, const float* grad_out, const int* idx,
+                                const float* weight, float* out_cl, hipStream_t st);
 int box_dist_workgroups(int B, int L, int K);
 int box_dist_bwd_workgroups(int B, int L, int K);
 long box_dist_bwd_scratch_bytes(int B, int L, int K, int D, int H, int W);
@@ -664,6 +666,29 @@ int issm_pn2_three_interpolate_grad(int32_t b, int32_t c, int32_t n, int32_t m, 
   PN2_PTRS("three_interpolate_grad", grad_out, idx, weight, grad_points);
   return launched(launch_three_interpolate_grad(b, c, n, m, grad_out, idx, weight, grad_points, (hipStream_t)stream),
                   "three_interpolate_grad");
+}
+
+int issm_pn2_group_points_grad_cl(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* grad_out,
+                                  const int32_t* idx, float* grad_points_cl, void* stream) {
+  PN2_SIZES("group_points_grad_cl", b, c, n, npoints, nsample);
+  if ((int64_t)b * c * npoints * nsample == 0) return ISSM_OK;
+  if (n == 0) return fail(ISSM_E_SHAPE, "group_points_grad_cl: no points to index");
+  if ((int64_t)npoints * nsample > 0x7fffffff || b > 65535)
+    return fail(ISSM_E_UNSUPPORTED, "group_points_grad_cl: too many indices per sample or batch > 65535");
+  PN2_PTRS("group_points_grad_cl", grad_out, idx, grad_points_cl);
+  return launched(launch_scatter_channel_last(false, b, c, n, npoints * nsample, grad_out, idx, nullptr, grad_points_cl,
+                                              (hipStream_t)stream), "group_points_grad_cl");
+}
+
+int issm_pn2_three_interpolate_grad_cl(int32_t b, int32_t c, int32_t n, int32_t m, const float* grad_out,
+                                       const int32_t* idx, const float* weight, float* grad_points_cl, void* stream) {
+  PN2_SIZES("three_interpolate_grad_cl", b, c, n, m);
+  if ((int64_t)b * c * n == 0) return ISSM_OK;
+  if (m == 0) return fail(ISSM_E_SHAPE, "three_interpolate_grad_cl: no points to index");
+  if (b > 65535) return fail(ISSM_E_UNSUPPORTED, "three_interpolate_grad_cl: batch %d > 65535", b);
+  PN2_PTRS("three_interpolate_grad_cl", grad_out, idx, weight, grad_points_cl);
+  return launched(launch_scatter_channel_last(true, b, c, m, n, grad_out, idx, weight, grad_points_cl, (hipStream_t)stream),
+                  "three_interpolate_grad_cl");
 }
 
 }  // extern "C"

@@ -10,7 +10,9 @@
 //    ballot, so the first `nsample` hits are found without a serial scan; the wave stops as soon as it has them.
 //  * 3-NN: one thread per unknown point, known points staged through LDS 256 at a time.
 //  * group / gather / interpolate: one thread per output element, innermost index fastest; the gradients scatter
-//    with hardware float atomics (duplicates in idx are the rule), as the reference does.
+//    with hardware float atomics (duplicates in idx are the rule), as the reference does -- either straight into
+//    the (b, c, n) layout, one scattered cache line per lane, or (the *_cl entry points) into a channel-last
+//    (b, n, c) buffer through an LDS transpose, 64 consecutive floats per instruction.
 #include "issm_dev.h"
 
 namespace issm {
@@ -227,6 +229,50 @@ __global__ __launch_bounds__(NTHREADS) void k_three_interpolate_grad(long total,
   const float g = grad_out[e];
 #pragma unroll
   for (int k = 0; k < 3; ++k) unsafeAtomicAdd(dst + min(max(idx[o + k], 0), m - 1), g * weight[o + k]);
+}
+
+// Gradients into a channel-last buffer, out_cl (b, n, c) += ...: a 64 x 64 tile of grad_out (channels x entries) is
+// read along the entries (coalesced), turned in LDS, and added with lanes running over channels, so one atomic
+// instruction covers 64 consecutive floats of one point instead of 64 scattered cache lines.
+// K3 == false: grouping, entries e = (j, s) with index idx[b][e], value grad_out[b][ch][e];
+// K3 == true: interpolation, entries j with three indices and weights each, value grad_out[b][ch][j] * weight[b][j][k].
+template <bool K3>
+__global__ __launch_bounds__(NTHREADS) void k_scatter_channel_last(int c, int n, int ne, const float* __restrict__ grad_out,
+                                                                   const int* __restrict__ idx, const float* __restrict__ weight,
+                                                                   float* __restrict__ out_cl) {
+  __shared__ float tile[64][65];
+  const int b = blockIdx.z, c0 = blockIdx.y * 64, e0 = blockIdx.x * 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int r = wave; r < 64; r += NTHREADS / 64) {
+    const int ch = c0 + r, e = e0 + lane;
+    tile[r][lane] = (ch < c && e < ne) ? grad_out[((long)b * c + ch) * ne + e] : 0.0f;
+  }
+  __syncthreads();
+  const int ch = c0 + lane;
+  for (int r = wave; r < 64; r += NTHREADS / 64) {
+    const int e = e0 + r;
+    if (e >= ne) break;  // wave-uniform
+    const float g = tile[lane][r];
+    if (K3) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const long o = ((long)b * ne + e) * 3 + k;
+        const int p = min(max(idx[o], 0), n - 1);
+        if (ch < c) unsafeAtomicAdd(out_cl + ((long)b * n + p) * c + ch, g * weight[o]);
+      }
+    } else {
+      const int p = min(max(idx[(long)b * ne + e], 0), n - 1);
+      if (ch < c) unsafeAtomicAdd(out_cl + ((long)b * n + p) * c + ch, g);
+    }
+  }
+}
+
+int launch_scatter_channel_last(bool k3, int b, int c, int n, int ne, const float* grad_out, const int* idx,
+                                const float* weight, float* out_cl, hipStream_t st) {
+  const dim3 g((ne + 63) / 64, (c + 63) / 64, b), t(NTHREADS);
+  if (k3) hipLaunchKernelGGL(k_scatter_channel_last<true>, g, t, 0, st, c, n, ne, grad_out, idx, weight, out_cl);
+  else hipLaunchKernelGGL(k_scatter_channel_last<false>, g, t, 0, st, c, n, ne, grad_out, idx, weight, out_cl);
+  return (int)hipGetLastError();
 }
 
 static unsigned blocks_for(long total) { return (unsigned)((total + NTHREADS - 1) / NTHREADS); }

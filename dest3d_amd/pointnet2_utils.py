@@ -129,10 +129,11 @@ class ThreeInterpolate(Function):
         g = _f(grad_out)
         Bsz, c, n = g.shape
         with torch.cuda.device(g.device):
-            out = torch.zeros((Bsz, c, m), dtype=torch.float32, device=g.device)
-            L.check(lib.issm_pn2_three_interpolate_grad(Bsz, c, n, m, g.data_ptr(), ix.data_ptr(), w.data_ptr(),
-                                                        out.data_ptr(), _st(g)), "issm_pn2_three_interpolate_grad")
-        return out.to(dt), None, None
+            # accumulated channel-last (coalesced atomics); the transpose is the gradient in the features' layout
+            out = torch.zeros((Bsz, m, c), dtype=torch.float32, device=g.device)
+            L.check(lib.issm_pn2_three_interpolate_grad_cl(Bsz, c, n, m, g.data_ptr(), ix.data_ptr(), w.data_ptr(),
+                                                           out.data_ptr(), _st(g)), "issm_pn2_three_interpolate_grad_cl")
+        return out.transpose(1, 2).to(dt), None, None
 
 
 three_interpolate = ThreeInterpolate.apply
@@ -161,10 +162,11 @@ class GroupingOperation(Function):
         g = _f(grad_out)
         Bsz, Cn, M, S = g.shape
         with torch.cuda.device(g.device):
-            out = torch.zeros((Bsz, Cn, N), dtype=torch.float32, device=g.device)
-            L.check(lib.issm_pn2_group_points_grad(Bsz, Cn, N, M, S, g.data_ptr(), ix.data_ptr(), out.data_ptr(), _st(g)),
-                    "issm_pn2_group_points_grad")
-        return out.to(dt), None
+            # accumulated channel-last (coalesced atomics); the transpose is the gradient in the features' layout
+            out = torch.zeros((Bsz, N, Cn), dtype=torch.float32, device=g.device)
+            L.check(lib.issm_pn2_group_points_grad_cl(Bsz, Cn, N, M, S, g.data_ptr(), ix.data_ptr(), out.data_ptr(), _st(g)),
+                    "issm_pn2_group_points_grad_cl")
+        return out.transpose(1, 2).to(dt), None
 
 
 grouping_operation = GroupingOperation.apply

@@ -397,6 +397,13 @@ int issm_pn2_three_interpolate(int32_t b, int32_t c, int32_t m, int32_t n, const
                                const float* weight, float* out, void* stream);
 int issm_pn2_three_interpolate_grad(int32_t b, int32_t c, int32_t n, int32_t m, const float* grad_out, const int32_t* idx,
                                     const float* weight, float* grad_points, void* stream);
+/* The same two gradients accumulated into a channel-last buffer, grad_points_cl (b, n, c) resp. (b, m, c), zeroed by
+ * the caller: its transpose is the reference's result.  No counterpart in the reference; the atomics then touch
+ * 64 consecutive floats per instruction instead of 64 scattered cache lines (about 10x faster at C = 128). */
+int issm_pn2_group_points_grad_cl(int32_t b, int32_t c, int32_t n, int32_t npoints, int32_t nsample, const float* grad_out,
+                                  const int32_t* idx, float* grad_points_cl, void* stream);
+int issm_pn2_three_interpolate_grad_cl(int32_t b, int32_t c, int32_t n, int32_t m, const float* grad_out,
+                                       const int32_t* idx, const float* weight, float* grad_points_cl, void* stream);
 
 #ifdef __cplusplus
 }

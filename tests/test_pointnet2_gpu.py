@@ -97,6 +97,36 @@ def test_group_and_gather_with_gradients():
     assert np.abs(f2.grad.cpu().numpy() - g1).max() <= 1e-5 * np.abs(g1).max()
 
 
+def test_reference_layout_gradient_entry_points():
+    """issm_pn2_group_points_grad / issm_pn2_three_interpolate_grad write the (b, c, n) layout directly (the Python
+    wrappers use the channel-last variants): called here through the C ABI."""
+    from dest3d_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(12)
+    B, C, N, M, S, n3 = 2, 70, 90, 11, 5, 33
+    idx = rng.integers(0, N, size=(B, M, S)).astype(np.int32)
+    gy = rng.standard_normal((B, C, M, S)).astype(np.float32)
+    tg, ti = _cuda(gy), _cuda(idx)
+    out = torch.zeros(B, C, N, device="cuda")
+    st = L.current_stream_ptr(out.device)
+    L.check(lib.issm_pn2_group_points_grad(B, C, N, M, S, tg.data_ptr(), ti.data_ptr(), out.data_ptr(), st), "group grad")
+    ref = R.group_points_grad(gy, idx, N)
+    assert np.abs(out.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    out_cl = torch.zeros(B, N, C, device="cuda")
+    L.check(lib.issm_pn2_group_points_grad_cl(B, C, N, M, S, tg.data_ptr(), ti.data_ptr(), out_cl.data_ptr(), st), "group grad cl")
+    assert np.abs(out_cl.transpose(1, 2).cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    i3 = rng.integers(0, N, size=(B, n3, 3)).astype(np.int32)
+    w3 = rng.uniform(0, 1, size=(B, n3, 3)).astype(np.float32)
+    g3 = rng.standard_normal((B, C, n3)).astype(np.float32)
+    out3 = torch.zeros(B, C, N, device="cuda")
+    tg3, ti3, tw3 = _cuda(g3), _cuda(i3), _cuda(w3)     # kept alive until the kernel has run
+    L.check(lib.issm_pn2_three_interpolate_grad(B, C, n3, N, tg3.data_ptr(), ti3.data_ptr(), tw3.data_ptr(),
+                                                out3.data_ptr(), st), "interp grad")
+    torch.cuda.synchronize()
+    ref3 = R.three_interpolate_grad(g3, i3, w3, N)
+    assert np.abs(out3.cpu().numpy() - ref3).max() <= 1e-5 * np.abs(ref3).max()
+
+
 def test_query_and_group_module():
     from dest3d_amd.pointnet2_utils import GroupAll, QueryAndGroup, furthest_point_sample, gather_operation
     rng = np.random.default_rng(8)
