@@ -272,6 +272,41 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
     return out
 
 
+def time_pointnet2_ops(torch, reps=5):
+    """The backbone's point-set operators at the detector's first set-abstraction shape (batch 8, 20000 points, 2048
+    centres, 64 samples, 128 / 256 channels), milliseconds per call."""
+    from dest3d_amd import pointnet2_utils as pn
+    torch.manual_seed(0)
+    B, N = 8, 20000
+    xyz = (8 * torch.rand(B, N, 3)).cuda()
+    feat = torch.randn(B, 128, N).cuda().requires_grad_()
+    res = {}
+
+    def t(name, fn):
+        out = fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            out = fn()
+        torch.cuda.synchronize()
+        res[name] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+        return out
+
+    fps = t("furthest_point_sample_2048_of_20000", lambda: pn.furthest_point_sample(xyz, 2048))
+    new_xyz = pn.gather_operation(xyz.transpose(1, 2).contiguous(), fps).transpose(1, 2).contiguous()
+    idx = t("ball_query_r0.2_64", lambda: pn.ball_query(0.2, 64, xyz, new_xyz))
+    g = t("grouping_c128_fwd", lambda: pn.grouping_operation(feat, idx))
+    gy = torch.randn_like(g)
+    t("grouping_c128_fwd_bwd", lambda: torch.autograd.grad(pn.grouping_operation(feat, idx), feat, gy))
+    d, i3 = t("three_nn_20000_x_2048", lambda: pn.three_nn(xyz, new_xyz))
+    w = torch.softmax(-d, -1)
+    f2 = torch.randn(B, 256, 2048).cuda().requires_grad_()
+    y = t("three_interpolate_c256_fwd", lambda: pn.three_interpolate(f2, i3, w))
+    gy2 = torch.randn_like(y)
+    t("three_interpolate_c256_fwd_bwd", lambda: torch.autograd.grad(pn.three_interpolate(f2, i3, w), f2, gy2))
+    return res
+
+
 def time_module_layer(torch, steps=10, warmup=3, dtype=None):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
@@ -311,6 +346,8 @@ def main():
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
     ap.add_argument("--only-layer", action="store_true",
                     help="time only the whole detector layer (module forward + backward) and print its JSON line")
+    ap.add_argument("--only-pointnet2", action="store_true",
+                    help="time only the backbone's point-set operators and print their JSON line (ms per call)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
     ap.add_argument("--traffic", type=float, default=None,
@@ -324,6 +361,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    if args.only_pointnet2:
+        print(json.dumps({"pointnet2_ops_ms": time_pointnet2_ops(torch)}))
+        return
     if args.only_layer:
         whole, enc = time_box_dist_layer(torch, args.steps, args.warmup)
         print(json.dumps({"detector_layer_bf16_fwd_bwd_us": round(time_module_layer(torch, args.steps, args.warmup), 2),

@@ -279,8 +279,12 @@ static unsigned blocks_for(long total) { return (unsigned)((total + NTHREADS - 1
 
 int launch_fps(int b, int n, int npoint, const float* xyz, float* temp, int* idxs, hipStream_t st) {
   const dim3 g(b), t(FPS_T);
-  if (n <= FPS_T * 8) hipLaunchKernelGGL(k_fps<8>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  if (n <= FPS_T * 4) hipLaunchKernelGGL(k_fps<4>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 8) hipLaunchKernelGGL(k_fps<8>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 16) hipLaunchKernelGGL(k_fps<16>, g, t, 0, st, n, npoint, xyz, temp, idxs);
   else if (n <= FPS_T * 24) hipLaunchKernelGGL(k_fps<24>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 32) hipLaunchKernelGGL(k_fps<32>, g, t, 0, st, n, npoint, xyz, temp, idxs);
+  else if (n <= FPS_T * 40) hipLaunchKernelGGL(k_fps<40>, g, t, 0, st, n, npoint, xyz, temp, idxs);
   else if (n <= FPS_T * 48) hipLaunchKernelGGL(k_fps<48>, g, t, 0, st, n, npoint, xyz, temp, idxs);
   else hipLaunchKernelGGL(k_fps<0>, g, t, 0, st, n, npoint, xyz, temp, idxs);
   return (int)hipGetLastError();
