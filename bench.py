@@ -272,6 +272,49 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
     return out
 
 
+def time_box_dist_vs_torch(torch, reps=3):
+    """BoxDistFun at the layer shape: the library's kernels against the same formulas written with PyTorch ops
+    (corner deltas, signed log, `grid_sample` on the (1, 16, 10, 10, 10) table, sum over corners -- the formulation of
+    models/dest_module.py:174-195 with zero angles), forward and forward + backward, milliseconds; and their largest
+    absolute difference."""
+    import torch.nn.functional as F
+    from dest3d_amd.box_dist import BoxDistFun, box_parametrization_to_corners
+    torch.manual_seed(0)
+    B, nP, nQ = 8, 1024, 256
+    bd = BoxDistFun(out_dim=16).cuda()
+    key_pos = 8.0 * torch.rand(B, nP, 3, device="cuda")
+    qpos = torch.cat([8.0 * torch.rand(B, nQ, 3, device="cuda"), 0.2 + 2.0 * torch.rand(B, nQ, 3, device="cuda")], -1)
+    ang = torch.zeros(B, nQ, device="cuda")
+
+    def with_torch_ops():
+        corners = box_parametrization_to_corners(qpos[..., :3], qpos[..., 3:], ang).detach()
+        deltas = corners.reshape(B, -1, 3)[:, :, None, :] - key_pos[:, None, :, :]
+        deltas = torch.sign(deltas) * torch.log2(torch.abs(deltas) * 512 + 1.0) / math.log2(8)
+        rpe = F.grid_sample(bd.rpe_table()[None], (deltas / 4.0).view(1, 1, 1, -1, 3), mode="bilinear",
+                            align_corners=False).reshape(-1, B, nQ, 8, nP)
+        return rpe.sum(dim=-2).permute(1, 3, 2, 0)
+
+    def with_kernels():
+        return bd(key_pos, qpos[..., :3], qpos[..., 3:], ang)
+
+    res = {}
+    for name, fn in (("kernels", with_kernels), ("torch_ops", with_torch_ops)):
+        for bw in (False, True):
+            for i in range(reps + 1):
+                if i == 1:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                bd.zero_grad(set_to_none=True)
+                d = fn()
+                if bw:
+                    d.square().sum().backward()
+            torch.cuda.synchronize()
+            res[f"{name}_{'fwd_bwd' if bw else 'fwd'}_ms"] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+    with torch.no_grad():
+        res["max_abs_difference"] = float((with_kernels() - with_torch_ops()).abs().max())
+    return res
+
+
 def time_pointnet2_ops(torch, reps=5):
     """The backbone's point-set operators at the detector's first set-abstraction shape (batch 8, 20000 points, 2048
     centres, 64 samples, 128 / 256 channels), milliseconds per call."""
@@ -346,6 +389,8 @@ def main():
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
     ap.add_argument("--only-layer", action="store_true",
                     help="time only the whole detector layer (module forward + backward) and print its JSON line")
+    ap.add_argument("--only-box-dist", action="store_true",
+                    help="time BoxDistFun: the kernels against the same formulas in PyTorch ops, and print the JSON line")
     ap.add_argument("--only-pointnet2", action="store_true",
                     help="time only the backbone's point-set operators and print their JSON line (ms per call)")
     ap.add_argument("--calib-copy", action="store_true",
@@ -361,6 +406,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    if args.only_box_dist:
+        print(json.dumps({"box_dist_8x1024x256": time_box_dist_vs_torch(torch)}))
+        return
     if args.only_pointnet2:
         print(json.dumps({"pointnet2_ops_ms": time_pointnet2_ops(torch)}))
         return

@@ -113,7 +113,8 @@ class BoxDistArgs(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("seqlen", C.c_int32), ("nquery", C.c_int32),
         ("D", C.c_int32), ("H", C.c_int32), ("W", C.c_int32), ("dtype", C.c_int32),
-        ("key", C.c_void_p), ("corners", C.c_void_p), ("angle", C.c_void_p), ("table", C.c_void_p),
+        ("key", C.c_void_p), ("corners", C.c_void_p), ("boxes", C.c_void_p), ("min_radius", C.c_float),
+        ("angle", C.c_void_p), ("table", C.c_void_p),
         ("log_scale", C.c_float), ("max_value", C.c_float),
         ("dist", C.c_void_p), ("qcenter", C.c_void_p), ("radius", C.c_void_p),
         ("weight_dist", C.c_float), ("weights", C.c_void_p),

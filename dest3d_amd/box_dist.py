@@ -52,10 +52,16 @@ class BoxDistFn(torch.autograd.Function):
         Bsz, nP = key_xyz.shape[:2]
         nQ = corners.shape[1]
         key, cor, ang = _f32c(key_xyz), _f32c(corners), _f32c(angle)
+        as_boxes = cor.dim() == 3          # (B, nQ, 7) boxes instead of (B, nQ, 8, 3) corners
+        assert cor.shape[2:] == ((7,) if as_boxes else (8, 3))
         a = L.BoxDistArgs()
         a.batch, a.seqlen, a.nquery = Bsz, nP, nQ
         a.dtype = L.dtype_code(out_dtype)
-        a.key, a.corners = key.data_ptr(), cor.data_ptr()
+        a.key = key.data_ptr()
+        if as_boxes:
+            a.boxes, a.min_radius = cor.data_ptr(), 0.64
+        else:
+            a.corners = cor.data_ptr()
         a.angle = None if ang is None else ang.data_ptr()
         a.log_scale, a.max_value = float(log_scale), float(max_value)
         a.stream = L.current_stream_ptr(key.device)
@@ -70,9 +76,13 @@ class BoxDistFn(torch.autograd.Function):
                 dist = torch.empty((Bsz, nP, nQ, CHANNELS), dtype=out_dtype, device=key.device)
                 a.dist = dist.data_ptr()
             if want_weights:
-                qc, rad = _f32c(qcenter), _f32c(radius)
                 weights = torch.empty((Bsz, nP, nQ), dtype=torch.float32, device=key.device)
-                a.qcenter, a.radius, a.weight_dist = qc.data_ptr(), rad.data_ptr(), float(weight_dist)
+                a.weight_dist = float(weight_dist)
+                if qcenter is not None:
+                    qc, rad = _f32c(qcenter), _f32c(radius)
+                    a.qcenter, a.radius = qc.data_ptr(), rad.data_ptr()
+                else:
+                    assert as_boxes, "weights need (qcenter, radius) or boxes"
                 a.weights = weights.data_ptr()
             L.check(lib.issm_box_dist_fwd(C.byref(a)), "issm_box_dist_fwd")
         ctx.save_for_backward(key, cor, ang)
@@ -95,7 +105,11 @@ class BoxDistFn(torch.autograd.Function):
                 a = L.BoxDistArgs()
                 a.batch, a.seqlen, a.nquery, a.D, a.H, a.W = Bsz, nP, nQ, D, H, W
                 a.dtype = L.dtype_code(out_dtype)
-                a.key, a.corners = key.data_ptr(), cor.data_ptr()
+                a.key = key.data_ptr()
+                if cor.dim() == 3:
+                    a.boxes, a.min_radius = cor.data_ptr(), 0.64
+                else:
+                    a.corners = cor.data_ptr()
                 a.angle = None if ang is None else ang.data_ptr()
                 a.log_scale, a.max_value = float(log_scale), float(max_value)
                 nbytes = lib.issm_box_dist_bwd_scratch_bytes(Bsz, nP, nQ, D, H, W)
@@ -150,14 +164,20 @@ class BoxDistFun(nn.Module):
     def forward(self, key_xyz, query_xyz, query_size, query_angle, weight_query_pos=None, weight_dist=15.0):
         """-> dist (B, nP, nQ, out_dim).  With ``weight_query_pos`` (B, nQ, 6) the locality weights (B, nP, nQ)
         of ``local_weight`` are computed in the same pass and returned as a second value."""
-        corners = box_parametrization_to_corners(query_xyz.float(), query_size.float(), query_angle.float()).detach()
+        # the kernel derives the corners (and, for the weights, centre and radius) from the boxes themselves
+        boxes = torch.cat([query_xyz, query_size, query_angle.unsqueeze(-1)], dim=-1).detach()
         table = self.rpe_table()
         out_dtype = table.dtype if table.dtype in (torch.float32, torch.bfloat16) else torch.float32
-        # an all-zero angle (what the decoder passes, dest_module.py:284) needs no rotation
-        angle = query_angle
         if weight_query_pos is None:
-            return BoxDistFn.apply(table, key_xyz, corners, angle, None, None, 0.0, self.log_scale, self.max_value,
+            return BoxDistFn.apply(table, key_xyz, boxes, query_angle, None, None, 0.0, self.log_scale, self.max_value,
                                    out_dtype, True, False)[0]
-        radius = weight_query_pos[..., 3:].float().square().sum(-1).sqrt().clamp_min(0.64)
-        return BoxDistFn.apply(table, key_xyz, corners, angle, weight_query_pos[..., :3], radius, float(weight_dist),
-                               self.log_scale, self.max_value, out_dtype, True, True)
+        same_boxes = (weight_query_pos.shape[-1] == 6 and query_xyz.data_ptr() == weight_query_pos.data_ptr()
+                      and query_size.data_ptr() == weight_query_pos[..., 3:].data_ptr()
+                      and query_xyz.stride() == weight_query_pos[..., :3].stride())
+        if same_boxes:        # query_pos[..., :3] / query_pos[..., 3:], as the decoder layer calls it
+            qc = rad = None   # the weight's boxes are the encoding's: centre and radius come from `boxes`
+        else:
+            qc = weight_query_pos[..., :3]
+            rad = weight_query_pos[..., 3:].float().square().sum(-1).sqrt().clamp_min(0.64)
+        return BoxDistFn.apply(table, key_xyz, boxes, query_angle, qc, rad, float(weight_dist), self.log_scale,
+                               self.max_value, out_dtype, True, True)

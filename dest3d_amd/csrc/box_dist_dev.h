@@ -13,25 +13,50 @@ struct BoxLane {
   float qx, qy, qz, radius;
 };
 
+// Corner c of box k: from the corner tensor, or from the box itself -- boxes (B, K, 7) = centre, size (l, w, h),
+// heading -- with the reference's corner order (dest_module.py:62-70 after the axis changes of :26-38):
+//   x = cx + sx l/2 cos + sz w/2 sin,  y = cy - sx l/2 sin + sz w/2 cos,  z = cz - sy h/2,
+//   sx = + + - - + + - -,  sy = + + + + - - - -,  sz = + - - + + - - +.
+__device__ __forceinline__ void box_corner(const BoxDistP& p, int b, int k, int c, float& x, float& y, float& z) {
+  if (p.boxes) {  // uniform
+    const float* q = p.boxes + ((long)b * p.K + k) * 7;
+    const float lx = ((c & 2) ? -0.5f : 0.5f) * q[3];
+    const float hy = ((c & 4) ? -0.5f : 0.5f) * q[5];
+    const float wz = (((c ^ (c >> 1)) & 1) ? -0.5f : 0.5f) * q[4];
+    const float cs = cosf(q[6]), sn = sinf(q[6]);
+    x = q[0] + lx * cs + wz * sn;
+    y = q[1] - lx * sn + wz * cs;
+    z = q[2] - hy;
+  } else {
+    const float* q = p.corners + (((long)b * p.K + k) * 8 + c) * 3;
+    x = q[0]; y = q[1]; z = q[2];
+  }
+}
+// rotation applied to the deltas of corner c of box k: the angle of query (8k + c) mod K, as the reference's tiling
+__device__ __forceinline__ void corner_rotation(const BoxDistP& p, int b, int k, int c, float& cs, float& sn) {
+  cs = 1.0f;
+  sn = 0.0f;
+  if (p.angle) {  // uniform
+    const float a = p.angle[(long)b * p.K + (k * 8 + c) % p.K];
+    cs = cosf(a);
+    sn = sinf(a);
+  }
+}
+
 __device__ __forceinline__ void load_box(const BoxDistP& p, int b, int k, BoxLane& bx) {
-  const float* c = p.corners + ((long)b * p.K + k) * 24;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    bx.cx[j] = c[3 * j];
-    bx.cy[j] = c[3 * j + 1];
-    bx.cz[j] = c[3 * j + 2];
-    bx.cs[j] = 1.0f;
-    bx.sn[j] = 0.0f;
-    if (p.angle) {  // uniform
-      const float a = p.angle[(long)b * p.K + (k * 8 + j) % p.K];
-      bx.cs[j] = cosf(a);
-      bx.sn[j] = sinf(a);
-    }
+    box_corner(p, b, k, j, bx.cx[j], bx.cy[j], bx.cz[j]);
+    corner_rotation(p, b, k, j, bx.cs[j], bx.sn[j]);
   }
   if (p.qcenter) {
     const float* q = p.qcenter + ((long)b * p.K + k) * 3;
     bx.qx = q[0]; bx.qy = q[1]; bx.qz = q[2];
     bx.radius = p.radius[(long)b * p.K + k];
+  } else if (p.boxes) {  // locality weight from the box: centre, radius = max(|size|, min_radius)
+    const float* q = p.boxes + ((long)b * p.K + k) * 7;
+    bx.qx = q[0]; bx.qy = q[1]; bx.qz = q[2];
+    bx.radius = fmaxf(sqrtf(q[3] * q[3] + q[4] * q[4] + q[5] * q[5]), p.min_radius);
   }
 }
 

@@ -219,18 +219,13 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
       const int l = (int)(bl % (unsigned)p.L), b = (int)(bl / (unsigned)p.L);
       const float* key = p.key + ((long)b * p.L + l) * 3;
       const float kx = key[0], ky = key[1], kz = key[2];
-      const float* cor = p.corners + ((long)b * p.K + k) * 24;
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (mask & (1u << c)) {
-          float cs = 1.0f, sn = 0.0f;
-          if (p.angle) {  // uniform
-            const float a = p.angle[(long)b * p.K + (k * 8 + c) % p.K];
-            cs = cosf(a);
-            sn = sinf(a);
-          }
-          float x, y, z;
-          corner_pos(p, cor[3 * c], cor[3 * c + 1], cor[3 * c + 2], cs, sn, kx, ky, kz, scale, x, y, z);
+          float cx, cy, cz, cs, sn, x, y, z;
+          box_corner(p, b, k, c, cx, cy, cz);
+          corner_rotation(p, b, k, c, cs, sn);
+          corner_pos(p, cx, cy, cz, cs, sn, kx, ky, kz, scale, x, y, z);
           const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
           float ax[3], ay[3], az[3];
           axis3((int)gx, x - gx, mx, ax);

@@ -513,10 +513,11 @@ static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
   if ((int64_t)a->D * a->H * a->W > 1024)
     return fail(ISSM_E_UNSUPPORTED, "box_dist: table of %d x %d x %d nodes (at most 1024 fit)", a->D, a->H, a->W);
   if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "box_dist: dtype %d", a->dtype);
-  if (!a->key || !a->corners) return fail(ISSM_E_NULL, "box_dist: key/corners is NULL");
+  if (!a->key || (!a->corners && !a->boxes)) return fail(ISSM_E_NULL, "box_dist: key or corners/boxes is NULL");
   if (!bwd) {
     if (a->dist && !a->table) return fail(ISSM_E_NULL, "box_dist: table is NULL");
-    if (a->weights && (!a->qcenter || !a->radius)) return fail(ISSM_E_NULL, "box_dist: qcenter/radius is NULL");
+    if (a->weights && !a->boxes && (!a->qcenter || !a->radius)) return fail(ISSM_E_NULL, "box_dist: qcenter/radius is NULL");
+    if (a->qcenter && !a->radius) return fail(ISSM_E_NULL, "box_dist: radius is NULL");
   } else if (!a->ddist || !a->partial || !a->dtable) {
     return fail(ISSM_E_NULL, "box_dist bwd: ddist/partial/dtable is NULL");
   }
@@ -525,7 +526,8 @@ static int box_dist_params(const issm_box_dist_args* a, BoxDistP* p, bool bwd) {
   p->nwg_bwd = box_dist_bwd_workgroups(a->batch, a->seqlen, a->nquery);
   if (bwd && (int64_t)a->batch * a->seqlen * a->nquery > ((int64_t)1 << 26))
     return fail(ISSM_E_UNSUPPORTED, "box_dist bwd: more than 2^26 (point, box) pairs");
-  p->key = a->key; p->corners = a->corners; p->angle = a->angle; p->table = a->table;
+  p->key = a->key; p->corners = a->corners; p->boxes = a->corners ? nullptr : a->boxes; p->min_radius = a->min_radius;
+  p->angle = a->angle; p->table = a->table;
   p->log_scale = a->log_scale; p->max_value = a->max_value; p->dist = a->dist;
   p->qcenter = a->qcenter; p->radius = a->radius; p->weight_dist = a->weight_dist; p->weights = a->weights;
   p->ddist = a->ddist; p->partial = a->partial; p->dtable = a->dtable;

@@ -92,7 +92,9 @@ struct HilbertP {
 struct BoxDistP {
   int B, L, K, D, H, W, dtype, nwg, nwg_bwd;
   const float* key;      // (B, L, 3)
-  const float* corners;  // (B, K, 8, 3)
+  const float* corners;  // (B, K, 8, 3), or NULL with boxes given
+  const float* boxes;    // (B, K, 7) centre, size, heading: corners (and the weight's centre / radius) derived from it
+  float min_radius;
   const float* angle;    // (B, K) or NULL (zero)
   const float* table;    // (16, D, H, W)
   float log_scale, max_value;

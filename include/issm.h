@@ -315,7 +315,10 @@ int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
  *     grid_sample(mode bilinear, padding zeros, align_corners False) with x indexing W, y H, z D;
  *   weights[b][l][k] = exp(weight_dist * min(radius[b][k] - |key_l - qcenter[b][k]|, 0)).
  * key (B, L, 3), corners (B, K, 8, 3), angle (B, K), table (16, D, H, W) with D*H*W <= 1024, qcenter (B, K, 3),
- * radius (B, K), weights (B, L, K), dtable (16, D, H, W): fp32 contiguous.  dist and ddist: (B, L, K, 16)
+ * radius (B, K), weights (B, L, K), dtable (16, D, H, W): fp32 contiguous.  Instead of corners (and of qcenter /
+ * radius) the boxes themselves may be given: boxes (B, K, 7) = centre, size (l, w, h), heading; the corners are
+ * then those of box_parametrization_to_corners (dest_module.py:99-103) and, for the weights, the centre is the
+ * box's and radius = max(|size|, min_radius).  dist and ddist: (B, L, K, 16)
  * contiguous in `dtype`.  Either output of the forward may be NULL (skipped).  The backward produces the table
  * gradient only (the reference detaches the corners; key positions and angles are inputs); partial:
  * issm_box_dist_bwd_scratch_bytes(...) bytes of scratch, 16-byte aligned (about 64 bytes per pair for large
@@ -327,6 +330,8 @@ typedef struct issm_box_dist_args {
   int32_t dtype;
   const float* key;
   const float* corners;
+  const float* boxes;
+  float min_radius;
   const float* angle;
   const float* table;
   float log_scale, max_value;

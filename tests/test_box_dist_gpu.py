@@ -72,7 +72,8 @@ def test_local_weight_and_fused_module_call():
     table = m.rpe_table().detach().double().cpu().numpy()
     ref = R.box_dist(key, qxyz, qsize, ang, table)
     assert _rel(dist.detach().cpu().numpy(), ref) <= 1e-4
-    assert torch.equal(w2, w)
+    # the fused call derives centre and radius from the boxes inside the kernel: equal up to the rounding of the radius
+    assert torch.allclose(w2, w, rtol=2e-4, atol=1e-7)
     dist.square().sum().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
     # gradient of the MLP through the table: against autograd of the same MLP fed the oracle's table gradient
