@@ -1,0 +1,168 @@
+"""The core of MultiHeadISSMScan as one autograd node.
+
+Between the input projections and the output projections, MultiHeadISSMScan.forward (models/dest_module.py:528-581)
+is a fixed chain: depthwise conv + SiLU of both branches, generation of dt / B / C from the distance encoding, the
+bidirectional scan, the average of the two directions, the gated RMSNorm.  Run as separate autograd Functions and
+PyTorch ops that is some forty small operations forward and as many autograd nodes backward, and at the detector's
+layer shape the host cannot issue them as fast as the GPU finishes them.  ``fused_scan_core`` makes the same calls
+into libissm_hip.so back to back inside one Function and chains their backward passes by hand; the arithmetic is the
+kernels' either way.  Used by ``scan_module.MultiHeadISSMScan`` for the bidirectional configuration with a distance
+encoding the generation kernel is built for; every other configuration takes the step-by-step path."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib as L
+from . import dwconv as _dw
+from . import layernorm_gated as _ln
+from . import param_gen as _pg
+from .issm_combined import _Problem, _scan_bwd, _scan_fwd
+
+
+def _kdt(t):
+    return t.dtype if t.dtype in (torch.float32, torch.bfloat16) else torch.float32
+
+
+class FusedScanCoreFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, zxbcdt, h0_lin, dist, weights, conv_w_f, conv_b_f, conv_w_b, conv_b_b, dt_w, bc_w, dt_bias, A_log, D,
+                norm_w, d_inner, nheads, ngroups, chunk_size, dt_limit, eps):
+        lib = L.load()
+        dev = zxbcdt.device
+        Bsz, Ln, _ = zxbcdt.shape
+        H, G, di = nheads, ngroups, d_inner
+        P, Cc = di // H, di + 2 * G
+        K = dist.shape[2]
+        kdt = _kdt(zxbcdt)
+        zx = zxbcdt.detach().to(kdt)
+        if zx.stride(-1) != 1:
+            zx = zx.contiguous()
+        z, xbc, dt_tok = zx[..., :di], zx[..., di:di + Cc], zx[..., di + Cc:]
+        with torch.cuda.device(dev):
+            st = L.current_stream_ptr(dev)
+            # 1. both depthwise convolutions + SiLU
+            cw = torch.stack([conv_w_f.detach().reshape(Cc, _dw.TAPS), conv_w_b.detach().reshape(Cc, _dw.TAPS)]).float()
+            cb = torch.stack([conv_b_f.detach(), conv_b_b.detach()]).float()
+            y = torch.empty((2, Bsz, Ln, Cc), dtype=kdt, device=dev)
+            pre = torch.empty_like(y)
+            a = _dw._args(xbc, 2)
+            a.w, a.bias, a.y, a.pre = cw.data_ptr(), cb.data_ptr(), y.data_ptr(), pre.data_ptr()
+            L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "issm_dwconv_silu_fwd")
+            x_f = y[0, ..., :di].contiguous().view(Bsz, Ln, H, P)
+            x_b = y[1, ..., :di].contiguous().view(Bsz, Ln, H, P)
+            # 2. dt / B / C (and the reversed-order B / C) from the distance encoding
+            bias = torch.cat([dt_tok.float() + dt_bias.detach().float(), y[0, ..., di:].float(), y[1, ..., di:].float()], -1)
+            W = torch.cat([dt_w.detach(), bc_w.detach()], 0).float()
+            d = dist.detach().to(kdt).contiguous()
+            wt = None if weights is None else weights.detach().float().contiguous()
+            dt = torch.empty((Bsz, Ln, H, K), dtype=kdt, device=dev)
+            bc = [torch.empty((Bsz, Ln, G, K), dtype=kdt, device=dev) for _ in range(4)]
+            raw = torch.empty_like(dt) if wt is not None else None
+            g = _pg._args(d, W, H, G, True)
+            g.bias = bias.data_ptr()
+            g.dt, g.Bm, g.Cm, g.Bm_back, g.Cm_back = (t.data_ptr() for t in (dt, *bc))
+            if wt is not None:
+                g.weights, g.dt_raw = wt.data_ptr(), raw.data_ptr()
+            L.check(lib.issm_param_gen_fwd(C.byref(g)), "issm_param_gen_fwd")
+            # 3. the bidirectional scan, queries as initial state
+            A = (-torch.exp(A_log.detach().float()))[:, None].expand(H, K)
+            h0 = h0_lin.detach().reshape(Bsz, K, H, P).permute(0, 2, 3, 1)
+            prob = _Problem([x_f, x_b], dt, A, [bc[0], bc[2]], [bc[1], bc[3]], chunk_size, D.detach(), [None, None], None,
+                            h0, None, wt is None, dt_limit)
+            outs, finals, ws = _scan_fwd(prob, True)
+            key = torch.add(outs[0], outs[1]).mul_(0.5).view(Bsz * Ln, di)
+            # 4. gated RMSNorm (norm(x * silu(z)))
+            z2 = z.reshape(Bsz * Ln, di) if z.is_contiguous() else z.as_strided((Bsz * Ln, di), (zx.stride(1), 1),
+                                                                                 z.storage_offset())
+            nw = norm_w.detach()
+            nw = (nw if nw.dtype in (torch.float32, torch.bfloat16) else nw.float()).contiguous()
+            key_n = torch.empty_like(key)
+            rstd = torch.empty(Bsz * Ln, dtype=torch.float32, device=dev)
+            n = _ln._norm_args(key, z2, nw, eps, None, False)
+            n.y, n.y_row_stride, n.rstd = key_n.data_ptr(), key_n.stride(0), rstd.data_ptr()
+            L.check(lib.issm_gated_rmsnorm_fwd(C.byref(n)), "issm_gated_rmsnorm_fwd")
+            last = torch.add(finals[0], finals[1]).mul_(0.5).permute(0, 3, 1, 2).reshape(Bsz, K, di)
+        ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log.detach())
+        ctx.prob, ctx.ws = prob, ws
+        ctx.meta = (Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, st)
+        ctx.dtypes = tuple(t.dtype for t in (zxbcdt, h0_lin, dist, conv_w_f, conv_b_f, conv_w_b, conv_b_b, dt_w, bc_w,
+                                              dt_bias, A_log, D, norm_w))
+        ctx.shapes = (conv_w_f.shape, conv_w_b.shape)
+        return key_n.view(Bsz, Ln, di).to(zxbcdt.dtype), last.to(h0_lin.dtype)
+
+    @staticmethod
+    def backward(ctx, dkey_n, dlast):
+        lib = L.load()
+        xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log = ctx.saved_tensors
+        Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, _ = ctx.meta
+        prob = ctx.prob
+        dev = key.device
+        (zdt, hdt, ddt_, wfdt, bfdt, wbdt, bbdt, dtwdt, bcwdt, dtbdt, aldt, Ddt, nwdt) = ctx.dtypes
+        with torch.cuda.device(dev):
+            # 4'. gated RMSNorm
+            dy = dkey_n.to(kdt).reshape(Bsz * Ln, di).contiguous()
+            dkey = torch.empty_like(key)
+            dz = torch.empty_like(key)
+            nb = lib.issm_rmsnorm_bwd_blocks(Bsz * Ln)
+            dwp = torch.empty((nb, di), dtype=torch.float32, device=dev)
+            dnw = torch.empty(di, dtype=torch.float32, device=dev)
+            n = _ln._norm_args(key, z2, nw, eps, None, False)
+            n.rstd = rstd.data_ptr()
+            n.dy, n.dy_row_stride = dy.data_ptr(), dy.stride(0)
+            n.dx, n.dx_row_stride = dkey.data_ptr(), dkey.stride(0)
+            n.dz, n.dz_row_stride = dz.data_ptr(), dz.stride(0)
+            n.dw_partial, n.dw = dwp.data_ptr(), dnw.data_ptr()
+            L.check(lib.issm_gated_rmsnorm_bwd(C.byref(n)), "issm_gated_rmsnorm_bwd")
+            # 3'. the scan: both directions receive half of the averaged outputs' gradients
+            dyh = dkey.mul_(0.5).view(Bsz, Ln, H, P)
+            dfin = dlast.float().reshape(Bsz, K, H, P).permute(0, 2, 3, 1).mul(0.5).contiguous()
+            dxs, ddt, dA, dBs, dCs, dD, _, _, dh0 = _scan_bwd(prob, ctx.ws, [dyh, dyh], [dfin, dfin], want_dz=False)
+            # 2'. parameter generation
+            R0, R = H + 2 * G, H + 4 * G
+            g = _pg._args(d, W, H, G, True)
+            g.ddt, g.dBm, g.dCm, g.dBm_back, g.dCm_back = (t.data_ptr() for t in (ddt, dBs[0], dCs[0], dBs[1], dCs[1]))
+            ddist = torch.empty_like(d) if ctx.needs_input_grad[2] else None
+            dbias = torch.empty((Bsz, Ln, R), dtype=torch.float32, device=dev)
+            nbp = lib.issm_param_gen_bwd_blocks(Bsz * Ln)
+            dwpart = torch.empty((max(nbp, 1), R0, 16), dtype=torch.float32, device=dev)
+            dW = torch.empty((R0, 16), dtype=torch.float32, device=dev)
+            g.ddist = None if ddist is None else ddist.data_ptr()
+            g.dbias, g.dw_partial, g.dW = dbias.data_ptr(), dwpart.data_ptr(), dW.data_ptr()
+            if wt is not None:
+                g.weights, g.dt_raw = wt.data_ptr(), raw.data_ptr()
+            L.check(lib.issm_param_gen_bwd(C.byref(g)), "issm_param_gen_bwd")
+            d_dt_tok = dbias[..., :H]
+            # 1'. the convolutions: gradients of (x, b-bias, c-bias) per branch
+            dyc = [torch.cat([dxs[0].view(Bsz, Ln, di), dbias[..., H:H + 2 * G].to(kdt)], -1),
+                   torch.cat([dxs[1].view(Bsz, Ln, di), dbias[..., H + 2 * G:].to(kdt)], -1)]
+            dxbc = torch.empty((Bsz, Ln, Cc), dtype=kdt, device=dev)
+            rows = lib.issm_dwconv_partial_rows(Bsz, Ln)
+            part = torch.empty((max(rows, 1), 2, 8, Cc), dtype=torch.float32, device=dev)
+            dcw = torch.empty((2, Cc, _dw.TAPS), dtype=torch.float32, device=dev)
+            dcb = torch.empty((2, Cc), dtype=torch.float32, device=dev)
+            a = _dw._args(xbc, 2)
+            a.w, a.pre = cw.data_ptr(), pre.data_ptr()
+            a.dy[0], a.dy[1] = dyc[0].data_ptr(), dyc[1].data_ptr()
+            a.du, a.partial, a.dw, a.dbias = dxbc.data_ptr(), part.data_ptr(), dcw.data_ptr(), dcb.data_ptr()
+            L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "issm_dwconv_silu_bwd")
+            dzx = torch.cat([dz.view(Bsz, Ln, di), dxbc, d_dt_tok.to(kdt)], -1)
+            dA_log = dA.sum(-1).mul_(-torch.exp(A_log.float()))
+            dh0_lin = dh0.permute(0, 3, 1, 2).reshape(Bsz, K, di)
+            ddt_bias = d_dt_tok.sum((0, 1))
+        wf_shape, wb_shape = ctx.shapes
+        return (dzx.to(zdt), dh0_lin.to(hdt), None if ddist is None else ddist.to(ddt_), None,
+                dcw[0].reshape(wf_shape).to(wfdt), dcb[0].to(bfdt), dcw[1].reshape(wb_shape).to(wbdt), dcb[1].to(bbdt),
+                dW[:H].to(dtwdt), dW[H:].to(bcwdt), ddt_bias.to(dtbdt), dA_log.to(aldt), dD.to(Ddt), dnw.to(nwdt),
+                None, None, None, None, None, None)
+
+
+def fused_scan_core(zxbcdt, h0_lin, dist, weights, conv_f, conv_b, dt_proj_w, bc_proj_w, dt_bias, A_log, D, norm_w, d_inner,
+                    nheads, ngroups, chunk_size, dt_limit, eps):
+    """zxbcdt (B, L, 2 d_inner + 2G + H): output of key_proj; h0_lin (B, K, d_inner): output of query_proj;
+    dist (B, L, K, 16); weights (B, L, K) fp32 or None; conv_f / conv_b: the two depthwise Conv1d modules.
+    Returns the normalised key (B, L, d_inner) and the averaged final state (B, K, d_inner)."""
+    return FusedScanCoreFn.apply(zxbcdt, h0_lin, dist, weights, conv_f.weight, conv_f.bias, conv_b.weight, conv_b.bias,
+                                 dt_proj_w, bc_proj_w, dt_bias, A_log, D, norm_w, d_inner, nheads, ngroups, chunk_size,
+                                 tuple(dt_limit), eps)

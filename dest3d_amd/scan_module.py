@@ -24,6 +24,7 @@ import torch.nn.functional as F
 
 from . import param_gen
 from .dwconv import dwconv_silu
+from .fused_layer import fused_scan_core
 from .issm_combined import ISSM_biscan_combined, ISSM_chunk_scan_combined
 from .layernorm_gated import RMSNorm as RMSNormGated
 
@@ -54,6 +55,7 @@ class MultiHeadISSMScan(nn.Module):
         self.headdim = self.d_inner // nheads
         self.dt_limit = dt_limit
         self.layer_idx = layer_idx
+        self.fused = True   # run the chain between the projections as one autograd node when the configuration allows
 
         # [z, x, b_bias, c_bias, dt_bias] from the key tokens (dest_module.py:471-474)
         self.key_proj = nn.Linear(d_model, 2 * self.d_inner + 2 * ngroups + nheads, bias=False)
@@ -147,6 +149,16 @@ class MultiHeadISSMScan(nn.Module):
     def forward(self, in_key, in_query, dist, key_xyz, mask=None):
         """in_key (B,L,D), in_query (B,K,D), dist (B,L,K,M), mask (B,L,K) float weights or bool
         "drop" flags -> out_key (B,L,D), out_query (B,K,D)   (dest_module.py:515-585)."""
+        if self.fused and self.use_biscan and param_gen.supported(dist, self.nheads, self.ngroups) and \
+                not (mask is not None and mask.requires_grad):
+            # the whole chain between the projections as one autograd node (same kernels, far fewer host operations)
+            wts = None if mask is None else (mask.float() if mask.is_floating_point() else (~mask).float())
+            key, last = fused_scan_core(self.key_proj(in_key), self.query_proj(in_query), dist, wts,
+                                        self.key_conv.dwconv, self.key_conv_back.dwconv, self.dt_proj.weight,
+                                        self.bc_proj.weight, self.dt_bias, self.A_log, self.D, self.key_norm.weight,
+                                        self.d_inner, self.nheads, self.ngroups, self.chunk_size, self.dt_limit,
+                                        self.key_norm.eps)
+            return self.out_key_proj(key), self.out_query_proj(self.query_norm(last))
         s = self.scan_inputs(in_key, in_query, dist, key_xyz, mask)
         kw = dict(D=self.D, initial_states=s["initial_states"], dt_softplus=s["softplus_in_kernel"],
                   dt_limit=self.dt_limit)

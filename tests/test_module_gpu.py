@@ -69,7 +69,7 @@ def _module_ref(sd, cfg, in_key, in_query, dist, mask):
     return out_key, last @ sd["out_query_proj.weight"].T
 
 
-@pytest.mark.parametrize("biscan,mask_kind", [(True, None), (True, "float"), (False, "bool")])
+@pytest.mark.parametrize("biscan,mask_kind", [(True, None), (True, "float"), (True, "bool"), (False, "bool"), (False, "float")])
 def test_module_matches_fp64_evaluation(biscan, mask_kind):
     from dest3d_amd.scan_module import MultiHeadISSMScan
     print(f"[case] module mirror biscan={biscan} mask={mask_kind}", flush=True)
