@@ -106,6 +106,7 @@ class DwConvArgs(C.Structure):
         ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("pre", C.c_void_p),
         ("dy", C.c_void_p * 2), ("du", C.c_void_p), ("partial", C.c_void_p), ("dw", C.c_void_p),
         ("dbias", C.c_void_p), ("stream", C.c_void_p),
+        ("split", C.c_int32), ("y_tail", C.c_void_p), ("dy_tail", C.c_void_p * 2),
     ]
 
 

@@ -72,7 +72,14 @@ __global__ __launch_bounds__(NTHREADS) void k_dwconv_fwd(DwConvP p) {
         const long o = (((long)s * p.B + b) * p.L + l) * p.C + c;
         if (BF) a = bf16_to_f(f_to_bf16(a));  // the saved pre-activation is what the backward differentiates
         dw_st<BF>(p.pre, o, a);
-        dw_st<BF>(p.y, o, a * sigmoidf_(a));
+        const float yv = a * sigmoidf_(a);
+        if (p.split > 0) {  // uniform: channels [0, split) and [split, C) go to two dense tensors
+          const long row = ((long)s * p.B + b) * p.L + l;
+          if (c < p.split) dw_st<BF>(p.y, row * p.split + c, yv);
+          else dw_st<BF>(p.y_tail, row * (p.C - p.split) + (c - p.split), yv);
+        } else {
+          dw_st<BF>(p.y, o, yv);
+        }
       }
     }
   }
@@ -102,7 +109,13 @@ __global__ __launch_bounds__(NTHREADS) void k_dwconv_bwd(DwConvP p) {
     for (int s = 0; s < S; ++s) {
       const long o = ((long)b * p.L + lc) * p.C + c;
       float dyv = 0.0f;
-      if (p.dy[s]) dyv = dw_ld<BF>(p.dy[s], o);  // uniform
+      if (p.split > 0) {  // uniform: the gradient arrives as the two dense tensors of the forward
+        const long row = (long)b * p.L + lc;
+        if (c < p.split) { if (p.dy[s]) dyv = dw_ld<BF>(p.dy[s], row * p.split + c); }
+        else if (p.dy_tail[s]) dyv = dw_ld<BF>(p.dy_tail[s], row * (p.C - p.split) + (c - p.split));
+      } else if (p.dy[s]) {
+        dyv = dw_ld<BF>(p.dy[s], o);
+      }
       const float pv = dw_ld<BF>(p.pre, (long)s * p.B * p.L * p.C + o);
       dyb[s][j] = in ? dyv : 0.0f;
       prb[s][j] = in ? pv : 0.0f;

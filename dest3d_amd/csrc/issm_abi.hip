@@ -480,6 +480,10 @@ static int dwconv_params(const issm_dwconv_args* a, DwConvP* p, bool bwd) {
   if (bwd && (!a->partial || !a->dw || !a->dbias)) return fail(ISSM_E_NULL, "dwconv bwd: partial/dw/dbias is NULL");
   p->B = a->batch; p->L = a->seqlen; p->C = a->channels; p->nsets = a->nsets; p->dtype = a->dtype;
   p->u = a->u; p->u_bs = a->u_batch_stride; p->u_ls = a->u_token_stride;
+  if (a->split < 0 || a->split >= a->channels) return fail(ISSM_E_SHAPE, "dwconv: split %d outside [0, channels)", a->split);
+  if (a->split > 0 && !bwd && !a->y_tail) return fail(ISSM_E_NULL, "dwconv: y_tail is NULL");
+  p->split = a->split; p->y_tail = a->y_tail;
+  p->dy_tail[0] = a->dy_tail[0]; p->dy_tail[1] = a->nsets > 1 ? a->dy_tail[1] : nullptr;
   p->w = a->w; p->bias = a->bias; p->y = a->y; p->pre = a->pre;
   p->dy[0] = a->dy[0]; p->dy[1] = a->nsets > 1 ? a->dy[1] : nullptr;
   p->du = a->du; p->partial = a->partial; p->nrows = dwconv_partial_rows(a->batch, a->seqlen);

@@ -115,9 +115,12 @@ struct DwConvP {
   long u_bs, u_ls;
   const float* w;      // (nsets, C, 7) fp32
   const float* bias;   // (nsets, C) fp32
-  void* y;             // (nsets, B, L, C) io dtype
+  void* y;             // (nsets, B, L, C) io dtype; with split > 0: (nsets, B, L, split), channels [0, split)
+  void* y_tail;        // split > 0: (nsets, B, L, C - split), channels [split, C)
+  int split;
   void* pre;           // (nsets, B, L, C) io dtype: convolution output before SiLU (saved for the backward)
-  const void* dy[2];   // (B, L, C) io dtype per set, or NULL
+  const void* dy[2];   // (B, L, C) io dtype per set, or NULL; with split > 0: (B, L, split)
+  const void* dy_tail[2];  // split > 0: (B, L, C - split) per set, or NULL
   void* du;            // (B, L, C) io dtype
   float* partial;      // (nrows, nsets, 8, C) fp32
   int nrows;

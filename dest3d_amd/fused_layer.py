@@ -45,15 +45,16 @@ class FusedScanCoreFn(torch.autograd.Function):
             # 1. both depthwise convolutions + SiLU
             cw = torch.stack([conv_w_f.detach().reshape(Cc, _dw.TAPS), conv_w_b.detach().reshape(Cc, _dw.TAPS)]).float()
             cb = torch.stack([conv_b_f.detach(), conv_b_b.detach()]).float()
-            y = torch.empty((2, Bsz, Ln, Cc), dtype=kdt, device=dev)
-            pre = torch.empty_like(y)
+            x = torch.empty((2, Bsz, Ln, H, P), dtype=kdt, device=dev)       # the conv writes x and the B / C biases apart
+            tail = torch.empty((2, Bsz, Ln, 2 * G), dtype=kdt, device=dev)
+            pre = torch.empty((2, Bsz, Ln, Cc), dtype=kdt, device=dev)
             a = _dw._args(xbc, 2)
-            a.w, a.bias, a.y, a.pre = cw.data_ptr(), cb.data_ptr(), y.data_ptr(), pre.data_ptr()
+            a.w, a.bias, a.y, a.pre = cw.data_ptr(), cb.data_ptr(), x.data_ptr(), pre.data_ptr()
+            a.split, a.y_tail = di, tail.data_ptr()
             L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "issm_dwconv_silu_fwd")
-            x_f = y[0, ..., :di].contiguous().view(Bsz, Ln, H, P)
-            x_b = y[1, ..., :di].contiguous().view(Bsz, Ln, H, P)
+            x_f, x_b = x[0], x[1]
             # 2. dt / B / C (and the reversed-order B / C) from the distance encoding
-            bias = torch.cat([dt_tok.float() + dt_bias.detach().float(), y[0, ..., di:].float(), y[1, ..., di:].float()], -1)
+            bias = torch.cat([dt_tok.float() + dt_bias.detach().float(), tail[0].float(), tail[1].float()], -1)
             W = torch.cat([dt_w.detach(), bc_w.detach()], 0).float()
             d = dist.detach().to(kdt).contiguous()
             wt = None if weights is None else weights.detach().float().contiguous()
@@ -135,8 +136,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_param_gen_bwd(C.byref(g)), "issm_param_gen_bwd")
             d_dt_tok = dbias[..., :H]
             # 1'. the convolutions: gradients of (x, b-bias, c-bias) per branch
-            dyc = [torch.cat([dxs[0].view(Bsz, Ln, di), dbias[..., H:H + 2 * G].to(kdt)], -1),
-                   torch.cat([dxs[1].view(Bsz, Ln, di), dbias[..., H + 2 * G:].to(kdt)], -1)]
+            dtail = [dbias[..., H:H + 2 * G].to(kdt).contiguous(), dbias[..., H + 2 * G:].to(kdt).contiguous()]
             dxbc = torch.empty((Bsz, Ln, Cc), dtype=kdt, device=dev)
             rows = lib.issm_dwconv_partial_rows(Bsz, Ln)
             part = torch.empty((max(rows, 1), 2, 8, Cc), dtype=torch.float32, device=dev)
@@ -144,7 +144,9 @@ class FusedScanCoreFn(torch.autograd.Function):
             dcb = torch.empty((2, Cc), dtype=torch.float32, device=dev)
             a = _dw._args(xbc, 2)
             a.w, a.pre = cw.data_ptr(), pre.data_ptr()
-            a.dy[0], a.dy[1] = dyc[0].data_ptr(), dyc[1].data_ptr()
+            a.split = di
+            a.dy[0], a.dy[1] = dxs[0].data_ptr(), dxs[1].data_ptr()
+            a.dy_tail[0], a.dy_tail[1] = dtail[0].data_ptr(), dtail[1].data_ptr()
             a.du, a.partial, a.dw, a.dbias = dxbc.data_ptr(), part.data_ptr(), dcw.data_ptr(), dcb.data_ptr()
             L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "issm_dwconv_silu_bwd")
             dzx = torch.cat([dz.view(Bsz, Ln, di), dxbc, d_dt_tok.to(kdt)], -1)

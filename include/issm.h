@@ -281,7 +281,10 @@ int issm_param_gen_bwd(const issm_pgen_args* args);
  *   pre[s][b][l][c] = bias[s][c] + sum_j w[s][c][j] u[b][l+j-3][c]   (zero outside [0, L)),  y = silu(pre).
  * u: `dtype`, channels contiguous, element strides u_batch_stride / u_token_stride.  w (nsets, C, 7) and
  * bias (nsets, C): fp32 contiguous.  y and pre: (nsets, B, L, C) contiguous in `dtype`; pre is the
- * convolution output before SiLU, which the backward reads.  Backward: dy[s] (B, L, C) contiguous or NULL
+ * convolution output before SiLU, which the backward reads.  With 0 < split < C the output is written as two dense
+ * tensors instead, y (nsets, B, L, split) for channels [0, split) and y_tail (nsets, B, L, C - split) for the rest
+ * (MultiHeadISSMScan splits the result into x and the B / C biases, dest_module.py:532), and the backward takes
+ * dy[s] (B, L, split) and dy_tail[s] (B, L, C - split).  Backward: dy[s] (B, L, C) contiguous or NULL
  * (zero); du (B, L, C) contiguous; dw (nsets, C, 7), dbias (nsets, C) fp32; partial:
  * issm_dwconv_partial_rows(B, L) * nsets * 8 * C floats of scratch. */
 typedef struct issm_dwconv_args {
@@ -300,6 +303,10 @@ typedef struct issm_dwconv_args {
   float* dw;
   float* dbias;
   void* stream;
+  /* optional split of the output channels (0 = none) */
+  int32_t split;
+  void* y_tail;
+  const void* dy_tail[2];
 } issm_dwconv_args;
 
 int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);

@@ -86,3 +86,47 @@ def test_dwconv_rejects_unbuilt_shapes():
     assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -5
     a.nsets = 1
     assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -1
+
+
+def test_dwconv_split_outputs_equal_the_slices():
+    """With `split` the forward writes channels [0, split) and [split, C) as two dense tensors and the backward
+    takes the gradient in the same two pieces: identical to slicing / concatenating around the unsplit call."""
+    import ctypes as C
+    from dest3d_amd import _lib as L
+    from dest3d_amd import dwconv as D
+    lib = L.load()
+    g = torch.Generator().manual_seed(3)
+    B, Ln, Cn, split = 2, 45, 38, 32
+    u = torch.randn(B, Ln, Cn, generator=g).cuda()
+    w = torch.randn(2, Cn, 7, generator=g).cuda()
+    b = torch.randn(2, Cn, generator=g).cuda()
+    dy = torch.randn(2, B, Ln, Cn, generator=g).cuda()
+
+    def run(split_at):
+        y = torch.empty(2, B, Ln, Cn if not split_at else split_at, device="cuda")
+        tail = torch.empty(2, B, Ln, Cn - split_at, device="cuda") if split_at else None
+        pre = torch.empty(2, B, Ln, Cn, device="cuda")
+        a = D._args(u, 2)
+        a.w, a.bias, a.y, a.pre = w.data_ptr(), b.data_ptr(), y.data_ptr(), pre.data_ptr()
+        keep = []
+        if split_at:
+            a.split, a.y_tail = split_at, tail.data_ptr()
+        L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "fwd")
+        du = torch.empty(B, Ln, Cn, device="cuda")
+        part = torch.empty(lib.issm_dwconv_partial_rows(B, Ln), 2, 8, Cn, device="cuda")
+        dw, db = torch.empty(2, Cn, 7, device="cuda"), torch.empty(2, Cn, device="cuda")
+        a.du, a.partial, a.dw, a.dbias = du.data_ptr(), part.data_ptr(), dw.data_ptr(), db.data_ptr()
+        for s in range(2):
+            if split_at:
+                keep += [dy[s, ..., :split_at].contiguous(), dy[s, ..., split_at:].contiguous()]
+                a.dy[s], a.dy_tail[s] = keep[-2].data_ptr(), keep[-1].data_ptr()
+            else:
+                a.dy[s] = dy[s].data_ptr()
+        L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "bwd")
+        torch.cuda.synchronize()
+        return y, tail, du, dw, db
+
+    y0, _, du0, dw0, db0 = run(0)
+    y1, t1, du1, dw1, db1 = run(split)
+    assert torch.equal(y1, y0[..., :split]) and torch.equal(t1, y0[..., split:])
+    assert torch.equal(du1, du0) and torch.equal(dw1, dw0) and torch.equal(db1, db0)
