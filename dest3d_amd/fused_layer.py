@@ -43,8 +43,16 @@ class FusedScanCoreFn(torch.autograd.Function):
         with torch.cuda.device(dev):
             st = L.current_stream_ptr(dev)
             # 1. both depthwise convolutions + SiLU
-            cw = torch.stack([conv_w_f.detach().reshape(Cc, _dw.TAPS), conv_w_b.detach().reshape(Cc, _dw.TAPS)]).float()
-            cb = torch.stack([conv_b_f.detach(), conv_b_b.detach()]).float()
+            # all small parameters in one fp32 buffer (one concatenation + one conversion instead of one per tensor);
+            # adjacent pieces form the stacked operands the kernels take
+            params = (conv_w_f, conv_w_b, conv_b_f, conv_b_b, dt_w, bc_w, dt_bias, A_log)
+            sizes = [t.numel() for t in params]
+            flat = torch.cat([t.detach().reshape(-1) for t in params]).float()
+            pieces = torch.split(flat, sizes)
+            cw = flat[:2 * Cc * _dw.TAPS].view(2, Cc, _dw.TAPS)
+            cb = flat[2 * Cc * _dw.TAPS:2 * Cc * _dw.TAPS + 2 * Cc].view(2, Cc)
+            W = flat[sum(sizes[:4]):sum(sizes[:6])].view(H + 2 * G, 16)      # rows: dt heads, B groups, C groups
+            dt_bias32, A_log32 = pieces[6], pieces[7]
             x = torch.empty((2, Bsz, Ln, H, P), dtype=kdt, device=dev)       # the conv writes x and the B / C biases apart
             tail = torch.empty((2, Bsz, Ln, 2 * G), dtype=kdt, device=dev)
             pre = torch.empty((2, Bsz, Ln, Cc), dtype=kdt, device=dev)
@@ -54,8 +62,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "issm_dwconv_silu_fwd")
             x_f, x_b = x[0], x[1]
             # 2. dt / B / C (and the reversed-order B / C) from the distance encoding
-            bias = torch.cat([dt_tok.float() + dt_bias.detach().float(), tail[0].float(), tail[1].float()], -1)
-            W = torch.cat([dt_w.detach(), bc_w.detach()], 0).float()
+            bias = torch.cat([dt_tok.float() + dt_bias32, tail[0].float(), tail[1].float()], -1)
             d = dist.detach().to(kdt).contiguous()
             wt = None if weights is None else weights.detach().float().contiguous()
             dt = torch.empty((Bsz, Ln, H, K), dtype=kdt, device=dev)
@@ -68,7 +75,7 @@ class FusedScanCoreFn(torch.autograd.Function):
                 g.weights, g.dt_raw = wt.data_ptr(), raw.data_ptr()
             L.check(lib.issm_param_gen_fwd(C.byref(g)), "issm_param_gen_fwd")
             # 3. the bidirectional scan, queries as initial state
-            A = (-torch.exp(A_log.detach().float()))[:, None].expand(H, K)
+            A = torch.exp(A_log32).neg_()[:, None].expand(H, K)
             h0 = h0_lin.detach().reshape(Bsz, K, H, P).permute(0, 2, 3, 1)
             prob = _Problem([x_f, x_b], dt, A, [bc[0], bc[2]], [bc[1], bc[3]], chunk_size, D.detach(), [None, None], None,
                             h0, None, wt is None, dt_limit)
@@ -85,7 +92,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             n.y, n.y_row_stride, n.rstd = key_n.data_ptr(), key_n.stride(0), rstd.data_ptr()
             L.check(lib.issm_gated_rmsnorm_fwd(C.byref(n)), "issm_gated_rmsnorm_fwd")
             last = torch.add(finals[0], finals[1]).mul_(0.5).permute(0, 3, 1, 2).reshape(Bsz, K, di)
-        ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log.detach())
+        ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log32)
         ctx.prob, ctx.ws = prob, ws
         ctx.meta = (Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, st)
         ctx.dtypes = tuple(t.dtype for t in (zxbcdt, h0_lin, dist, conv_w_f, conv_b_f, conv_w_b, conv_b_b, dt_w, bc_w,
@@ -150,13 +157,22 @@ class FusedScanCoreFn(torch.autograd.Function):
             a.du, a.partial, a.dw, a.dbias = dxbc.data_ptr(), part.data_ptr(), dcw.data_ptr(), dcb.data_ptr()
             L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "issm_dwconv_silu_bwd")
             dzx = torch.cat([dz.view(Bsz, Ln, di), dxbc, d_dt_tok.to(kdt)], -1)
-            dA_log = dA.sum(-1).mul_(-torch.exp(A_log.float()))
+            dA_log = dA.sum(-1).mul_(torch.exp(A_log).neg_())
             dh0_lin = dh0.permute(0, 3, 1, 2).reshape(Bsz, K, di)
             ddt_bias = d_dt_tok.sum((0, 1))
+            # parameter gradients: one buffer, one conversion to the parameters' dtype when they share one
+            grads = [dcw[0], dcb[0], dcw[1], dcb[1], dW[:H], dW[H:], ddt_bias, dA_log, dD, dnw]
+            pdts = (wfdt, bfdt, wbdt, bbdt, dtwdt, bcwdt, dtbdt, aldt, Ddt, nwdt)
+            if len(set(pdts)) == 1 and pdts[0] != torch.float32:
+                sizes = [t.numel() for t in grads]
+                grads = list(torch.split(torch.cat([t.reshape(-1) for t in grads]).to(pdts[0]), sizes))
+            else:
+                grads = [t.to(dt_) for t, dt_ in zip(grads, pdts)]
         wf_shape, wb_shape = ctx.shapes
-        return (dzx.to(zdt), dh0_lin.to(hdt), None if ddist is None else ddist.to(ddt_), None,
-                dcw[0].reshape(wf_shape).to(wfdt), dcb[0].to(bfdt), dcw[1].reshape(wb_shape).to(wbdt), dcb[1].to(bbdt),
-                dW[:H].to(dtwdt), dW[H:].to(bcwdt), ddt_bias.to(dtbdt), dA_log.to(aldt), dD.to(Ddt), dnw.to(nwdt),
+        grads[0], grads[2] = grads[0].reshape(wf_shape), grads[2].reshape(wb_shape)
+        grads[4], grads[5] = grads[4].reshape(H, 16), grads[5].reshape(2 * G, 16)
+        grads[8] = grads[8].reshape(prob.D.shape)
+        return (dzx.to(zdt), dh0_lin.to(hdt), None if ddist is None else ddist.to(ddt_), None, *grads,
                 None, None, None, None, None, None)
 
 
