@@ -350,11 +350,12 @@ def time_pointnet2_ops(torch, reps=5):
     return res
 
 
-def time_module_layer(torch, steps=10, warmup=3, dtype=None):
+def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
     models/dest_module.py:283-290), forward + backward through autograd, microseconds.  Includes the PyTorch
-    projections and norms around the scan."""
+    projections and norms around the scan.  With `as_graph` the step is recorded once into a HIP graph (the pattern
+    of torch.cuda.graphs for a whole training step) and the replays are timed: the GPU's time without the host's."""
     from dest3d_amd.scan_module import MultiHeadISSMScan
     torch.manual_seed(0)
     dtype = dtype or torch.bfloat16
@@ -370,6 +371,21 @@ def time_module_layer(torch, steps=10, warmup=3, dtype=None):
         ok, oq = m(key, query, dist, None, weights)
         (ok.float().square().mean() + oq.float().square().mean()).backward()
 
+    if as_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        m.zero_grad(set_to_none=True)
+        key.grad = query.grad = dist.grad = None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            ok, oq = m(key, query, dist, None, weights)
+            (ok.float().square().mean() + oq.float().square().mean()).backward()
+        step = graph.replay
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -415,6 +431,8 @@ def main():
     if args.only_layer:
         whole, enc = time_box_dist_layer(torch, args.steps, args.warmup)
         print(json.dumps({"detector_layer_bf16_fwd_bwd_us": round(time_module_layer(torch, args.steps, args.warmup), 2),
+                          "detector_layer_bf16_fwd_bwd_as_hip_graph_us":
+                              round(time_module_layer(torch, args.steps, args.warmup, as_graph=True), 2),
                           "box_dist_plus_layer_bf16_fwd_bwd_us": round(whole, 2),
                           "box_dist_and_weight_fwd_us": round(enc, 2), "steps": args.steps, "warmup": args.warmup}))
         return
@@ -457,6 +475,7 @@ def main():
             del r
         SHAPE["P"] = 32
         variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
+        variants["detector_layer_bf16_fwd_bwd_as_hip_graph"] = round(time_module_layer(torch, as_graph=True), 2)
         variants["detector_layer_fp32_fwd_bwd"] = round(time_module_layer(torch, dtype=torch.float32), 2)
         variants["box_dist_plus_layer_bf16_fwd_bwd"] = round(time_box_dist_layer(torch)[0], 2)
     line = {

@@ -18,6 +18,8 @@
 
 namespace issm {
 
+typedef int i4 __attribute__((ext_vector_type(4)));
+
 constexpr int BDS_SEG = 2048;      // entries per work item
 constexpr int BDS_MAXBINS = 9280;  // (D + 2)(H + 2)(W + 2) for D*H*W <= 1024 is at most 1026 * 3 * 3
 constexpr int BDS_NWG = 512;       // workgroups of the count and fill passes (they must walk identically)
@@ -31,16 +33,19 @@ struct SortP {
   int* items;                   // [maxitems][3] bin, first entry, one past the last entry
   unsigned long long* records;  // [maxrecords] pair index | corner mask << 32
   long long* item_out;          // [maxitems][BDS_OUT]
-  long long* dtab;              // [cells][16]
+  float* boxtab;                // [B * K][40] corners x, y, z and rotations cos, sin of every box, 8 values each
+  long long* dtab;              // [2][cells][16]: sums of the low 32 bits of the items' results, sums of the rest
   int nbins, maxitems;
   long maxrecords;
 };
 
-// Fixed-point scale: a term weight * ddist is at most 8 max|ddist|, so with 2^27 / max|ddist| it converts to a 32-bit
-// integer (one instruction); the sums are kept in 64 bits (2^26 pairs * 8 * 2^27 < 2^63).
+// Fixed point: weights in units of 2^-24, ddist in units of max|ddist| * 2^-22.  A term is at most 8 * 2^24 * 2^22 =
+// 2^49 and a work item's sum at most 2^60; the table takes the items' sums as two 64-bit halves (low 32 bits and
+// the rest), each far from overflow for the 2^26 pairs the launcher admits.
+constexpr float BDS_W_SCALE = 16777216.0f;
 __device__ __forceinline__ float bds_scale(const unsigned* scal) {
   const float gmax = __uint_as_float(scal[0]);
-  return gmax > 0.0f ? 134217728.0f / gmax : 1.0f;
+  return gmax > 0.0f ? 4194304.0f / gmax : 1.0f;
 }
 
 __device__ __forceinline__ int bds_bin(const BoxDistP& p, int mx, int my, int mz) {
@@ -53,7 +58,21 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_clear(BoxDistP p, SortP s) {
   const int i = blockIdx.x * NTHREADS + threadIdx.x;
   if (i < 4) s.scal[i] = 0u;
   if (i < s.nbins) s.counts[i] = 0;
-  if (i < cells * BD_C) s.dtab[i] = 0;
+  if (i < cells * BD_C) s.dtab[i] = s.dtab[cells * BD_C + i] = 0;
+}
+
+// Corners and rotations of every box, once: the accumulation pass visits a box from many lanes, and evaluating the
+// sines and cosines there again for every entry cost more than everything else in it.
+__global__ __launch_bounds__(NTHREADS) void k_bds_boxes(BoxDistP p, SortP s) {
+  const int i = blockIdx.x * NTHREADS + threadIdx.x;
+  if (i >= p.B * p.K) return;
+  BoxLane bx;
+  load_box(p, i / p.K, i % p.K, bx);
+  float* o = s.boxtab + (long)i * 40;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    o[c] = bx.cx[c]; o[8 + c] = bx.cy[c]; o[16 + c] = bx.cz[c]; o[24 + c] = bx.cs[c]; o[32 + c] = bx.sn[c];
+  }
 }
 
 // The walk shared by count and fill: thread = (b, l, k) as in the forward, f(bin, pair index, corner mask).
@@ -188,20 +207,55 @@ __device__ __forceinline__ void axis3(int i, float f, int m, float (&a)[3]) {
   for (int j = 0; j < 3; ++j) a[j] = (s0 == j ? 1.0f - f : 0.0f) + (s0 + 1 == j ? f : 0.0f);
 }
 
+// 4 x 4 transpose of bytes: in q[0..3] byte d of q[r] is digit d of entry r; out t[d] holds digit d of the four
+// entries.
+__device__ __forceinline__ void digits4(const unsigned (&q)[4], unsigned (&t)[4]) {
+  const unsigned x0 = __builtin_amdgcn_perm(q[1], q[0], 0x05010400u), x1 = __builtin_amdgcn_perm(q[1], q[0], 0x07030602u);
+  const unsigned y0 = __builtin_amdgcn_perm(q[3], q[2], 0x05010400u), y1 = __builtin_amdgcn_perm(q[3], q[2], 0x07030602u);
+  t[0] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+  t[1] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+  t[2] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+  t[3] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+}
+// 16 entries' fixed-point values (one dword each, four signed digits) -> per digit the 16 bytes of a matrix operand
+__device__ __forceinline__ void digit_operands(const unsigned* row, i4 (&op)[4]) {
+  unsigned t[4][4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const uint4 v = *(const uint4*)(row + 4 * m);
+    const unsigned q[4] = {v.x, v.y, v.z, v.w};
+    digits4(q, t[m]);
+  }
+#pragma unroll
+  for (int d = 0; d < 4; ++d) op[d] = (i4){(int)t[0][d], (int)t[1][d], (int)t[2][d], (int)t[3][d]};
+}
+// A 32-bit integer as four signed base-256 digits, one per byte: v = sum d_i 256^i with d_i in [-128, 127].
+__device__ __forceinline__ unsigned signed_digits(int v) { return ((unsigned)v + 0x80808080u) ^ 0x80808080u; }
+
+// One work item: out[node][ch] = sum over the item's entries of weight[entry][node] * ddist[entry][ch], exactly, in
+// integers, on the matrix cores.  Weights are taken to 2^-24 and ddist to 2^-22 of its largest magnitude; both are
+// written as signed base-256 digits, and the product of two values is the sum of the products of their digits,
+// 256^(i+j) apart: twelve int8 products (v_mfma_i32_16x16x64_i8: 16 nodes x 16 channels x 64 entries) that add into
+// six 32-bit accumulators, one per power of 256.  Integer sums do not depend on the order of the entries, which the
+// fill pass does not fix, so the result is reproducible bit for bit.  Wave w of a batch of 256 entries owns entries
+// 64 w .. 64 w + 63: it stages their values as Wq[node][entry], Gq[channel][entry] and reads back 16 entries per lane.
+constexpr int BDS_ROW = 64 + 4;  // dwords per staged row: lanes of one 16-lane group start 4 banks apart
 template <bool BF>
 __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
-  __shared__ float Wl[NTHREADS][27];  // odd row length: the lanes' rows start in different banks
-  __shared__ __attribute__((aligned(16))) float Gl[NTHREADS][BD_C];
+  __shared__ __attribute__((aligned(16))) unsigned Wq[4][27][BDS_ROW];
+  __shared__ __attribute__((aligned(16))) unsigned Gq[4][BD_C][BDS_ROW];
   const int item = blockIdx.x;
   if (item >= (int)s.scal[1]) return;  // uniform
   const int bin = s.items[3 * item], first = s.items[3 * item + 1], last = s.items[3 * item + 2];
   const int mx = bin % (p.W + 2) - 2, my = (bin / (p.W + 2)) % (p.H + 2) - 2, mz = bin / ((p.W + 2) * (p.H + 2)) - 2;
   const float scale = 1.0f / (3.0f * p.max_value);
-  const float fx_scale = bds_scale(s.scal);
-  const int t0 = threadIdx.x, t1 = threadIdx.x + NTHREADS;  // the thread's (node, channel) results
-  const int slot0 = t0 >> 4, slot1 = t1 >> 4, ch = t0 & 15;
-  const bool has1 = t1 < BDS_OUT;
-  long long acc0 = 0, acc1 = 0;
+  const float g_scale = bds_scale(s.scal);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, kg = lane >> 4;
+  i4 acc[2][6];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int c = 0; c < 6; ++c) acc[t][c] = (i4){0, 0, 0, 0};
   for (int base = first; base < last; base += NTHREADS) {
     const int e = base + threadIdx.x;
     float w[27];
@@ -219,13 +273,15 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
       const int l = (int)(bl % (unsigned)p.L), b = (int)(bl / (unsigned)p.L);
       const float* key = p.key + ((long)b * p.L + l) * 3;
       const float kx = key[0], ky = key[1], kz = key[2];
+      f4 bt[10];  // the box: x[8], y[8], z[8], cos[8], sin[8]
+#pragma unroll
+      for (int j = 0; j < 10; ++j) bt[j] = *(const f4*)(s.boxtab + ((long)b * p.K + k) * 40 + 4 * j);
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (mask & (1u << c)) {
-          float cx, cy, cz, cs, sn, x, y, z;
-          box_corner(p, b, k, c, cx, cy, cz);
-          corner_rotation(p, b, k, c, cs, sn);
-          corner_pos(p, cx, cy, cz, cs, sn, kx, ky, kz, scale, x, y, z);
+          float x, y, z;
+          corner_pos(p, bt[c >> 2][c & 3], bt[2 + (c >> 2)][c & 3], bt[4 + (c >> 2)][c & 3], bt[6 + (c >> 2)][c & 3],
+                     bt[8 + (c >> 2)][c & 3], kx, ky, kz, scale, x, y, z);
           const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
           float ax[3], ay[3], az[3];
           axis3((int)gx, x - gx, mx, ax);
@@ -258,22 +314,59 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
         for (int j = 0; j < 4; ++j) g[j] = src[j];
       }
     }
+    // a weight is at most 8 (eight corners on one node): 2^27 as an integer; |ddist * g_scale| <= 2^22 (three digits)
 #pragma unroll
-    for (int j = 0; j < 27; ++j) Wl[threadIdx.x][j] = w[j];
+    for (int j = 0; j < 27; ++j) Wq[wave][j][lane] = signed_digits(__float2int_rn(w[j] * BDS_W_SCALE));
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *(f4*)&Gl[threadIdx.x][4 * j] = g[j] * fx_scale;
+    for (int j = 0; j < 4; ++j) {
+      Gq[wave][4 * j + 0][lane] = signed_digits(__float2int_rn(g[j].x * g_scale));
+      Gq[wave][4 * j + 1][lane] = signed_digits(__float2int_rn(g[j].y * g_scale));
+      Gq[wave][4 * j + 2][lane] = signed_digits(__float2int_rn(g[j].z * g_scale));
+      Gq[wave][4 * j + 3][lane] = signed_digits(__float2int_rn(g[j].w * g_scale));
+    }
     __syncthreads();
-    const int nb = min(NTHREADS, last - base);  // rows nb .. 255 hold zeros: the loop may run past nb in steps of 4
-#pragma unroll 4
-    for (int ee = 0; ee < ((nb + 3) & ~3); ++ee) {
-      const float gv = Gl[ee][ch];
-      acc0 += (long long)__float2int_rn(Wl[ee][slot0] * gv);  // |weight * ddist * scale| <= 8 * 2^27: fits 32 bits
-      if (has1) acc1 += (long long)__float2int_rn(Wl[ee][slot1] * gv);
+    if (base + wave * 64 < last) {  // uniform per wave: the wave's 64 entries hold something
+      i4 bop[4];
+      digit_operands(&Gq[wave][r][16 * kg], bop);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int node = 16 * t + r;
+        i4 aop[4];
+        digit_operands(&Wq[wave][node < 27 ? node : 0][16 * kg], aop);
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          if (node >= 27) aop[d] = (i4){0, 0, 0, 0};
+#pragma unroll
+        for (int dw = 0; dw < 4; ++dw)
+#pragma unroll
+          for (int dg = 0; dg < 3; ++dg)
+            acc[t][dw + dg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[dw], bop[dg], acc[t][dw + dg], 0, 0, 0);
+      }
     }
     __syncthreads();
   }
-  s.item_out[(long)item * BDS_OUT + t0] = acc0;
-  if (has1) s.item_out[(long)item * BDS_OUT + t1] = acc1;
+  // 256^c apart, in 64 bits; then the four waves' sums.  The lane holds nodes 16 t + 4 kg + i, channel r.
+  long long* red = (long long*)&Wq[0][0][0];  // [wave][t * 4 + i][lane]: 16 KB of the staging area
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      long long v = 0;
+#pragma unroll
+      for (int c = 5; c >= 0; --c) v = v * 256 + (long long)acc[t][c][i];
+      red[(wave * 8 + t * 4 + i) * 64 + lane] = v;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int ti = h * 4 + wave, node = 16 * (ti >> 2) + 4 * kg + (ti & 3);
+    if (node < 27) {
+      long long v = 0;
+#pragma unroll
+      for (int w2 = 0; w2 < 4; ++w2) v += red[(w2 * 8 + ti) * 64 + lane];
+      s.item_out[(long)item * BDS_OUT + node * BD_C + r] = v;
+    }
+  }
 }
 
 __global__ __launch_bounds__(NTHREADS) void k_bds_scatter(BoxDistP p, SortP s) {
@@ -286,14 +379,18 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_scatter(BoxDistP p, SortP s) {
             jz = bin / ((p.W + 2) * (p.H + 2)) - 2 + slot / 9;
   if (jx < 0 || jx >= p.W || jy < 0 || jy >= p.H || jz < 0 || jz >= p.D) return;
   const long long v = s.item_out[id];
-  if (v != 0) atomicAdd((unsigned long long*)&s.dtab[((long)(jz * p.H + jy) * p.W + jx) * BD_C + ch], (unsigned long long)v);
+  if (v == 0) return;
+  const long e = ((long)(jz * p.H + jy) * p.W + jx) * BD_C + ch;
+  atomicAdd((unsigned long long*)&s.dtab[e], (unsigned long long)v & 0xffffffffull);                      // low half, >= 0
+  atomicAdd((unsigned long long*)&s.dtab[(long)p.D * p.H * p.W * BD_C + e], (unsigned long long)(v >> 32));  // the rest, signed
 }
 
 __global__ __launch_bounds__(NTHREADS) void k_bds_finish(BoxDistP p, SortP s) {
   const int cells = p.D * p.H * p.W;
   const int e = blockIdx.x * NTHREADS + threadIdx.x;  // e = cell * 16 + ch
   if (e >= cells * BD_C) return;
-  p.dtable[(long)(e % BD_C) * cells + e / BD_C] = (float)((double)s.dtab[e] / (double)bds_scale(s.scal));
+  const double v = (double)s.dtab[cells * BD_C + e] * 4294967296.0 + (double)s.dtab[e];
+  p.dtable[(long)(e % BD_C) * cells + e / BD_C] = (float)(v / ((double)BDS_W_SCALE * (double)bds_scale(s.scal)));
 }
 
 template <bool BF>
@@ -321,7 +418,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_gmax(BoxDistP p, unsigned* sca
 static long bds_align(long v) { return (v + 15) & ~15L; }
 
 struct BdsLayout {
-  long scal, counts, binoff, wgbase, items, records, item_out, dtab, total;
+  long scal, counts, binoff, wgbase, items, records, item_out, dtab, boxtab, total;
   int nbins, maxitems;
   long maxrecords;
 };
@@ -338,7 +435,8 @@ static BdsLayout bds_layout(int B, int L, int K, int D, int H, int W) {
   y.items = o; o = bds_align(o + (long)y.maxitems * 12);
   y.records = o; o = bds_align(o + maxrec * 8);
   y.item_out = o; o = bds_align(o + (long)y.maxitems * BDS_OUT * 8);
-  y.dtab = o; o = bds_align(o + (long)D * H * W * BD_C * 8);
+  y.dtab = o; o = bds_align(o + (long)D * H * W * BD_C * 16);  // two halves
+  y.boxtab = o; o = bds_align(o + (long)B * K * 40 * 4);
   y.total = o;
   return y;
 }
@@ -358,6 +456,7 @@ int launch_box_dist_bwd_sorted(const BoxDistP& p, hipStream_t st) {
   s.records = (unsigned long long*)(base + y.records);
   s.item_out = (long long*)(base + y.item_out);
   s.dtab = (long long*)(base + y.dtab);
+  s.boxtab = (float*)(base + y.boxtab);
   s.nbins = y.nbins;
   s.maxitems = y.maxitems;
   s.maxrecords = (long)p.B * p.L * p.K * 8;
@@ -367,6 +466,7 @@ int launch_box_dist_bwd_sorted(const BoxDistP& p, hipStream_t st) {
   hipLaunchKernelGGL(k_bds_clear, dim3((nclear + NTHREADS - 1) / NTHREADS), b, 0, st, p, s);
   if (p.dtype) hipLaunchKernelGGL(k_bds_gmax<true>, dim3(512), b, 0, st, p, s.scal);
   else hipLaunchKernelGGL(k_bds_gmax<false>, dim3(512), b, 0, st, p, s.scal);
+  hipLaunchKernelGGL(k_bds_boxes, dim3((p.B * p.K + NTHREADS - 1) / NTHREADS), b, 0, st, p, s);
   hipLaunchKernelGGL(k_bds_count, dim3(BDS_NWG), b, 0, st, p, s);
   hipLaunchKernelGGL(k_bds_plan, dim3(1), b, 0, st, s);
   hipLaunchKernelGGL(k_bds_wgbase, dim3((y.nbins + 63) / 64), dim3(64), 0, st, s);
