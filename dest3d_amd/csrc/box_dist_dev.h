@@ -78,12 +78,12 @@ __device__ __forceinline__ float node_pos(float v, float log_scale, float scale,
   return (g + 1.0f) * (0.5f * n) - 0.5f;
 }
 
-// The 8 neighbours of one sampling position: LDS offset (in floats) of the node and its weight (0 outside).
+// The 8 neighbours of one sampling position: LDS offset of the node (node index * stride) and its weight (0 outside).
 struct Tri {
   int off[8];
   float w[8];
 };
-__device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, float z, Tri& t) {
+__device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, float z, Tri& t, int stride = BD_C) {
   const float fx = floorf(x), fy = floorf(y), fz = floorf(z);
   const float ax = x - fx, ay = y - fy, az = z - fz;
   const int ix = (int)fx, iy = (int)fy, iz = (int)fz;
@@ -94,7 +94,7 @@ __device__ __forceinline__ void trilinear(const BoxDistP& p, float x, float y, f
     const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
     const float w = (dx ? ax : 1.0f - ax) * (dy ? ay : 1.0f - ay) * (dz ? az : 1.0f - az);
     t.w[n] = ok ? w : 0.0f;
-    t.off[n] = ok ? ((jz * p.H + jy) * p.W + jx) * BD_C : 0;
+    t.off[n] = ok ? ((jz * p.H + jy) * p.W + jx) * stride : 0;
   }
 }
 
@@ -151,7 +151,7 @@ __device__ __forceinline__ bool corner_window(const BoxDistP& p, const BoxLane& 
 }
 // visit the window's nodes that lie inside the table and carry weight: f(LDS offset in floats, weight)
 template <class F>
-__device__ __forceinline__ void for_window(const BoxDistP& p, const Window& win, F f) {
+__device__ __forceinline__ void for_window(const BoxDistP& p, const Window& win, F f, int stride = BD_C) {
 #pragma unroll
   for (int k = 0; k < 3; ++k)
 #pragma unroll
@@ -161,7 +161,7 @@ __device__ __forceinline__ void for_window(const BoxDistP& p, const Window& win,
         const int jx = win.mx + j, jy = win.my + i, jz = win.mz + k;
         const bool ok = jx >= 0 && jx < p.W && jy >= 0 && jy < p.H && jz >= 0 && jz < p.D;
         const float w = win.w[k * 9 + i * 3 + j];
-        if (ok && w != 0.0f) f(((jz * p.H + jy) * p.W + jx) * BD_C, w);
+        if (ok && w != 0.0f) f(((jz * p.H + jy) * p.W + jx) * stride, w);
       }
 }
 
