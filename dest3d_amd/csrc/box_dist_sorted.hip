@@ -123,14 +123,19 @@ __device__ int bds_scan(const int* v, int* out, int n, int* part) {
   for (int e = e0; e < e1; ++e) sum += v[e];
   part[threadIdx.x] = sum;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int t = 0; t < NTHREADS; ++t) {
-      const int c = part[t];
-      part[t] = run;
-      run += c;
+  if (threadIdx.x < 64) {  // exclusive scan of the 256 partial sums by one wave: 4 per lane, then across the lanes
+    const int t0 = threadIdx.x * 4;
+    const int c0 = part[t0], c1 = part[t0 + 1], c2 = part[t0 + 2], c3 = part[t0 + 3];
+    const int mine = c0 + c1 + c2 + c3;
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int v = __shfl_up(incl, o, 64);
+      if ((int)threadIdx.x >= o) incl += v;
     }
-    part[NTHREADS] = run;
+    const int excl = incl - mine;
+    part[t0] = excl; part[t0 + 1] = excl + c0; part[t0 + 2] = excl + c0 + c1; part[t0 + 3] = excl + c0 + c1 + c2;
+    if (threadIdx.x == 63) part[NTHREADS] = incl;
   }
   __syncthreads();
   int run = part[threadIdx.x];
@@ -171,17 +176,17 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_plan(SortP s) {
 }
 
 // Base position of every counting workgroup inside every bin: a running sum over the workgroups, in order (thread
-// = bin; 16 loads in flight at a time).
+// = bin; 64 loads in flight at a time).
 __global__ __launch_bounds__(64) void k_bds_wgbase(SortP s) {
   const int e = blockIdx.x * 64 + threadIdx.x;
   if (e >= s.nbins) return;
   int run = s.binoff[e];
-  for (int w0 = 0; w0 < BDS_NWG; w0 += 16) {
-    int c[16];
+  for (int w0 = 0; w0 < BDS_NWG; w0 += 64) {
+    int c[64];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) c[j] = s.wgbase[(long)(w0 + j) * s.nbins + e];
+    for (int j = 0; j < 64; ++j) c[j] = s.wgbase[(long)(w0 + j) * s.nbins + e];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < 64; ++j) {
       s.wgbase[(long)(w0 + j) * s.nbins + e] = run;
       run += c[j];
     }
@@ -393,26 +398,45 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_finish(BoxDistP p, SortP s) {
   p.dtable[(long)(e % BD_C) * cells + e / BD_C] = (float)(v / ((double)BDS_W_SCALE * (double)bds_scale(s.scal)));
 }
 
+// max |ddist|, four wide loads in flight per lane (n is a multiple of 16)
 template <bool BF>
 __global__ __launch_bounds__(NTHREADS) void k_bds_gmax(BoxDistP p, unsigned* scal) {
   const long n = (long)p.B * p.L * p.K * BD_C;
-  float m = 0.0f;
-  for (long e = ((long)blockIdx.x * NTHREADS + threadIdx.x) * 8; e < n; e += (long)gridDim.x * NTHREADS * 8) {
-    if (BF) {
-      const uint4 v = *(const uint4*)((const uint16_t*)p.ddist + e);
-      const unsigned w[4] = {v.x, v.y, v.z, v.w};
+  const long per = BF ? 8 : 4, step = (long)gridDim.x * NTHREADS * per;  // elements per 16-byte load; per sweep
+  unsigned m = 0u;  // largest magnitude as a bit pattern: orders like the float for non-negative values
+  for (long e = ((long)blockIdx.x * NTHREADS + threadIdx.x) * per; e < n; e += 4 * step) {
+    uint4 v[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        m = fmaxf(m, fmaxf(fabsf(__uint_as_float(w[j] << 16)), fabsf(__uint_as_float(w[j] & 0xffff0000u))));
-    } else {
-      const f4 a = *(const f4*)((const float*)p.ddist + e), c = *(const f4*)((const float*)p.ddist + e + 4);
-      m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
-      m = fmaxf(m, fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+    for (int j = 0; j < 4; ++j) {
+      const long ej = e + j * step;
+      v[j] = *(const uint4*)((const char*)p.ddist + (ej < n ? ej : e) * (BF ? 2 : 4));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (BF) {
+          const unsigned lo = (w[i] << 16) & 0x7fffffffu, hi = w[i] & 0x7fff0000u;
+          m = max(m, (lo <= 0x7f800000u ? lo : 0u));  // NaN patterns are left out
+          m = max(m, (hi <= 0x7f800000u ? hi : 0u));
+        } else {
+          const unsigned a = w[i] & 0x7fffffffu;
+          m = max(m, (a <= 0x7f800000u ? a : 0u));
+        }
+      }
     }
   }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-  if ((threadIdx.x & 63) == 0 && m > 0.0f && m == m) atomicMax(scal, __float_as_uint(m));
+  for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o, 64));
+  __shared__ unsigned wm[NTHREADS / 64];
+  if ((threadIdx.x & 63) == 0) wm[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {  // one atomic per workgroup: thousands on one address would take longer than the sweep
+#pragma unroll
+    for (int w = 1; w < NTHREADS / 64; ++w) m = max(m, wm[w]);
+    if (m > 0u) atomicMax(scal, m);
+  }
 }
 
 static long bds_align(long v) { return (v + 15) & ~15L; }
