@@ -247,6 +247,7 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
     key_pos = 8.0 * torch.rand(8, 1024, 3, device="cuda")
     query_pos = torch.cat([8.0 * torch.rand(8, 256, 3, device="cuda"), 0.2 + 2.0 * torch.rand(8, 256, 3, device="cuda")], -1)
     zero_angle = torch.zeros(8, 256, device="cuda")
+    g_key, g_query = torch.randn_like(key) / 64, torch.randn_like(query) / 64   # what the next layer hands back
 
     def encode():
         return bd(key_pos, query_pos[..., :3], query_pos[..., 3:], zero_angle, weight_query_pos=query_pos)
@@ -257,7 +258,7 @@ def time_box_dist_layer(torch, steps=10, warmup=3):
         key.grad = query.grad = None
         dist, weights = encode()
         ok, oq = m(key, query, dist, key_pos, weights)
-        (ok.float().square().mean() + oq.float().square().mean()).backward()
+        torch.autograd.backward((ok, oq), (g_key, g_query))
 
     out = []
     for fn in (step, encode):
@@ -353,8 +354,9 @@ def time_pointnet2_ops(torch, reps=5):
 def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
-    models/dest_module.py:283-290), forward + backward through autograd, microseconds.  Includes the PyTorch
-    projections and norms around the scan.  With `as_graph` the step is recorded once into a HIP graph (the pattern
+    models/dest_module.py:283-290), forward + backward through autograd from given output gradients (as inside a
+    stack of layers: no loss is computed here), microseconds.  Includes the PyTorch projections and norms around the
+    scan.  With `as_graph` the step is recorded once into a HIP graph (the pattern
     of torch.cuda.graphs for a whole training step) and the replays are timed: the GPU's time without the host's."""
     from dest3d_amd.scan_module import MultiHeadISSMScan
     torch.manual_seed(0)
@@ -365,11 +367,13 @@ def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
     dist = (0.5 * torch.randn(8, 1024, 256, 16, device="cuda")).to(dtype).requires_grad_()
     weights = torch.exp(-15.0 * (torch.rand(8, 1024, 256, device="cuda") - 0.5).clamp_min(0.0))
 
+    g_key, g_query = torch.randn_like(key) / 64, torch.randn_like(query) / 64   # what the next layer hands back
+
     def step():
         m.zero_grad(set_to_none=True)   # as an optimizer step would: no accumulation into old gradients
         key.grad = query.grad = dist.grad = None
         ok, oq = m(key, query, dist, None, weights)
-        (ok.float().square().mean() + oq.float().square().mean()).backward()
+        torch.autograd.backward((ok, oq), (g_key, g_query))
 
     if as_graph:
         side = torch.cuda.Stream()
@@ -384,7 +388,7 @@ def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             ok, oq = m(key, query, dist, None, weights)
-            (ok.float().square().mean() + oq.float().square().mean()).backward()
+            torch.autograd.backward((ok, oq), (g_key, g_query))
         step = graph.replay
     for _ in range(warmup):
         step()

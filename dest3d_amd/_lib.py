@@ -107,6 +107,7 @@ class DwConvArgs(C.Structure):
         ("dy", C.c_void_p * 2), ("du", C.c_void_p), ("partial", C.c_void_p), ("dw", C.c_void_p),
         ("dbias", C.c_void_p), ("stream", C.c_void_p),
         ("split", C.c_int32), ("y_tail", C.c_void_p), ("dy_tail", C.c_void_p * 2),
+        ("du_batch_stride", C.c_int64), ("du_token_stride", C.c_int64),
     ]
 
 

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(NTHREADS) void k_dwconv_bwd(DwConvP p) {
 #pragma unroll
         for (int j = 0; j < DW_TAPS; ++j) gw[s][j] = fmaf(d0, ub_[i + j], gw[s][j]);
       }
-      if (p.du) dw_st<BF>(p.du, ((long)b * p.L + l) * p.C + c, du);
+      if (p.du) dw_st<BF>(p.du, (long)b * p.du_bs + (long)l * p.du_ls + c, du);
     }
   }
   const int ntile = (p.L + DW_TL - 1) / DW_TL;

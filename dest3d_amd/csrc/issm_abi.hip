@@ -486,7 +486,11 @@ static int dwconv_params(const issm_dwconv_args* a, DwConvP* p, bool bwd) {
   p->dy_tail[0] = a->dy_tail[0]; p->dy_tail[1] = a->nsets > 1 ? a->dy_tail[1] : nullptr;
   p->w = a->w; p->bias = a->bias; p->y = a->y; p->pre = a->pre;
   p->dy[0] = a->dy[0]; p->dy[1] = a->nsets > 1 ? a->dy[1] : nullptr;
+  if ((a->du_batch_stride || a->du_token_stride) && (a->du_token_stride < a->channels || a->du_batch_stride < 0))
+    return fail(ISSM_E_STRIDE, "dwconv: du strides (%lld, %lld)", (long long)a->du_batch_stride, (long long)a->du_token_stride);
   p->du = a->du; p->partial = a->partial; p->nrows = dwconv_partial_rows(a->batch, a->seqlen);
+  p->du_ls = a->du_token_stride ? a->du_token_stride : a->channels;
+  p->du_bs = a->du_token_stride ? a->du_batch_stride : (long)a->seqlen * a->channels;
   p->dw = a->dw; p->dbias = a->dbias;
   return ISSM_OK;
 }

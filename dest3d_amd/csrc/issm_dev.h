@@ -121,7 +121,8 @@ struct DwConvP {
   void* pre;           // (nsets, B, L, C) io dtype: convolution output before SiLU (saved for the backward)
   const void* dy[2];   // (B, L, C) io dtype per set, or NULL; with split > 0: (B, L, split)
   const void* dy_tail[2];  // split > 0: (B, L, C - split) per set, or NULL
-  void* du;            // (B, L, C) io dtype
+  void* du;            // (B, L, C) io dtype, element strides du_bs, du_ls, channels contiguous
+  long du_bs, du_ls;
   float* partial;      // (nrows, nsets, 8, C) fp32
   int nrows;
   float* dw;           // (nsets, C, 7) fp32

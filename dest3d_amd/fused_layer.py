@@ -62,7 +62,9 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "issm_dwconv_silu_fwd")
             x_f, x_b = x[0], x[1]
             # 2. dt / B / C (and the reversed-order B / C) from the distance encoding
-            bias = torch.cat([dt_tok.float() + dt_bias32, tail[0].float(), tail[1].float()], -1)
+            bias = torch.empty((Bsz, Ln, H + 4 * G), dtype=torch.float32, device=dev)
+            torch.add(dt_tok, dt_bias32, out=bias[..., :H])
+            bias[..., H:].unflatten(-1, (2, 2 * G)).copy_(tail.permute(1, 2, 0, 3))
             d = dist.detach().to(kdt).contiguous()
             wt = None if weights is None else weights.detach().float().contiguous()
             dt = torch.empty((Bsz, Ln, H, K), dtype=kdt, device=dev)
@@ -75,13 +77,16 @@ class FusedScanCoreFn(torch.autograd.Function):
                 g.weights, g.dt_raw = wt.data_ptr(), raw.data_ptr()
             L.check(lib.issm_param_gen_fwd(C.byref(g)), "issm_param_gen_fwd")
             # 3. the bidirectional scan, queries as initial state
-            A = torch.exp(A_log32).neg_()[:, None].expand(H, K)
+            A1 = torch.exp(A_log32).neg_()
+            A = A1[:, None].expand(H, K)
             h0 = h0_lin.detach().reshape(Bsz, K, H, P).permute(0, 2, 3, 1)
             prob = _Problem([x_f, x_b], dt, A, [bc[0], bc[2]], [bc[1], bc[3]], chunk_size, D.detach(), [None, None], None,
                             h0, None, wt is None, dt_limit)
             outs, finals, ws = _scan_fwd(prob, True)
-            key = torch.add(outs[0], outs[1]).mul_(0.5).view(Bsz * Ln, di)
-            # 4. gated RMSNorm (norm(x * silu(z)))
+            # 4. gated RMSNorm (norm(x * silu(z))) of the two directions' average: the norm of s / 2 with eps is the norm
+            # of s with 4 eps, so the sum goes in as it is and the halving never runs (nor its backward)
+            key = torch.add(outs[0], outs[1]).view(Bsz * Ln, di)
+            eps = 4.0 * eps
             z2 = z.reshape(Bsz * Ln, di) if z.is_contiguous() else z.as_strided((Bsz * Ln, di), (zx.stride(1), 1),
                                                                                  z.storage_offset())
             nw = norm_w.detach()
@@ -91,8 +96,9 @@ class FusedScanCoreFn(torch.autograd.Function):
             n = _ln._norm_args(key, z2, nw, eps, None, False)
             n.y, n.y_row_stride, n.rstd = key_n.data_ptr(), key_n.stride(0), rstd.data_ptr()
             L.check(lib.issm_gated_rmsnorm_fwd(C.byref(n)), "issm_gated_rmsnorm_fwd")
-            last = torch.add(finals[0], finals[1]).mul_(0.5).permute(0, 3, 1, 2).reshape(Bsz, K, di)
-        ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log32)
+            last = torch.lerp(finals[0].permute(0, 3, 1, 2), finals[1].permute(0, 3, 1, 2), 0.5,
+                              out=torch.empty((Bsz, K, H, P), dtype=finals[0].dtype, device=dev)).view(Bsz, K, di)
+        ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A1)
         ctx.prob, ctx.ws = prob, ws
         ctx.meta = (Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, st)
         ctx.dtypes = tuple(t.dtype for t in (zxbcdt, h0_lin, dist, conv_w_f, conv_b_f, conv_w_b, conv_b_b, dt_w, bc_w,
@@ -103,7 +109,7 @@ class FusedScanCoreFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dkey_n, dlast):
         lib = L.load()
-        xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A_log = ctx.saved_tensors
+        xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A1 = ctx.saved_tensors
         Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, _ = ctx.meta
         prob = ctx.prob
         dev = key.device
@@ -112,7 +118,8 @@ class FusedScanCoreFn(torch.autograd.Function):
             # 4'. gated RMSNorm
             dy = dkey_n.to(kdt).reshape(Bsz * Ln, di).contiguous()
             dkey = torch.empty_like(key)
-            dz = torch.empty_like(key)
+            Wd = di + Cc + H                      # row of d zxbcdt: [dz | d xbc | d dt]; each producer writes its part
+            dzx = torch.empty((Bsz, Ln, Wd), dtype=kdt, device=dev)
             nb = lib.issm_rmsnorm_bwd_blocks(Bsz * Ln)
             dwp = torch.empty((nb, di), dtype=torch.float32, device=dev)
             dnw = torch.empty(di, dtype=torch.float32, device=dev)
@@ -120,12 +127,13 @@ class FusedScanCoreFn(torch.autograd.Function):
             n.rstd = rstd.data_ptr()
             n.dy, n.dy_row_stride = dy.data_ptr(), dy.stride(0)
             n.dx, n.dx_row_stride = dkey.data_ptr(), dkey.stride(0)
-            n.dz, n.dz_row_stride = dz.data_ptr(), dz.stride(0)
+            n.dz, n.dz_row_stride = dzx.data_ptr(), Wd
             n.dw_partial, n.dw = dwp.data_ptr(), dnw.data_ptr()
             L.check(lib.issm_gated_rmsnorm_bwd(C.byref(n)), "issm_gated_rmsnorm_bwd")
-            # 3'. the scan: both directions receive half of the averaged outputs' gradients
-            dyh = dkey.mul_(0.5).view(Bsz, Ln, H, P)
-            dfin = dlast.float().reshape(Bsz, K, H, P).permute(0, 2, 3, 1).mul(0.5).contiguous()
+            # 3'. the scan: both directions receive the gradient of their sum, and half of the averaged final states'
+            dyh = dkey.view(Bsz, Ln, H, P)
+            dfin = torch.mul(dlast.reshape(Bsz, K, H, P).permute(0, 2, 3, 1), 0.5,
+                             out=torch.empty((Bsz, H, P, K), dtype=torch.float32, device=dev))
             dxs, ddt, dA, dBs, dCs, dD, _, _, dh0 = _scan_bwd(prob, ctx.ws, [dyh, dyh], [dfin, dfin], want_dz=False)
             # 2'. parameter generation
             R0, R = H + 2 * G, H + 4 * G
@@ -143,8 +151,8 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_param_gen_bwd(C.byref(g)), "issm_param_gen_bwd")
             d_dt_tok = dbias[..., :H]
             # 1'. the convolutions: gradients of (x, b-bias, c-bias) per branch
-            dtail = [dbias[..., H:H + 2 * G].to(kdt).contiguous(), dbias[..., H + 2 * G:].to(kdt).contiguous()]
-            dxbc = torch.empty((Bsz, Ln, Cc), dtype=kdt, device=dev)
+            dtail = torch.empty((2, Bsz, Ln, 2 * G), dtype=kdt, device=dev)
+            dtail.copy_(dbias[..., H:].unflatten(-1, (2, 2 * G)).permute(2, 0, 1, 3))
             rows = lib.issm_dwconv_partial_rows(Bsz, Ln)
             part = torch.empty((max(rows, 1), 2, 8, Cc), dtype=torch.float32, device=dev)
             dcw = torch.empty((2, Cc, _dw.TAPS), dtype=torch.float32, device=dev)
@@ -154,10 +162,12 @@ class FusedScanCoreFn(torch.autograd.Function):
             a.split = di
             a.dy[0], a.dy[1] = dxs[0].data_ptr(), dxs[1].data_ptr()
             a.dy_tail[0], a.dy_tail[1] = dtail[0].data_ptr(), dtail[1].data_ptr()
-            a.du, a.partial, a.dw, a.dbias = dxbc.data_ptr(), part.data_ptr(), dcw.data_ptr(), dcb.data_ptr()
+            a.du = dzx.data_ptr() + di * dzx.element_size()
+            a.du_batch_stride, a.du_token_stride = Ln * Wd, Wd
+            a.partial, a.dw, a.dbias = part.data_ptr(), dcw.data_ptr(), dcb.data_ptr()
             L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "issm_dwconv_silu_bwd")
-            dzx = torch.cat([dz.view(Bsz, Ln, di), dxbc, d_dt_tok.to(kdt)], -1)
-            dA_log = dA.sum(-1).mul_(torch.exp(A_log).neg_())
+            dzx[..., di + Cc:].copy_(d_dt_tok)
+            dA_log = dA.sum(-1).mul_(A1)
             dh0_lin = dh0.permute(0, 3, 1, 2).reshape(Bsz, K, di)
             ddt_bias = d_dt_tok.sum((0, 1))
             # parameter gradients: one buffer, one conversion to the parameters' dtype when they share one

@@ -285,7 +285,7 @@ int issm_param_gen_bwd(const issm_pgen_args* args);
  * tensors instead, y (nsets, B, L, split) for channels [0, split) and y_tail (nsets, B, L, C - split) for the rest
  * (MultiHeadISSMScan splits the result into x and the B / C biases, dest_module.py:532), and the backward takes
  * dy[s] (B, L, split) and dy_tail[s] (B, L, C - split).  Backward: dy[s] (B, L, C) contiguous or NULL
- * (zero); du (B, L, C) contiguous; dw (nsets, C, 7), dbias (nsets, C) fp32; partial:
+ * (zero); du (B, L, C), contiguous unless the du strides say otherwise; dw (nsets, C, 7), dbias (nsets, C) fp32; partial:
  * issm_dwconv_partial_rows(B, L) * nsets * 8 * C floats of scratch. */
 typedef struct issm_dwconv_args {
   int32_t batch, seqlen, channels, nsets, taps; /* taps must be 7 */
@@ -307,6 +307,8 @@ typedef struct issm_dwconv_args {
   int32_t split;
   void* y_tail;
   const void* dy_tail[2];
+  /* element strides of du (0, 0 = contiguous (B, L, C)): lets the gradient land inside a wider row */
+  int64_t du_batch_stride, du_token_stride;
 } issm_dwconv_args;
 
 int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);
