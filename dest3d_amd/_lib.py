@@ -94,7 +94,7 @@ class PGenArgs(C.Structure):
         ("dCm_back", C.c_void_p),
         ("ddist", C.c_void_p), ("dbias", C.c_void_p), ("dweights", C.c_void_p),
         ("dw_partial", C.c_void_p), ("dW", C.c_void_p),
-        ("stream", C.c_void_p),
+        ("stream", C.c_void_p), ("dbias_sum", C.c_void_p),
     ]
 
 

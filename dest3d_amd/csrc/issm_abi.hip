@@ -444,6 +444,8 @@ static int pgen_params(const issm_pgen_args* a, PGenP* p, bool bwd) {
   p->dt = a->dt; p->Bm = a->Bm; p->Cm = a->Cm; p->Bb = a->Bm_back; p->Cb = a->Cm_back;
   p->ddt = a->ddt; p->dB = a->dBm; p->dC = a->dCm; p->dBb = a->dBm_back; p->dCb = a->dCm_back;
   p->weights = a->weights; p->dt_raw = a->dt_raw; p->dweights = a->weights ? a->dweights : nullptr;
+  if (a->dbias_sum && !a->dbias) return fail(ISSM_E_NULL, "param_gen: dbias_sum needs dbias");
+  p->dbias_sum = a->dbias_sum;
   p->ddist = a->ddist; p->dbias = a->dbias; p->dw_partial = a->dw_partial; p->dW = a->dW;
   p->nblocks = pgen_bwd_blocks(a->tokens);
   return ISSM_OK;

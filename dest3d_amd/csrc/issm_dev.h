@@ -143,6 +143,7 @@ struct PGenP {
   const void *ddt, *dB, *dC, *dBb, *dCb;           // gradients of the outputs
   void* ddist;           // (tokens, K, M) io dtype
   float* dbias;          // (tokens, R) fp32
+  float* dbias_sum;      // (R) fp32 or NULL: dbias summed over the tokens
   float* dw_partial;     // (nblocks, R0, M) fp32
   float* dW;             // (R0, M) fp32
   int nblocks;

@@ -387,18 +387,29 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
     p.dw_partial[(long)blockIdx.x * R0 * PG_M + e] = (wred[0][e] + wred[1][e]) + (wred[2][e] + wred[3][e]);
 }
 
-// dW = fixed-order sum of the per-workgroup partials: one workgroup per entry of dW
+// dW = fixed-order sum of the per-workgroup partials: one workgroup per entry of dW; the workgroups after those sum
+// one column of dbias over the tokens each (same tree, so both are reproducible)
 __global__ __launch_bounds__(NTHREADS) void k_pgen_dw(PGenP p) {
   __shared__ float red[NTHREADS];
   const int n = (p.H + 2 * p.G) * PG_M;
   const int c = blockIdx.x;
   float a0 = 0.0f, a1 = 0.0f;
-  int b = threadIdx.x;
-  for (; b + NTHREADS < p.nblocks; b += 2 * NTHREADS) {
-    a0 += p.dw_partial[(long)b * n + c];
-    a1 += p.dw_partial[(long)(b + NTHREADS) * n + c];
+  if (c < n) {
+    int b = threadIdx.x;
+    for (; b + NTHREADS < p.nblocks; b += 2 * NTHREADS) {
+      a0 += p.dw_partial[(long)b * n + c];
+      a1 += p.dw_partial[(long)(b + NTHREADS) * n + c];
+    }
+    if (b < p.nblocks) a0 += p.dw_partial[(long)b * n + c];
+  } else {
+    const int R = p.H + 2 * p.G + (p.has_back ? 2 * p.G : 0), r = c - n;
+    long t = threadIdx.x;
+    for (; t + NTHREADS < p.tokens; t += 2 * NTHREADS) {
+      a0 += p.dbias[t * R + r];
+      a1 += p.dbias[(t + NTHREADS) * R + r];
+    }
+    if (t < p.tokens) a0 += p.dbias[t * R + r];
   }
-  if (b < p.nblocks) a0 += p.dw_partial[(long)b * n + c];
   red[threadIdx.x] = a0 + a1;
   __syncthreads();
 #pragma unroll
@@ -406,7 +417,10 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_dw(PGenP p) {
     if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) p.dW[c] = red[0];
+  if (threadIdx.x == 0) {
+    if (c < n) p.dW[c] = red[0];
+    else p.dbias_sum[c - n] = red[0];
+  }
 }
 
 int pgen_bwd_blocks(long tokens) { return (int)((tokens + PG_TOK - 1) / PG_TOK); }
@@ -437,7 +451,8 @@ int launch_pgen_bwd(const PGenP& p, hipStream_t st) {
   }
   int e = (int)hipGetLastError();
   if (e) return e;
-  hipLaunchKernelGGL(k_pgen_dw, dim3(R0 * PG_M), dim3(NTHREADS), 0, st, p);
+  const int R = R0 + (p.has_back ? 2 * p.G : 0);
+  hipLaunchKernelGGL(k_pgen_dw, dim3(R0 * PG_M + (p.dbias_sum ? R : 0)), dim3(NTHREADS), 0, st, p);
   return (int)hipGetLastError();
 }
 

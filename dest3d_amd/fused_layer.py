@@ -146,6 +146,8 @@ class FusedScanCoreFn(torch.autograd.Function):
             dW = torch.empty((R0, 16), dtype=torch.float32, device=dev)
             g.ddist = None if ddist is None else ddist.data_ptr()
             g.dbias, g.dw_partial, g.dW = dbias.data_ptr(), dwpart.data_ptr(), dW.data_ptr()
+            dbias_sum = torch.empty(R, dtype=torch.float32, device=dev)
+            g.dbias_sum = dbias_sum.data_ptr()
             if wt is not None:
                 g.weights, g.dt_raw = wt.data_ptr(), raw.data_ptr()
             L.check(lib.issm_param_gen_bwd(C.byref(g)), "issm_param_gen_bwd")
@@ -169,7 +171,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             dzx[..., di + Cc:].copy_(d_dt_tok)
             dA_log = dA.sum(-1).mul_(A1)
             dh0_lin = dh0.permute(0, 3, 1, 2).reshape(Bsz, K, di)
-            ddt_bias = d_dt_tok.sum((0, 1))
+            ddt_bias = dbias_sum[:H]
             # parameter gradients: one buffer, one conversion to the parameters' dtype when they share one
             grads = [dcw[0], dcb[0], dcw[1], dcb[1], dW[:H], dW[H:], ddt_bias, dA_log, dD, dnw]
             pdts = (wfdt, bfdt, wbdt, bbdt, dtwdt, bcwdt, dtbdt, aldt, Ddt, nwdt)

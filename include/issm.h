@@ -247,7 +247,8 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
  * MultiHeadISSMScan multiplies into dt (dest_module.py:553-559): when given, dt = softplus(raw) * weights
  * (softplus with torch's threshold 20), the raw values go to dt_raw (tokens, H, K, `dtype`; required then, and
  * read back by the backward), and dweights (tokens, K) fp32, if not NULL, receives
- * sum_h ddt[t][h][k] * softplus(raw[t][h][k]). */
+ * sum_h ddt[t][h][k] * softplus(raw[t][h][k]).  dbias_sum needs dbias (it is summed in a fixed order after it
+ * is written). */
 typedef struct issm_pgen_args {
   int64_t tokens;
   int32_t K, M, H, G;
@@ -267,6 +268,7 @@ typedef struct issm_pgen_args {
   float* dw_partial;
   float* dW;
   void* stream;
+  float* dbias_sum; /* optional, (R) fp32: dbias summed over the tokens (the dt_bias parameter's gradient is its first H) */
 } issm_pgen_args;
 
 int issm_param_gen_bwd_blocks(int64_t tokens);
