@@ -44,11 +44,14 @@ def test_box_dist_forward_and_table_gradient(case):
     dist = box_dist(t, tk, corners, ta if angles else None)
     ref = R.box_dist(key, qxyz, qsize, ang, table)
     assert dist.shape == (B, nP, nQ, 16) and dist.is_contiguous()
-    assert _rel(dist.detach().cpu().numpy(), ref) <= 1e-4
+    e_fwd = _rel(dist.detach().cpu().numpy(), ref)
+    assert e_fwd <= 2e-5
     g = rng.standard_normal(ref.shape).astype(np.float32)
     dist.backward(torch.from_numpy(g).cuda())
     gref = R.box_dist_table_grad(key, qxyz, qsize, ang, table.shape, g)
-    assert _rel(t.grad.cpu().numpy(), gref) <= 1e-4
+    e_bwd = _rel(t.grad.cpu().numpy(), gref)
+    print(f"    pairs {B * nP * nQ}: dist err {e_fwd:.2e}, table gradient err {e_bwd:.2e}", flush=True)
+    assert e_bwd <= 2e-5
     # bf16 output
     dist_bf = box_dist(t.detach(), tk, corners, ta if angles else None, out_dtype=torch.bfloat16)
     assert dist_bf.dtype == torch.bfloat16
