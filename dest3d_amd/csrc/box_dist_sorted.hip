@@ -203,13 +203,13 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_fill(BoxDistP p, SortP s) {
   });
 }
 
-// weights of one axis over the window's three nodes: the corner's base node is `i`, its fraction `f`, the window
-// starts at `m`.  A base node outside [m, m + 1] can only come from a position within rounding of a node, where the
-// weight it would carry is ~0: such parts are dropped.
-__device__ __forceinline__ void axis3(int i, float f, int m, float (&a)[3]) {
-  const int s0 = i - m;
+// Trilinear weights of one axis over the window's three nodes m, m + 1, m + 2 for a sample at node position x: the
+// hat function max(0, 1 - |x - node|), which is (1 - f, f) on the two nodes around x and zero on the third -- no
+// floor, no case distinction.  (An entry only holds corners whose base node is m or m + 1.)
+__device__ __forceinline__ void axis3(float x, float m, float (&a)[3]) {
+  const float t = x - m;
 #pragma unroll
-  for (int j = 0; j < 3; ++j) a[j] = (s0 == j ? 1.0f - f : 0.0f) + (s0 + 1 == j ? f : 0.0f);
+  for (int j = 0; j < 3; ++j) a[j] = fmaxf(1.0f - fabsf(t - (float)j), 0.0f);
 }
 
 // 4 x 4 transpose of bytes: in q[0..3] byte d of q[r] is digit d of entry r; out t[d] holds digit d of the four
@@ -253,6 +253,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
   if (item >= (int)s.scal[1]) return;  // uniform
   const int bin = s.items[3 * item], first = s.items[3 * item + 1], last = s.items[3 * item + 2];
   const int mx = bin % (p.W + 2) - 2, my = (bin / (p.W + 2)) % (p.H + 2) - 2, mz = bin / ((p.W + 2) * (p.H + 2)) - 2;
+  const float fmx = (float)mx, fmy = (float)my, fmz = (float)mz;
   const float scale = 1.0f / (3.0f * p.max_value);
   const float g_scale = bds_scale(s.scal);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, kg = lane >> 4;
@@ -287,11 +288,10 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
           float x, y, z;
           corner_pos(p, bt[c >> 2][c & 3], bt[2 + (c >> 2)][c & 3], bt[4 + (c >> 2)][c & 3], bt[6 + (c >> 2)][c & 3],
                      bt[8 + (c >> 2)][c & 3], kx, ky, kz, scale, x, y, z);
-          const float gx = floorf(x), gy = floorf(y), gz = floorf(z);
           float ax[3], ay[3], az[3];
-          axis3((int)gx, x - gx, mx, ax);
-          axis3((int)gy, y - gy, my, ay);
-          axis3((int)gz, z - gz, mz, az);
+          axis3(x, fmx, ax);
+          axis3(y, fmy, ay);
+          axis3(z, fmz, az);
 #pragma unroll
           for (int i = 0; i < 3; ++i)
 #pragma unroll
