@@ -333,9 +333,9 @@ int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
  * contiguous in `dtype`.  Either output of the forward may be NULL (skipped).  The backward produces the table
  * gradient only (the reference detaches the corners; key positions and angles are inputs); partial:
  * issm_box_dist_bwd_scratch_bytes(...) bytes of scratch, 16-byte aligned (about 64 bytes per pair for large
- * problems: the pairs are sorted by the table cells they touch).  The gradient is accumulated in 64-bit fixed
- * point scaled to max|ddist|, so it does not depend on the order of the adds (reproducible bit for bit; absolute
- * resolution 2^-24 max|ddist| per term); at most 2^26 (point, box) pairs per call. */
+ * problems: the pairs are sorted by the table cells they touch).  The gradient is accumulated in integers -- for
+ * large problems weights in units of 2^-24 and ddist in units of 2^-22 max|ddist|, exact products and sums -- so it
+ * does not depend on the order of the adds (reproducible bit for bit); at most 2^26 (point, box) pairs per call. */
 typedef struct issm_box_dist_args {
   int32_t batch, seqlen, nquery, D, H, W;
   int32_t dtype;
