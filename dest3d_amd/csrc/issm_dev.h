@@ -385,14 +385,27 @@ __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t
 struct Unit {
   int b, dir, bt, c, h, g;
 };
+// Order of the units: heads fastest.  With two directions the next index is the direction, and chunk j of the
+// forward direction is paired with chunk nc - 1 - j of the reversed one: the same block of tokens, so the two
+// workgroups that read one head's dt tile (the largest operand, shared by the directions) run side by side on one
+// XCD and the second read is served by its L2.
 __device__ __forceinline__ Unit decode_unit(const KP& p, int u) {
   Unit r;
   r.h = u % p.H;
   u /= p.H;
-  r.c = u % p.nc;
-  r.bt = u / p.nc;
-  r.dir = r.bt % p.ndir;
-  r.b = r.bt / p.ndir;
+  if (p.ndir == 2) {
+    r.dir = u & 1;
+    u >>= 1;
+    const int j = u % p.nc;
+    r.b = u / p.nc;
+    r.c = r.dir ? p.nc - 1 - j : j;
+    r.bt = r.b * 2 + r.dir;
+  } else {
+    r.c = u % p.nc;
+    r.bt = u / p.nc;
+    r.dir = r.bt % p.ndir;
+    r.b = r.bt / p.ndir;
+  }
   r.g = r.h / p.hpg;
   return r;
 }
