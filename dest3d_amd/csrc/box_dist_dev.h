@@ -185,7 +185,7 @@ __device__ __forceinline__ Items my_items(const BoxDistP& p) {
 // is the bound the launcher checks).
 __device__ __forceinline__ float bd_scale(const unsigned* scal) {
   const float gmax = __uint_as_float(scal[0]);
-  return gmax > 0.0f ? 17179869184.0f / gmax : 1.0f;
+  return gmax > 1e-27f ? 17179869184.0f / gmax : 1.0f;  // below that the quotient could overflow; such gradients round to 0
 }
 
 

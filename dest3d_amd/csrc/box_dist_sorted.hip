@@ -45,7 +45,7 @@ struct SortP {
 constexpr float BDS_W_SCALE = 16777216.0f;
 __device__ __forceinline__ float bds_scale(const unsigned* scal) {
   const float gmax = __uint_as_float(scal[0]);
-  return gmax > 0.0f ? 4194304.0f / gmax : 1.0f;
+  return gmax > 1e-30f ? 4194304.0f / gmax : 1.0f;  // below that the quotient could overflow; such gradients round to 0
 }
 
 __device__ __forceinline__ int bds_bin(const BoxDistP& p, int mx, int my, int mz) {

@@ -105,6 +105,21 @@ def test_table_gradient_is_bit_reproducible():
     t = torch.randn(16, 10, 10, 10, generator=torch.Generator().manual_seed(2)).cuda().requires_grad_()
     box_dist(t, tk, corners).backward(torch.zeros_like(g))
     assert t.grad.abs().max().item() == 0.0
+    # the fixed point is scaled to max|ddist|: upstream gradients of any magnitude give the same relative result,
+    # vanishing ones a finite (zero) one; both sides of the 65536-pair switch between the two accumulation paths
+    for npts in (200, 20):
+        gs = g[:, :npts].contiguous()
+        ref = None
+        for scale in (1.0, 1e30, 1e-25, 1e-37):
+            t = torch.randn(16, 10, 10, 10, generator=torch.Generator().manual_seed(2)).cuda().requires_grad_()
+            box_dist(t, tk[:, :npts].contiguous(), corners).backward(gs * scale)
+            assert torch.isfinite(t.grad).all()
+            if ref is None:
+                ref = t.grad.double()
+            elif scale > 1e-30:
+                assert _rel((t.grad.double() / scale).cpu().numpy(), ref.cpu().numpy()) <= 1e-6, (npts, scale)
+            else:
+                assert t.grad.abs().max().item() <= 1e-30
 
 
 def test_box_dist_rejects_unbuilt_shapes():
