@@ -5,14 +5,16 @@
 // first sorted by where they land: a pair contributes one *entry* per window of 3 x 3 x 3 nodes it touches (one if
 // its corners are on one side of the point, two if it straddles the point along one axis, ...), entries are binned
 // by window anchor with a counting sort, and then all entries of a bin share their 27 nodes, so the gradient of a
-// bin is a dense (27 x entries) . (entries x 16) product accumulated in registers.  Passes:
+// bin is a dense (27 x entries) . (entries x 16) product, taken exactly on the int8 matrix cores.  Passes:
+//   gmax, boxes   max|ddist| (scale of the fixed point); corners and rotations of every box, once
 //   count   workgroup histograms of the entries' bins (LDS integer atomics, one per entry)
 //   plan    bin offsets and the list of work items (bin, range of at most BDS_SEG entries); then each counting
 //           workgroup's base inside each bin (a scan over workgroups, so the ranges do not depend on timing)
 //   fill    the same walk again, writing each entry's record (pair index, corner mask) into its bin
 //   accum   one workgroup per work item: 256 entries at a time, lane = entry recomputes the window weights of its
-//           corners and stages them with ddist in LDS; then thread = (node of the window, channel) adds
-//           weight * ddist over the entries, in 64-bit fixed point (order-independent, hence reproducible)
+//           corners and stages them with ddist in LDS as fixed-point values split into signed base-256 digits; each
+//           wave then multiplies its 64 entries' digits with v_mfma_i32_16x16x64_i8 (integer sums: order-independent,
+//           hence reproducible)
 //   scatter / finish   work-item results into the table (integer atomics in global memory, a few 10^5), then float.
 #include "box_dist_dev.h"
 
