@@ -450,7 +450,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
   for (int hh = 0; hh < p.hpg; ++hh) {
-    u.h = u.g * p.hpg + hh;
+    // the reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
+    // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first
+    u.h = u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh);
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
