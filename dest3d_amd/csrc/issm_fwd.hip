@@ -349,7 +349,6 @@ template <int PT>
 struct FwdScanSmem {
   static constexpr int LDPT = PT * 16 + 4;
   float xs[CS * LDPT];      // x [s][p]
-  float ms[CS * LDC];       // tril(M) [l][s]
   float ct[CS * LDN];       // C * exp2(cs) [l][n]
   float hs[PT * 16 * LDN];  // H [p][n]
 };
@@ -377,13 +376,27 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   cf = lane_coef(p, u.h, n, vn);
   lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
   pn_load<PT>(p, hsrc, 0, hv);
+  // M of this wave's 16 rows goes straight into matrix-operand registers (lane (row cm, group g4) holds columns
+  // 16 kb + 4 g4 .. + 3 of the blocks kb <= wave, the upper triangle of the diagonal block zeroed): no LDS tile, which
+  // lets a fourth workgroup live on the CU
+  f4 mf[4];
+  {
+    const float* mrow = cabt + sq_off(p, u.bt, u.c, u.h) + (wave * 16 + cm) * CS + 4 * g4;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      mf[kb] = (f4){0, 0, 0, 0};
+      if (kb <= wave) mf[kb] = *(const f4*)(mrow + 16 * kb);
+      if (kb == wave) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (4 * g4 + j > cm) mf[kb][j] = 0.0f;
+      }
+    }
+  }
   {
     float xv[CS * PT * 16 / NTHREADS];
-    f4 mv[4];
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
-    tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
     lp_store<PT>(xv, s.xs, LDPT);
-    tril_store(mv, s.ms);
   }
   f4 acc[PT];
 #pragma unroll
@@ -416,9 +429,18 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     __syncthreads();
   }
   // y[l][p] += sum_{s<=l} M[l][s] x[s][p]; rows of this wave only need s < 16(wave+1)
-  for (int kb = 0; kb < (wave + 1) * 16; kb += 16)
 #pragma unroll
-    for (int pt = 0; pt < PT; ++pt) mma16_mk(acc[pt], s.ms, LDC, wave * 16, s.xs, LDPT, pt * 16, kb, lane);
+  for (int kb = 0; kb < 4; ++kb)
+    if (kb <= wave) {  // uniform
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt) {
+        const float* bp = s.xs + (16 * kb + 4 * g4) * LDPT + pt * 16 + cm;
+        acc[pt] = mfma4(mf[kb][0], bp[0], acc[pt]);
+        acc[pt] = mfma4(mf[kb][1], bp[LDPT], acc[pt]);
+        acc[pt] = mfma4(mf[kb][2], bp[2 * LDPT], acc[pt]);
+        acc[pt] = mfma4(mf[kb][3], bp[3 * LDPT], acc[pt]);
+      }
+    }
 
   const TensorD& to = p.out[u.dir];
   const TensorD& tz = p.z[u.dir];
