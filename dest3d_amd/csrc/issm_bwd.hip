@@ -645,14 +645,13 @@ template <int PT>
 struct BwdDxSmem {
   static constexpr int LDPT = PT * 16 + 4;
   float dys[CS * LDPT];
-  float ms[CS * LDC];
   float bt[CS * LDN];       // B dt' exp2(last - cs) [m][n]; later dy*x products
   float dss[PT * 16 * LDN]; // dS [p][n]
 };
 
 // partD: (Bt*nc*H, P) per-unit sums over rows of dy*x
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restrict__ dy_ws,
+__global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(KP p, const float* __restrict__ dy_ws,
                                                      const float* __restrict__ dstates,
                                                      const float* __restrict__ cabt, float* __restrict__ partD) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -675,13 +674,25 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
   cf = lane_coef(p, u.h, n, vn);
   lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
   pn_load<PT>(p, ds, 0, sv);
+  // M^T of this wave's 16 columns goes straight into matrix-operand registers (lane (column cm, group g4) holds
+  // rows 16 kb + 4 g4 .. + 3 of the blocks kb >= wave, the upper triangle of the diagonal block zeroed): no LDS tile,
+  // which lets a fourth workgroup live on the CU
+  float mf[4][4];
+  {
+    const float* mcol = cabt + sq_off(p, u.bt, u.c, u.h) + (4 * g4) * CS + wave * 16 + cm;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mf[kb][j] = 0.0f;
+        if (kb >= wave) mf[kb][j] = mcol[(16 * kb + j) * CS];
+        if (kb == wave && cm > 4 * g4 + j) mf[kb][j] = 0.0f;
+      }
+  }
   {
     float dv[CS * PT * 16 / NTHREADS];
-    f4 mv[4];
     dy_load<IOB, PT, FULL>(p, u, dy_ws, dv);
-    tril_load(cabt + sq_off(p, u.bt, u.c, u.h), mv);
     lp_store<PT>(dv, s.dys, LDPT);
-    tril_store(mv, s.ms);
   }
   f4 acc[PT];
 #pragma unroll
@@ -713,9 +724,16 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dx(KP p, const float* __restri
     __syncthreads();
   }
   // dx[m][p] += sum_{l>=m} M[l][m] dy[l][p]
-  for (int kb = wave * 16; kb < CS; kb += 16)
 #pragma unroll
-    for (int pt = 0; pt < PT; ++pt) mma16_kk(acc[pt], s.ms, LDC, wave * 16, s.dys, LDPT, pt * 16, kb, lane);
+  for (int kb = 0; kb < 4; ++kb)
+    if (kb >= wave) {  // uniform
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt) {
+        const float* bp = s.dys + (16 * kb + 4 * g4) * LDPT + pt * 16 + cm;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[pt] = mfma4(mf[kb][j], bp[j * LDPT], acc[pt]);
+      }
+    }
 
   const TensorD& tx = p.x[u.dir];
   const TensorD& tdx = p.dx[u.dir];
