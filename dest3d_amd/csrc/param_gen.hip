@@ -162,7 +162,7 @@ __device__ __forceinline__ float dsoftplus_(float x) { return x <= 20.0f ? sigmo
 // FULLK: K is a multiple of 64, so no load or store needs a bound on k, and every per-lane address is a
 // pointer advanced once per trip plus a compile-time offset.  UNR blocks of 16 k have their loads in flight together.
 template <bool BF, bool FULLK, bool HASW>
-__global__ __launch_bounds__(NTHREADS) void k_pgen_bwd(PGenP p) {
+__global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
   constexpr int UNR = HASW ? 2 : 4;
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   typedef typename std::conditional<BF, uint2, f4>::type T4;
