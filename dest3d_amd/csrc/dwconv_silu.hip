@@ -108,16 +108,18 @@ __global__ __launch_bounds__(NTHREADS) void k_dwconv_bwd(DwConvP p) {
 #pragma unroll
     for (int s = 0; s < S; ++s) {
       const long o = ((long)b * p.L + lc) * p.C + c;
-      float dyv = 0.0f;
-      if (p.split > 0) {  // uniform: the gradient arrives as the two dense tensors of the forward
-        const long row = (long)b * p.L + lc;
-        if (c < p.split) { if (p.dy[s]) dyv = dw_ld<BF>(p.dy[s], row * p.split + c); }
-        else if (p.dy_tail[s]) dyv = dw_ld<BF>(p.dy_tail[s], row * (p.C - p.split) + (c - p.split));
-      } else if (p.dy[s]) {
-        dyv = dw_ld<BF>(p.dy[s], o);
-      }
+      // with a split the gradient arrives as the two dense tensors of the forward: which one a lane reads is chosen
+      // by selecting the address, not by a branch (an absent tensor reads `pre` and counts as zero), so that all
+      // loads of the thread stay in flight together
+      const bool head = p.split <= 0 || c < p.split;
+      const void* src = head ? p.dy[s] : p.dy_tail[s];
+      const long row = (long)b * p.L + lc;
+      long off = o;
+      if (p.split > 0) off = head ? row * p.split + c : row * (p.C - p.split) + (c - p.split);  // uniform condition
+      const bool have = src != nullptr;
+      const float dyv = dw_ld<BF>(have ? src : p.pre, have ? off : o);
       const float pv = dw_ld<BF>(p.pre, (long)s * p.B * p.L * p.C + o);
-      dyb[s][j] = in ? dyv : 0.0f;
+      dyb[s][j] = (in && have) ? dyv : 0.0f;
       prb[s][j] = in ? pv : 0.0f;
     }
   }
