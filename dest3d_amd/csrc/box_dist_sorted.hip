@@ -281,6 +281,13 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
       const int l = (int)(bl % (unsigned)p.L), b = (int)(bl / (unsigned)p.L);
       const float* key = p.key + ((long)b * p.L + l) * 3;
       const float kx = key[0], ky = key[1], kz = key[2];
+      // ddist of the pair: requested before the corner loop (and unpacked after it) so that its latency runs under it
+      uint4 graw[4];
+      {
+        const uint4* src = (const uint4*)((const char*)p.ddist + (long)pid * BD_C * (BF ? 2 : 4));
+#pragma unroll
+        for (int j = 0; j < (BF ? 2 : 4); ++j) graw[j] = src[j];
+      }
       f4 bt[10];  // the box: x[8], y[8], z[8], cos[8], sin[8]
 #pragma unroll
       for (int j = 0; j < 10; ++j) bt[j] = *(const f4*)(s.boxtab + ((long)b * p.K + k) * 40 + 4 * j);
@@ -305,20 +312,17 @@ __global__ __launch_bounds__(NTHREADS) void k_bds_accum(BoxDistP p, SortP s) {
         }
       }
       if (BF) {
-        const uint4* src = (const uint4*)((const uint16_t*)p.ddist + (long)pid * BD_C);
-        const uint4 a = src[0], c = src[1];
-        g[0] = (f4){__uint_as_float(a.x << 16), __uint_as_float(a.x & 0xffff0000u), __uint_as_float(a.y << 16),
-                    __uint_as_float(a.y & 0xffff0000u)};
-        g[1] = (f4){__uint_as_float(a.z << 16), __uint_as_float(a.z & 0xffff0000u), __uint_as_float(a.w << 16),
-                    __uint_as_float(a.w & 0xffff0000u)};
-        g[2] = (f4){__uint_as_float(c.x << 16), __uint_as_float(c.x & 0xffff0000u), __uint_as_float(c.y << 16),
-                    __uint_as_float(c.y & 0xffff0000u)};
-        g[3] = (f4){__uint_as_float(c.z << 16), __uint_as_float(c.z & 0xffff0000u), __uint_as_float(c.w << 16),
-                    __uint_as_float(c.w & 0xffff0000u)};
-      } else {
-        const f4* src = (const f4*)((const float*)p.ddist + (long)pid * BD_C);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) g[j] = src[j];
+        for (int j = 0; j < 2; ++j) {
+          const uint4 v = graw[j];
+          g[2 * j] = (f4){__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                          __uint_as_float(v.y & 0xffff0000u)};
+          g[2 * j + 1] = (f4){__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xffff0000u), __uint_as_float(v.w << 16),
+                              __uint_as_float(v.w & 0xffff0000u)};
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) g[j] = __builtin_bit_cast(f4, graw[j]);
       }
     }
     // a weight is at most 8 (eight corners on one node): 2^27 as an integer; |ddist * g_scale| <= 2^22 (three digits)
