@@ -51,45 +51,44 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd(NormP p) {
 
 // ---- fast paths: one group per row, ncols a multiple of 4 and at most 1024 ---------------------------------
 // A lane owns vectors lane, lane + 64, ... of 4 consecutive columns; the row stays in registers between the
-// reduction and the second use, loads and stores are as wide as each tensor's row alignment allows (8 bytes for
-// bf16, 16 for fp32 when aligned), and the backward keeps its dw partial in registers instead of
-// read-modify-writing LDS.
-// `al` (uniform per tensor): 0 = the 4 elements are aligned for one load, 1 = for two half loads, 2 = element loads
+// reduction and the second use, loads and stores are 8 bytes (bf16) or 16 bytes (fp32) wide, and the backward keeps
+// its dw partial in registers instead of read-modify-writing LDS.
+// Rows may start at any element (a column slice of a wider row): the 4 elements are read through a type that only
+// promises element alignment, which the compiler turns into one wide access on this target (unaligned global
+// accesses are legal on gfx9 under HSA) -- one code path, no case distinction around the loads.  `al` is unused.
+struct __attribute__((packed, aligned(2))) RowBf4 {
+  unsigned lo, hi;
+};
+struct __attribute__((packed, aligned(4))) RowF4 {
+  float x, y, z, w;
+};
 template <bool BF>
-__device__ __forceinline__ f4 ld4(const void* p, long off, bool ok, int al) {
-  f4 r = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (!ok) return r;
+__device__ __forceinline__ f4 ld4(const void* p, long off, bool ok, int /*al*/) {
+  // an absent lane reads offset 0 and the value is replaced by zero: no branch around the load, so that a thread's
+  // loads stay in flight together
+  f4 r;
+  off = ok ? off : 0;
   if (BF) {
-    const uint16_t* q = (const uint16_t*)p + off;
-    uint2 w;
-    if (al == 0) w = *(const uint2*)q;
-    else if (al == 1) w = make_uint2(*(const unsigned*)q, *(const unsigned*)(q + 2));
-    else w = make_uint2((unsigned)q[0] | ((unsigned)q[1] << 16), (unsigned)q[2] | ((unsigned)q[3] << 16));
-    r.x = __uint_as_float(w.x << 16); r.y = __uint_as_float(w.x & 0xffff0000u);
-    r.z = __uint_as_float(w.y << 16); r.w = __uint_as_float(w.y & 0xffff0000u);
+    const RowBf4 w = *(const RowBf4*)((const uint16_t*)p + off);
+    r.x = __uint_as_float(w.lo << 16); r.y = __uint_as_float(w.lo & 0xffff0000u);
+    r.z = __uint_as_float(w.hi << 16); r.w = __uint_as_float(w.hi & 0xffff0000u);
   } else {
-    const float* q = (const float*)p + off;
-    if (al == 0) r = *(const f4*)q;
-    else if (al == 1) {
-      const float2 a = *(const float2*)q, b = *(const float2*)(q + 2);
-      r = (f4){a.x, a.y, b.x, b.y};
-    } else r = (f4){q[0], q[1], q[2], q[3]};
+    const RowF4 w = *(const RowF4*)((const float*)p + off);
+    r = (f4){w.x, w.y, w.z, w.w};
   }
+  if (!ok) r = (f4){0.0f, 0.0f, 0.0f, 0.0f};
   return r;
 }
 template <bool BF>
-__device__ __forceinline__ void st4(void* p, long off, f4 v, int al) {
+__device__ __forceinline__ void st4(void* p, long off, f4 v, int /*al*/) {
   if (BF) {
-    uint16_t* q = (uint16_t*)p + off;
-    const unsigned lo = pack_bf16(v.x, v.y), hi = pack_bf16(v.z, v.w);
-    if (al == 0) *(uint2*)q = make_uint2(lo, hi);
-    else if (al == 1) { *(unsigned*)q = lo; *(unsigned*)(q + 2) = hi; }
-    else { q[0] = (uint16_t)lo; q[1] = (uint16_t)(lo >> 16); q[2] = (uint16_t)hi; q[3] = (uint16_t)(hi >> 16); }
+    RowBf4 w;
+    w.lo = pack_bf16(v.x, v.y); w.hi = pack_bf16(v.z, v.w);
+    *(RowBf4*)((uint16_t*)p + off) = w;
   } else {
-    float* q = (float*)p + off;
-    if (al == 0) *(f4*)q = v;
-    else if (al == 1) { *(float2*)q = make_float2(v.x, v.y); *(float2*)(q + 2) = make_float2(v.z, v.w); }
-    else { q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w; }
+    RowF4 w;
+    w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+    *(RowF4*)((float*)p + off) = w;
   }
 }
 // alignment class of rows starting at q with `stride` elements between them
@@ -97,6 +96,18 @@ __device__ __forceinline__ int al_of(const void* q, long stride, bool bf) {
   const uintptr_t a = (uintptr_t)q | ((uintptr_t)(stride < 0 ? -stride : stride) * (bf ? 2 : 4));
   const uintptr_t full = bf ? 7 : 15;
   return (a & full) == 0 ? 0 : ((a & (full >> 1)) == 0 ? 1 : 2);
+}
+// The lane's norm weights (fp32 or bf16 by `wdt`), zero for absent vectors: one wide load each, and one branch on
+// the dtype around all of them (a branch per load would make each wait for the previous one)
+template <int NV>
+__device__ __forceinline__ void ldw(const void* w, int lane, int nvec, int wdt, f4 (&out)[NV]) {
+  if (wdt) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) out[v] = ld4<true>(w, 4 * (lane + 64 * v), lane + 64 * v < nvec, 0);
+  } else {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) out[v] = ld4<false>(w, 4 * (lane + 64 * v), lane + 64 * v < nvec, 0);
+  }
 }
 __device__ __forceinline__ f4 silu4(f4 z, f4& sg) {
   f4 g;
@@ -112,17 +123,24 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
   if (row >= p.rows) return;
   const int nvec = p.ncols >> 2;
   const int ax = al_of(p.x, p.xs, BF), az = al_of(p.z, p.zs, BF), ay = al_of(p.y, p.ys, BF);
-  f4 x[NV], gate[NV];
-  float ss = 0.0f;
+  // all loads of the row first (x, z, the weights), nothing between them: one memory round trip per row
+  const void* zp = p.z ? p.z : p.x;  // without a gate the second load repeats the first and is not used
+  const long zs = p.z ? p.zs : p.xs;
+  f4 x[NV], gate[NV], wv[NV];
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     const int vi = lane + 64 * v;
     const bool ok = vi < nvec;
     x[v] = ld4<BF>(p.x, row * p.xs + 4 * vi, ok, ax);
-    gate[v] = (f4){1.0f, 1.0f, 1.0f, 1.0f};
+    gate[v] = ld4<BF>(zp, row * zs + 4 * vi, ok, az);
+  }
+  ldw<NV>(p.w, lane, nvec, p.wdt, wv);
+  float ss = 0.0f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
     if (p.z) {
       f4 sg;
-      gate[v] = silu4(ld4<BF>(p.z, row * p.zs + 4 * vi, ok, az), sg);
+      gate[v] = silu4(gate[v], sg);
       if (!p.nbg) x[v] *= gate[v];
     }
     ss += (x[v].x * x[v].x + x[v].y * x[v].y) + (x[v].z * x[v].z + x[v].w * x[v].w);
@@ -134,10 +152,7 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
   for (int v = 0; v < NV; ++v) {
     const int vi = lane + 64 * v;
     if (vi < nvec) {
-      f4 w;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] = ldv(p.w, 4 * vi + i, p.wdt);
-      f4 y = x[v] * rstd * w;
+      f4 y = x[v] * rstd * wv[v];
       if (p.z && p.nbg) y *= gate[v];
       st4<BF>(p.y, row * p.ys + 4 * vi, y, ay);
     }
@@ -152,30 +167,37 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd_fast(NormP p) {
   const int adx = al_of(p.dx, p.dxs, BF), adz = al_of(p.dz, p.dzs, BF);
   f4 w[NV], dwacc[NV];
 #pragma unroll
-  for (int v = 0; v < NV; ++v) {
-    const int vi = lane + 64 * v;
-    dwacc[v] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
-    w[v] = dwacc[v];
-    if (vi < nvec) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[v][i] = ldv(p.w, 4 * vi + i, p.wdt);
-    }
-  }
-  for (long row = blockIdx.x; row < p.rows; row += p.nblocks) {
-    const float rstd = p.rstd[row];
-    f4 xo[NV], dyo[NV], z[NV], sg[NV], gate[NV];
-    float c1 = 0.0f;
+  for (int v = 0; v < NV; ++v) dwacc[v] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+  ldw<NV>(p.w, lane, nvec, p.wdt, w);
+  // The loads of the next row are requested before the current row is worked on (x, dy, z and rstd back to back,
+  // nothing between them), so that a row costs no memory round trip of its own.
+  const void* zp = p.z ? p.z : p.x;  // without a gate the third load repeats the first and is not used
+  const long zs = p.z ? p.zs : p.xs;
+  f4 xn[NV], dyn[NV], zn[NV];
+  float rstd_n = 0.0f;
+  auto fetch = [&](long row) {
+    rstd_n = p.rstd[row];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
       const int vi = lane + 64 * v;
       const bool ok = vi < nvec;
-      xo[v] = ld4<BF>(p.x, row * p.xs + 4 * vi, ok, ax);
-      dyo[v] = ld4<BF>(p.dy, row * p.dys + 4 * vi, ok, ady);
+      xn[v] = ld4<BF>(p.x, row * p.xs + 4 * vi, ok, ax);
+      dyn[v] = ld4<BF>(p.dy, row * p.dys + 4 * vi, ok, ady);
+      zn[v] = ld4<BF>(zp, row * zs + 4 * vi, ok, az);
+    }
+  };
+  if ((long)blockIdx.x < p.rows) fetch(blockIdx.x);
+  for (long row = blockIdx.x; row < p.rows; row += p.nblocks) {
+    const float rstd = rstd_n;
+    f4 xo[NV], dyo[NV], z[NV], sg[NV], gate[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) { xo[v] = xn[v]; dyo[v] = dyn[v]; z[v] = zn[v]; }
+    if (row + p.nblocks < p.rows) fetch(row + p.nblocks);
+    float c1 = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
       gate[v] = (f4){1.0f, 1.0f, 1.0f, 1.0f};
-      if (p.z) {
-        z[v] = ld4<BF>(p.z, row * p.zs + 4 * vi, ok, az);
-        gate[v] = silu4(z[v], sg[v]);
-      }
+      if (p.z) gate[v] = silu4(z[v], sg[v]);
       const f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
       const f4 d = (p.z && p.nbg) ? dyo[v] * gate[v] : dyo[v];
       const f4 t = vv * rstd * d * w[v];
