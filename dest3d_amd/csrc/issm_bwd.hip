@@ -683,11 +683,12 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        mf[kb][j] = 0.0f;
-        if (kb >= wave) mf[kb][j] = mcol[(16 * kb + j) * CS];
-        if (kb == wave && cm > 4 * g4 + j) mf[kb][j] = 0.0f;
-      }
+      for (int j = 0; j < 4; ++j) mf[kb][j] = mcol[(16 * max(kb, wave) + j) * CS];  // no branch between the loads
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (kb < wave || (kb == wave && cm > 4 * g4 + j)) mf[kb][j] = 0.0f;
   }
   {
     float dv[CS * PT * 16 / NTHREADS];
@@ -751,12 +752,13 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
       odx[r] = (ok && tdx.ptr) ? pr * (int)tdx.s1 + pp : -1;
     }
     gload<IOB, 4>(tx.ptr, (long)u.b * tx.s0 + (long)u.h * tx.s2, ox, xv);
+    float dcoef = 0.0f;  // skip coefficient of the lane's column, read once
+    if (p.D) dcoef = (p.flags & F_D_HDIM) ? p.D[u.h * p.P + min(pt * 16 + cm, p.P - 1)] : p.D[u.h];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm;
       const float dyv = s.dys[l * LDPT + pp];
-      v[r] = acc[pt][r];
-      if (p.D) v[r] += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + (pp < p.P ? pp : 0)] : p.D[u.h]) * dyv;
+      v[r] = fmaf(dcoef, dyv, acc[pt][r]);
       prod[l * LDN + pp] = dyv * xv[r];
     }
     gstore<IOB, 4>(const_cast<void*>(tdx.ptr), (long)u.b * tdx.s0 + (long)u.h * tdx.s2, odx, v);

@@ -717,13 +717,21 @@ __device__ __forceinline__ void pn_load(const KP& p, const float* __restrict__ s
   for (int i = 0; i < R::CNT; ++i) {
     const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
     const bool ok = e < R::TOT && pp < p.P;
-    const float* q = src + (long)pp * p.N + n0 + c4;
+    const long o = (long)pp * p.N + n0 + c4;
+    // absent rows / columns read the slab's first elements and count as zero: a conditional load would become a
+    // branch, and a branch per load makes each wait for the one before
     if (vec) {
-      r.v[i] = (ok && n0 + c4 < p.N) ? *(const f4*)q : (f4){0, 0, 0, 0};
+      const bool in = ok && n0 + c4 < p.N;
+      const f4 w = *(const f4*)(src + (in ? o : 0));
+      r.v[i] = in ? w : (f4){0, 0, 0, 0};
     } else {
       f4 w;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = (ok && n0 + c4 + j < p.N) ? q[j] : 0.0f;
+      for (int j = 0; j < 4; ++j) {
+        const bool in = ok && n0 + c4 + j < p.N;
+        const float t = src[in ? o + j : 0];
+        w[j] = in ? t : 0.0f;
+      }
       r.v[i] = w;
     }
   }

@@ -383,15 +383,12 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   {
     const float* mrow = cabt + sq_off(p, u.bt, u.c, u.h) + (wave * 16 + cm) * CS + 4 * g4;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      mf[kb] = (f4){0, 0, 0, 0};
-      if (kb <= wave) mf[kb] = *(const f4*)(mrow + 16 * kb);
-      if (kb == wave) {
+    for (int kb = 0; kb < 4; ++kb) mf[kb] = *(const f4*)(mrow + 16 * min(kb, wave));  // no branch between the loads
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (4 * g4 + j > cm) mf[kb][j] = 0.0f;
-      }
-    }
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (kb > wave || (kb == wave && 4 * g4 + j > cm)) mf[kb][j] = 0.0f;
   }
   {
     float xv[CS * PT * 16 / NTHREADS];
@@ -448,14 +445,17 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
   for (int pt = 0; pt < PT; ++pt) {
     int off[4];
     float v[4];
+    // the skip coefficient of the lane's column, read once and without a lane-dependent branch (absent columns read
+    // the head's last one; their results are not stored)
+    float dcoef = 0.0f;
+    if (p.D) dcoef = (p.flags & F_D_HDIM) ? p.D[u.h * p.P + min(pt * 16 + cm, p.P - 1)] : p.D[u.h];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm;
       const int tt = u.c * CS + l;
       const bool ok = tt < p.L && pp < p.P;
       const int pr = ok ? phys_row(p, u.dir, tt) : 0;
-      v[r] = acc[pt][r];
-      if (p.D && ok) v[r] += ((p.flags & F_D_HDIM) ? p.D[u.h * p.P + pp] : p.D[u.h]) * s.xs[l * LDPT + pp];
+      v[r] = fmaf(dcoef, s.xs[l * LDPT + pp], acc[pt][r]);
       if (tz.ptr && ok) {
         if (out_x) out_x[(((long)u.bt * p.L + pr) * p.H + u.h) * p.P + pp] = v[r];
         const float zz = ldv(tz.ptr, (long)u.b * tz.s0 + (long)pr * tz.s1 + (long)u.h * tz.s2 + pp, p.io_dt);
