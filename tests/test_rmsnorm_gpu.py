@@ -54,3 +54,32 @@ def test_rmsnorm_strided_rows_and_import_shim():
     y = m(x, z)
     yr = R.gated_rmsnorm_ref(x.cpu(), m.weight.detach().cpu(), z=z.cpu(), eps=1e-5, norm_before_gate=False)
     _check("y", y, yr, FWD32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_rows_at_odd_element_offsets(dtype):
+    """Rows that start at odd element offsets of a wider row with an odd stride (2-byte aligned in bf16, 4-byte in
+    fp32): the 8 / 16-byte accesses of the fast path promise element alignment only.  Forward and backward."""
+    from dest3d_amd import RMSNorm
+    _say(f"rmsnorm rows at odd offsets, stride 601, {dtype}")
+    g = torch.Generator().manual_seed(3)
+    big = torch.randn(40, 601, generator=g).to(dtype)
+    w = torch.randn(288, generator=g) * 0.5 + 1.0
+    dy = torch.randn(40, 288, generator=g).to(dtype)
+    xs, zs = slice(1, 289), slice(301, 589)
+    ins = [big[:, xs].double().clone().requires_grad_(), w.double().clone().requires_grad_(),
+           big[:, zs].double().clone().requires_grad_()]
+    yr = R.gated_rmsnorm_ref(ins[0], ins[1], z=ins[2], eps=1e-5, norm_before_gate=False)
+    (yr * dy.double()).sum().backward()
+    m = RMSNorm(288, eps=1e-5, norm_before_gate=False, device="cuda")
+    with torch.no_grad():
+        m.weight.copy_(w)
+    bg = big.cuda().requires_grad_()
+    y = m(bg[:, xs], bg[:, zs])
+    (y.float() * dy.cuda().float()).sum().backward()
+    torch.cuda.synchronize()
+    ft, bt = (FWD32, BWD32) if dtype == torch.float32 else (FWD16, BWD16)
+    _check("y", y, yr, ft)
+    _check("dx", bg.grad[:, xs], ins[0].grad, bt)
+    _check("dz", bg.grad[:, zs], ins[2].grad, bt)
+    _check("dw", m.weight.grad, ins[1].grad, bt)
