@@ -362,15 +362,18 @@ __device__ __forceinline__ void bwd_mid_level(const float (&cs)[16], const float
       op[k] = (up ? Cv[k] : Bd[k]) * e;
     }
   }
+  // all 16 dM values first, then the products: read one by one, each read's LDS latency would sit in front of its
+  // matrix instruction (two waves per SIMD do not hide it)
+  float av[16];
+#pragma unroll
+  for (int I = 0; I < 4; ++I)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) av[4 * I + jj] = dms[I * (16 * LDC + 16) + a_base + jj * a_step];
 #pragma unroll
   for (int I = 0; I < 4; ++I) {
-    const float* ap = dms + I * (16 * LDC + 16) + a_base;
     f4 acc = {0, 0, 0, 0};
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const float a = ap[jj * a_step];
-      acc = mfma4(nz ? a : 0.0f, op[4 * I + jj], acc);
-    }
+    for (int jj = 0; jj < 4; ++jj) acc = mfma4(nz ? av[4 * I + jj] : 0.0f, op[4 * I + jj], acc);
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const float v = ee[4 * I + rr] * acc[rr];
