@@ -295,19 +295,22 @@ __device__ __forceinline__ void bwd_big_level(const float (&cs)[16], const float
     f4 acc = {0, 0, 0, 0};
     if (LV == 5) {
       if (I >= 2) {  // F: rows of tiles 2,3 gather from the lower rows s in tiles 0,1
+        const f4 av0 = *(const f4*)(dms + (I * 16 + cm) * LDC + 4 * g4);
+        const f4 av1 = *(const f4*)(dms + (I * 16 + cm) * LDC + 16 + 4 * g4);
 #pragma unroll
-        for (int J = 0; J < 2; ++J) {
-          const f4 av = *(const f4*)(dms + (I * 16 + cm) * LDC + J * 16 + 4 * g4);
+        for (int j = 0; j < 4; ++j) acc = mfma4(av0[j], op[j], acc);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc = mfma4(av[j], op[4 * J + j], acc);
-        }
-      } else {  // G: rows of tiles 0,1 gather from the upper rows l in tiles 2,3
+        for (int j = 0; j < 4; ++j) acc = mfma4(av1[j], op[4 + j], acc);
+      } else {  // G: rows of tiles 0,1 gather from the upper rows l in tiles 2,3 (all eight reads first)
+        float a8[8];
 #pragma unroll
-        for (int J = 2; J < 4; ++J) {
-          const float* ap = dms + (J * 16 + 4 * g4) * LDC + I * 16 + cm;
+        for (int J = 2; J < 4; ++J)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc = mfma4(ap[j * LDC], op[4 * J + j], acc);
-        }
+          for (int j = 0; j < 4; ++j) a8[4 * (J - 2) + j] = dms[(J * 16 + 4 * g4 + j) * LDC + I * 16 + cm];
+#pragma unroll
+        for (int J = 2; J < 4; ++J)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc = mfma4(a8[4 * (J - 2) + j], op[4 * J + j], acc);
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
