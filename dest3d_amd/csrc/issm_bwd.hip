@@ -600,20 +600,35 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     }
     dcs[15] += gl;
     {
+      // suffix sums up the 64 rows; the cross-lane steps of the four tiles are issued together (see lane_prep)
+      float c[4], v[4], t[4];
+#pragma unroll
+      for (int J = 3; J >= 0; --J) {
+        float a = 0.0f;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          a += dcs[4 * J + j];
+          dcs[4 * J + j] = a;
+        }
+        c[J] = a;
+      }
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl_down(c[J], 16, 64);
+#pragma unroll
+      for (int J = 0; J < 4; ++J) v[J] = g4 <= 2 ? c[J] + t[J] : c[J];
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl_down(v[J], 32, 64);
+#pragma unroll
+      for (int J = 0; J < 4; ++J) v[J] = g4 <= 1 ? v[J] + t[J] : v[J];  // inclusive from the last lane group down
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl(v[J], cm, 64);           // tile totals
       float carry = 0.0f;  // sum over all rows after the current tile
 #pragma unroll
       for (int J = 3; J >= 0; --J) {
-        float c = 0.0f;
-#pragma unroll
-        for (int j = 3; j >= 0; --j) {
-          c += dcs[4 * J + j];
-          dcs[4 * J + j] = c;
-        }
-        const float incl = scan_g_incl_rev(c, g4);
-        const float add = carry + (incl - c);
+        const float add = carry + (v[J] - c[J]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) dcs[4 * J + j] += add;
-        carry += __shfl(incl, cm, 64);
+        carry += t[J];
       }
     }
     float sumA = 0.0f, sumB = 0.0f;

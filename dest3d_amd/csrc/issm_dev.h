@@ -579,20 +579,38 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
     for (int k = 0; k < 16; ++k)
       if (!(vn && lane_row(k, g4) < rm.nvalid)) dtp[k] = 0.0f;
   }
+  // Running sum down the 64 rows: in the lane over its four rows of each tile, then across the four lane groups
+  // of a tile, then across the tiles.  The cross-lane steps of the four tiles do not depend on each other, so each
+  // step is issued for all four before any result is used (a cross-lane fetch goes through the LDS pipe: taken tile
+  // by tile, twelve latencies would line up instead of three).  Same operations in the same order as tile by tile.
+  float c[4], v[4], t[4];
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    float a = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a += dtp[4 * J + j] * A2;
+      cs[4 * J + j] = a;
+    }
+    c[J] = a;
+  }
+#pragma unroll
+  for (int J = 0; J < 4; ++J) t[J] = __shfl_up(c[J], 16, 64);
+#pragma unroll
+  for (int J = 0; J < 4; ++J) v[J] = g4 >= 1 ? c[J] + t[J] : c[J];
+#pragma unroll
+  for (int J = 0; J < 4; ++J) t[J] = __shfl_up(v[J], 32, 64);
+#pragma unroll
+  for (int J = 0; J < 4; ++J) v[J] = g4 >= 2 ? v[J] + t[J] : v[J];  // inclusive over the lane groups
+#pragma unroll
+  for (int J = 0; J < 4; ++J) t[J] = __shfl(v[J], cm + 48, 64);      // tile totals
   float carry = 0.0f;
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    float c = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      c += dtp[4 * J + j] * A2;
-      cs[4 * J + j] = c;
-    }
-    const float incl = scan_g_incl(c, g4);
-    const float add = carry + (incl - c);
+    const float add = carry + (v[J] - c[J]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) cs[4 * J + j] += add;
-    carry += __shfl(incl, cm + 48, 64);
+    carry += t[J];
   }
   return carry;
 }
