@@ -278,9 +278,12 @@ __device__ __forceinline__ void bwd_big_level(const float (&cs)[16], const float
                                               const float* __restrict__ dms, float (&e1)[16], float (&x2)[16], int cm,
                                               int g4) {
   float op[16], ee[16];
+  // reference rows: one cross-lane fetch (level 32) or two (level 16), before anything waits for them
+  const float ref_a = __shfl(LV == 4 ? cs[3] : cs[7], cm + 48, 64);
+  const float ref_b = LV == 4 ? __shfl(cs[11], cm + 48, 64) : ref_a;
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    const float ref = LV == 4 ? __shfl(cs[4 * (J & 2) + 3], cm + 48, 64) : __shfl(cs[7], cm + 48, 64);
+    const float ref = (J & 2) ? ref_b : ref_a;
     const bool upper = LV == 4 ? (J & 1) : (J & 2);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -352,10 +355,13 @@ __device__ __forceinline__ void bwd_mid_level(const float (&cs)[16], const float
   const bool nz = LV == 2 ? (g4 == (cg ^ 1)) : ((g4 >> 1) != (cg >> 1));
   const int a_base = iup ? cm * LDC + 4 * g4 : 4 * g4 * LDC + cm;  // dM[i][kk] (i upper) or dM[kk][i] (i lower)
   const int a_step = iup ? 1 : LDC;
-  float op[16], ee[16];
+  float op[16], ee[16], refs[4];
+#pragma unroll
+  for (int J = 0; J < 4; ++J)  // the four cross-lane fetches together
+    refs[J] = LV == 2 ? __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64) : __shfl(cs[4 * J + 3], cm + 16, 64);
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    const float ref = LV == 2 ? __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64) : __shfl(cs[4 * J + 3], cm + 16, 64);
+    const float ref = refs[J];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
