@@ -27,7 +27,7 @@ def _inputs(B, nP, nQ, seed, angles):
 # the table gradient scatters with LDS atomics below 65536 (point, box) pairs and sorts by window above: both sizes
 CASES = [(2, 37, 256, False, (10, 10, 10)), (1, 5, 300, True, (10, 10, 10)), (2, 64, 19, True, (4, 6, 7)),
          (1, 1, 1, False, (10, 10, 10)), (2, 160, 256, False, (10, 10, 10)), (1, 230, 300, True, (10, 10, 10)),
-         (1, 1100, 64, True, (4, 6, 7))]
+         (1, 1100, 64, True, (4, 6, 7)), (1, 1500, 43, True, (10, 10, 10))]   # two point segments, ragged box group
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_P%d_Q%d_ang%d_%dx%dx%d" % (*c[:3], int(c[3]), *c[4]))
