@@ -27,7 +27,7 @@ EXPORTS = [
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
     "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
-    "issm_hilbert_codes",
+    "issm_hilbert_codes", "issm_transpose_states",
     "issm_pn2_furthest_point_sampling", "issm_pn2_ball_query", "issm_pn2_group_points", "issm_pn2_group_points_grad",
     "issm_pn2_gather_points", "issm_pn2_gather_points_grad", "issm_pn2_three_nn", "issm_pn2_three_interpolate",
     "issm_pn2_three_interpolate_grad", "issm_pn2_group_points_grad_cl", "issm_pn2_three_interpolate_grad_cl",
@@ -124,6 +124,15 @@ class BoxDistArgs(C.Structure):
     ]
 
 
+class TransposeArgs(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("rows", C.c_int32), ("cols", C.c_int32),
+        ("in_dtype", C.c_int32), ("out_dtype", C.c_int32),
+        ("in0", C.c_void_p), ("in1", C.c_void_p), ("out", C.c_void_p),
+        ("alpha", C.c_float), ("stream", C.c_void_p),
+    ]
+
+
 class HilbertArgs(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("npoint", C.c_int32), ("bits", C.c_int32), ("order", C.c_int32 * 3),
@@ -166,6 +175,7 @@ def load() -> C.CDLL:
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
     lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
     lib.issm_hilbert_codes.argtypes = [P(HilbertArgs)]
+    lib.issm_transpose_states.argtypes = [P(TransposeArgs)]
     i32, f32 = C.c_int32, C.c_float
     lib.issm_pn2_furthest_point_sampling.argtypes = [i32, i32, i32, vp, vp, vp, vp]
     lib.issm_pn2_ball_query.argtypes = [i32, i32, i32, f32, i32, vp, vp, vp, vp]

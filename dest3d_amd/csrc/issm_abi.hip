@@ -26,6 +26,14 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
 int launch_hilbert_codes(const HilbertP& p, hipStream_t st);
+struct TrP {
+  int B, R, C, in_dt, out_dt;
+  const void* in0;
+  const void* in1;
+  void* out;
+  float alpha;
+};
+int launch_transpose_states(const TrP& p, hipStream_t st);
 int launch_fps(int b, int n, int npoint, const float* xyz, float* temp, int* idxs, hipStream_t st);
 int launch_ball_query(int b, int n, int m, float radius, int nsample, const float* new_xyz, const float* xyz, int* idx,
                       hipStream_t st);
@@ -563,6 +571,20 @@ int issm_box_dist_bwd(const issm_box_dist_args* a) {
   if (rc) return rc;
   if (p.nwg_bwd == 0) return ISSM_OK;
   return launched(launch_box_dist_bwd(p, (hipStream_t)a->stream), "box_dist_bwd");
+}
+
+int issm_transpose_states(const issm_transpose_args* a) {
+  if (!a) return fail(ISSM_E_NULL, "transpose: args is NULL");
+  if (a->batch < 0 || a->rows < 0 || a->cols < 0) return fail(ISSM_E_SHAPE, "transpose: bad shape");
+  if ((a->in_dtype != ISSM_F32 && a->in_dtype != ISSM_BF16) || (a->out_dtype != ISSM_F32 && a->out_dtype != ISSM_BF16))
+    return fail(ISSM_E_DTYPE, "transpose: dtypes %d -> %d", a->in_dtype, a->out_dtype);
+  if (a->batch == 0 || a->rows == 0 || a->cols == 0) return ISSM_OK;
+  if (!a->in0 || !a->out) return fail(ISSM_E_NULL, "transpose: in0/out is NULL");
+  if (a->batch > 65535 || (a->rows + 63) / 64 > 65535) return fail(ISSM_E_SHAPE, "transpose: batch / rows too large for one launch");
+  TrP p;
+  p.B = a->batch; p.R = a->rows; p.C = a->cols; p.in_dt = a->in_dtype; p.out_dt = a->out_dtype;
+  p.in0 = a->in0; p.in1 = a->in1; p.out = a->out; p.alpha = a->alpha;
+  return launched(launch_transpose_states(p, (hipStream_t)a->stream), "transpose_states");
 }
 
 int issm_hilbert_codes(const issm_hilbert_args* a) {

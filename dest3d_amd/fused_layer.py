@@ -25,6 +25,25 @@ def _kdt(t):
     return t.dtype if t.dtype in (torch.float32, torch.bfloat16) else torch.float32
 
 
+def _transpose_states(lib, in0, in1, alpha, out_dtype):
+    """(B, R, C) -> (B, C, R): alpha * (in0 + in1) in `out_dtype`; in1 may be None (issm_transpose_states)."""
+    if in0.dtype not in (torch.float32, torch.bfloat16):
+        in0 = in0.float()
+        in1 = None if in1 is None else in1.float()
+    in0 = in0.contiguous()
+    in1 = None if in1 is None else in1.to(in0.dtype).contiguous()
+    Bsz, R, Cn = in0.shape
+    out = torch.empty((Bsz, Cn, R), dtype=out_dtype, device=in0.device)
+    a = L.TransposeArgs()
+    a.batch, a.rows, a.cols = Bsz, R, Cn
+    a.in_dtype, a.out_dtype = L.dtype_code(in0.dtype), L.dtype_code(out_dtype)
+    a.in0, a.in1, a.out = in0.data_ptr(), None if in1 is None else in1.data_ptr(), out.data_ptr()
+    a.alpha = alpha
+    a.stream = L.current_stream_ptr(in0.device)
+    L.check(lib.issm_transpose_states(C.byref(a)), "issm_transpose_states")
+    return out
+
+
 class FusedScanCoreFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, zxbcdt, h0_lin, dist, weights, conv_w_f, conv_b_f, conv_w_b, conv_b_b, dt_w, bc_w, dt_bias, A_log, D,
@@ -79,7 +98,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             # 3. the bidirectional scan, queries as initial state
             A1 = torch.exp(A_log32).neg_()
             A = A1[:, None].expand(H, K)
-            h0 = h0_lin.detach().reshape(Bsz, K, H, P).permute(0, 2, 3, 1)
+            h0 = _transpose_states(lib, h0_lin.detach().reshape(Bsz, K, di), None, 1.0, _kdt(h0_lin)).view(Bsz, H, P, K)
             prob = _Problem([x_f, x_b], dt, A, [bc[0], bc[2]], [bc[1], bc[3]], chunk_size, D.detach(), [None, None], None,
                             h0, None, wt is None, dt_limit)
             outs, finals, ws = _scan_fwd(prob, True)
@@ -96,8 +115,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             n = _ln._norm_args(key, z2, nw, eps, None, False)
             n.y, n.y_row_stride, n.rstd = key_n.data_ptr(), key_n.stride(0), rstd.data_ptr()
             L.check(lib.issm_gated_rmsnorm_fwd(C.byref(n)), "issm_gated_rmsnorm_fwd")
-            last = torch.lerp(finals[0].permute(0, 3, 1, 2), finals[1].permute(0, 3, 1, 2), 0.5,
-                              out=torch.empty((Bsz, K, H, P), dtype=finals[0].dtype, device=dev)).view(Bsz, K, di)
+            last = _transpose_states(lib, finals[0].view(Bsz, di, K), finals[1].view(Bsz, di, K), 0.5, _kdt(h0_lin))
         ctx.save_for_backward(xbc, pre, cw, d, W, wt, raw, key, z2, nw, rstd, A1)
         ctx.prob, ctx.ws = prob, ws
         ctx.meta = (Bsz, Ln, K, H, G, di, P, Cc, kdt, eps, st)
@@ -132,8 +150,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_gated_rmsnorm_bwd(C.byref(n)), "issm_gated_rmsnorm_bwd")
             # 3'. the scan: both directions receive the gradient of their sum, and half of the averaged final states'
             dyh = dkey.view(Bsz, Ln, H, P)
-            dfin = torch.mul(dlast.reshape(Bsz, K, H, P).permute(0, 2, 3, 1), 0.5,
-                             out=torch.empty((Bsz, H, P, K), dtype=torch.float32, device=dev))
+            dfin = _transpose_states(lib, dlast.reshape(Bsz, K, di), None, 0.5, torch.float32).view(Bsz, H, P, K)
             dxs, ddt, dA, dBs, dCs, dD, _, _, dh0 = _scan_bwd(prob, ctx.ws, [dyh, dyh], [dfin, dfin], want_dz=False)
             # 2'. parameter generation
             R0, R = H + 2 * G, H + 4 * G
@@ -170,7 +187,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             L.check(lib.issm_dwconv_silu_bwd(C.byref(a)), "issm_dwconv_silu_bwd")
             dzx[..., di + Cc:].copy_(d_dt_tok)
             dA_log = dA.sum(-1).mul_(A1)
-            dh0_lin = dh0.permute(0, 3, 1, 2).reshape(Bsz, K, di)
+            dh0_lin = _transpose_states(lib, dh0.reshape(Bsz, di, K), None, 1.0, hdt if hdt in (torch.float32, torch.bfloat16) else torch.float32)
             ddt_bias = dbias_sum[:H]
             # parameter gradients: one buffer, one conversion to the parameters' dtype when they share one
             grads = [dcw[0], dcb[0], dcw[1], dcb[1], dW[:H], dW[H:], ddt_bias, dA_log, dD, dnw]

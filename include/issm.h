@@ -317,6 +317,25 @@ int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);
 int issm_dwconv_silu_fwd(const issm_dwconv_args* args);
 int issm_dwconv_silu_bwd(const issm_dwconv_args* args);
 
+/* ---- queries <-> scan states -----------------------------------------------------------------
+ * The rearrangements around the scan in MultiHeadISSMScan.forward: queries become initial states
+ * ("b l (h hd) -> b h hd l", models/dest_module.py:537-538) and the two directions' final states become the query
+ * output ("(last + last_back) / 2", "b h p l -> b l (h p)", :575 and :582); the backward needs the same two the
+ * other way round.  One batched transpose with the sum, the scale and the dtype conversion folded in:
+ *   out[b][c][r] = alpha * (in0[b][r][c] + in1[b][r][c]),   in0 / in1 (B, R, C), out (B, C, R), all contiguous;
+ * in1 may be NULL.  in_dtype applies to in0 and in1, out_dtype to out (issm_dtype). */
+typedef struct issm_transpose_args {
+  int32_t batch, rows, cols;
+  int32_t in_dtype, out_dtype;
+  const void* in0;
+  const void* in1;
+  void* out;
+  float alpha;
+  void* stream;
+} issm_transpose_args;
+
+int issm_transpose_states(const issm_transpose_args* args);
+
 /* ---- box-to-point distance encoding and locality weight ----------------------------------
  * BoxDistFun.forward (models/dest_module.py:174-195) and ISSMDecoderLayer.local_weight (:240-249), the two
  * (B, L, K) fields computed right before MultiHeadISSMScan:

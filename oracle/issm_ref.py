@@ -95,11 +95,14 @@ def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
     else:
         h = initial_states.to(dtype)
     ys = []
+    # one unbind per tensor: its backward is a single stack, where indexing [:, t] in the loop would write a
+    # full-length zero tensor per step and make the backward quadratic in L
+    dts, Bs, Cs, xs = dtp.unbind(1), Bh.unbind(1), Ch.unbind(1), x_.unbind(1)
     for t in range(L):
-        decay = torch.exp(dtp[:, t] * A_[None])                       # (B,H,N)
-        inject = (dtp[:, t] * Bh[:, t])[:, :, None, :] * x_[:, t][..., None]
+        decay = torch.exp(dts[t] * A_[None])                          # (B,H,N)
+        inject = (dts[t] * Bs[t])[:, :, None, :] * xs[t][..., None]
         h = decay[:, :, None, :] * h + inject
-        ys.append(torch.einsum("bhpn,bhn->bhp", h, Ch[:, t]))
+        ys.append(torch.einsum("bhpn,bhn->bhp", h, Cs[t]))
     y = torch.stack(ys, dim=1)                                        # (B,L,H,P)
     if D is not None:
         D_ = D.to(dtype)
