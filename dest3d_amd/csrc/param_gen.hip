@@ -60,38 +60,74 @@ __device__ __forceinline__ void st1(void* p, long i, float v) {
   if (BF) ((uint16_t*)p)[i] = f_to_bf16(v); else ((float*)p)[i] = v;
 }
 
-// Forward: thread = (token, k).  W and the token's biases are uniform across the workgroup's lanes of a token.
-template <bool BF>
+// KV adjacent outputs of one row as one store (4 bytes for two bf16, 8 / 16 bytes for two / four floats).
+template <bool BF, int KV>
+__device__ __forceinline__ void stv(void* p, long i, const float (&v)[KV]) {
+  if constexpr (KV == 1) {
+    st1<BF>(p, i, v[0]);
+  } else if constexpr (BF) {
+    unsigned w[KV / 2];
+#pragma unroll
+    for (int j = 0; j < KV / 2; ++j) w[j] = (unsigned)f_to_bf16(v[2 * j]) | ((unsigned)f_to_bf16(v[2 * j + 1]) << 16);
+    unsigned* q = (unsigned*)((uint16_t*)p + i);
+#pragma unroll
+    for (int j = 0; j < KV / 2; ++j) q[j] = w[j];
+  } else {
+    float* q = (float*)p + i;
+#pragma unroll
+    for (int j = 0; j < KV / 2; ++j) *(float2*)(q + 2 * j) = make_float2(v[2 * j], v[2 * j + 1]);
+  }
+}
+
+// Forward: thread = (token, KV adjacent k) -- KV = 2 whenever K is even, so that every store instruction of a wave
+// covers 256 (bf16) or 512 bytes instead of 128 / 256.  W and the token's biases are uniform across the lanes of a
+// token: scalar operands.
+template <bool BF, int KV>
 __global__ __launch_bounds__(NTHREADS) void k_pgen_fwd(PGenP p) {
   const int R0 = p.H + 2 * p.G, R = R0 + (p.has_back ? 2 * p.G : 0);
-  const int kchunks = (p.K + NTHREADS - 1) / NTHREADS;
-  const long t = blockIdx.x / kchunks;
-  const int k = (blockIdx.x % kchunks) * NTHREADS + threadIdx.x;
-  if (k >= p.K) return;
-  float d[PG_M];
-  load_row16<BF>(p.dist, (t * p.K + k) * PG_M, d);
+  const int per_tok = (p.K + KV - 1) / KV;  // threads per token
+  const long gid = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  const long t = gid / per_tok;
+  const int k = (int)(gid % per_tok) * KV;
+  if (t >= p.tokens) return;
+  float d[KV][PG_M];
+#pragma unroll
+  for (int j = 0; j < KV; ++j) load_row16<BF>(p.dist, (t * p.K + k + j) * PG_M, d[j]);
+  float wk[KV];
+#pragma unroll
+  for (int j = 0; j < KV; ++j) wk[j] = p.weights ? p.weights[t * p.K + k + j] : 1.0f;
   const float* bias = p.bias + t * R;
   for (int r = 0; r < R0; ++r) {
     const float* w = p.W + r * PG_M;  // uniform: scalar loads
-    float s = 0.0f;
+    float s[KV], v[KV];
 #pragma unroll
-    for (int m = 0; m < PG_M; ++m) s = fmaf(w[m], d[m], s);
+    for (int j = 0; j < KV; ++j) {
+      s[j] = 0.0f;
+#pragma unroll
+      for (int m = 0; m < PG_M; ++m) s[j] = fmaf(w[m], d[j][m], s[j]);
+      v[j] = s[j] + bias[r];
+    }
     if (r < p.H) {
-      float v = s + bias[r];
       if (p.weights) {  // uniform: dt = softplus(raw) * weight, raw kept for the backward
-        if (BF) v = bf16_to_f(f_to_bf16(v));  // the saved value is what the backward differentiates
-        st1<BF>(p.dt_raw, (t * p.H + r) * p.K + k, v);
-        v = softplus_(v) * p.weights[t * p.K + k];
+        if (BF) {
+#pragma unroll
+          for (int j = 0; j < KV; ++j) v[j] = bf16_to_f(f_to_bf16(v[j]));  // the saved value is what the backward differentiates
+        }
+        stv<BF, KV>(p.dt_raw, (t * p.H + r) * p.K + k, v);
+#pragma unroll
+        for (int j = 0; j < KV; ++j) v[j] = softplus_(v[j]) * wk[j];
       }
-      st1<BF>(p.dt, (t * p.H + r) * p.K + k, v);
-    } else if (r < p.H + p.G) {
-      const int g = r - p.H;
-      st1<BF>(p.Bm, (t * p.G + g) * p.K + k, s + bias[r]);
-      if (p.has_back) st1<BF>(p.Bb, (t * p.G + g) * p.K + k, s + bias[R0 + g]);
+      stv<BF, KV>(p.dt, (t * p.H + r) * p.K + k, v);
     } else {
-      const int g = r - p.H - p.G;
-      st1<BF>(p.Cm, (t * p.G + g) * p.K + k, s + bias[r]);
-      if (p.has_back) st1<BF>(p.Cb, (t * p.G + g) * p.K + k, s + bias[R0 + p.G + g]);
+      const bool isB = r < p.H + p.G;
+      const int g = isB ? r - p.H : r - p.H - p.G;
+      stv<BF, KV>(isB ? p.Bm : p.Cm, (t * p.G + g) * p.K + k, v);
+      if (p.has_back) {
+        const float bb = bias[R0 + (isB ? 0 : p.G) + g];
+#pragma unroll
+        for (int j = 0; j < KV; ++j) v[j] = s[j] + bb;
+        stv<BF, KV>(isB ? p.Bb : p.Cb, (t * p.G + g) * p.K + k, v);
+      }
     }
   }
 }
@@ -426,10 +462,21 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_dw(PGenP p) {
 int pgen_bwd_blocks(long tokens) { return (int)((tokens + PG_TOK - 1) / PG_TOK); }
 
 int launch_pgen_fwd(const PGenP& p, hipStream_t st) {
-  const long kchunks = (p.K + NTHREADS - 1) / NTHREADS;
-  const unsigned blocks = (unsigned)(p.tokens * kchunks);
-  if (p.dtype) hipLaunchKernelGGL(k_pgen_fwd<true>, dim3(blocks), dim3(NTHREADS), 0, st, p);
-  else hipLaunchKernelGGL(k_pgen_fwd<false>, dim3(blocks), dim3(NTHREADS), 0, st, p);
+  // pairs of outputs go out as one store: K even and every output 8-byte aligned
+  uintptr_t bits = 0;
+  for (const void* q : {(const void*)p.dt, (const void*)p.dt_raw, (const void*)p.Bm, (const void*)p.Cm, (const void*)p.Bb,
+                        (const void*)p.Cb})
+    bits |= (uintptr_t)q;
+  const int kv = (p.K % 2 == 0 && (bits & 7) == 0) ? 2 : 1;
+  const long threads = p.tokens * ((p.K + kv - 1) / kv);
+  const unsigned blocks = (unsigned)((threads + NTHREADS - 1) / NTHREADS);
+  if (p.dtype) {
+    if (kv == 2) hipLaunchKernelGGL((k_pgen_fwd<true, 2>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    else hipLaunchKernelGGL((k_pgen_fwd<true, 1>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+  } else {
+    if (kv == 2) hipLaunchKernelGGL((k_pgen_fwd<false, 2>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+    else hipLaunchKernelGGL((k_pgen_fwd<false, 1>), dim3(blocks), dim3(NTHREADS), 0, st, p);
+  }
   return (int)hipGetLastError();
 }
 
