@@ -31,6 +31,8 @@ CASES = [
     (1, 33, 300, 2, 2, True, torch.float32),
     (2, 64, 256, 8, 1, True, torch.bfloat16),
     (1, 19, 77, 3, 1, False, torch.bfloat16),
+    (1, 11, 50, 3, 1, True, torch.bfloat16),     # K even, not a multiple of 4
+    (2, 6, 77, 2, 1, False, torch.float32),      # K odd
 ]
 
 
@@ -68,6 +70,8 @@ WCASES = [
     (1, 9, 100, 4, 2, False, torch.float32),
     (2, 33, 128, 8, 1, True, torch.bfloat16),
     (1, 7, 52, 3, 1, True, torch.bfloat16),
+    (1, 5, 50, 2, 1, True, torch.bfloat16),
+    (1, 4, 33, 2, 1, False, torch.float32),
 ]
 
 
