@@ -196,20 +196,41 @@ MEASURED_TRAFFIC_BYTES = {
 
 
 def stage_work(ndir):
-    """Algorithmic FLOPs (2*MAC; exps not counted) and bytes per launch of each kernel."""
-    B_, L_, H, P, N, cs = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "cs"))
+    """Algorithmic FLOPs (2*MAC; exps not counted) and algorithmic bytes (every operand read once, every result
+    written once, in the run's 4-byte types; dt counted once for both directions) per launch of each kernel."""
+    B_, L_, H, P, N, G, cs = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "G", "cs"))
     U = B_ * ndir * H * math.ceil(L_ / cs)
     tri = cs * (cs + 1) // 2
-    E_cs, E_st = U * P * N, B_ * ndir * H * P * N
+    E_cs, E_st = U * P * N, B_ * ndir * H * P * N          # chunk states; initial / final states
+    E_x, E_bc = ndir * B_ * L_ * H * P, ndir * B_ * L_ * G * N   # x / y / dy / dx; B, C and their gradients
+    E_dt, E_m, E_v = B_ * L_ * H * N, U * cs * cs, U * N   # dt / ddt; intra-chunk matrix M / dM; per-chunk vectors
     return {
-        "chunk_local": ("mfma", 2 * U * (cs * P * N + tri * N)),
-        "chunk_scan": ("mfma", 2 * U * (cs * P * N + tri * P)),
-        "bwd_dstates": ("mfma", 2 * U * (cs * P * N + tri * P)),
-        "bwd_chunk": ("mfma", 2 * U * (2 * cs * P * N + 2 * tri * N)),
-        "bwd_dx": ("mfma", 2 * U * (cs * P * N + tri * P)),
-        "state_passing_fwd": ("hbm", 4 * (2 * E_cs + U * N + 2 * E_st)),
-        "state_passing_bwd": ("hbm", 4 * (3 * E_cs + 2 * U * N + 2 * E_st)),
+        # reads dt, x, B, C; writes chunk-local end states S, M, the chunks' total decay
+        "chunk_local": (2 * U * (cs * P * N + tri * N), 4 * (E_dt + E_x + 2 * E_bc + E_cs + E_m + E_v)),
+        # reads dt, C, x, states H, M; writes y
+        "chunk_scan": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + E_x + E_cs + E_m + E_x)),
+        # reads dt, C, dy, x; writes dH, dM
+        "bwd_dstates": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + 2 * E_x + E_cs + E_m)),
+        # both launches: read dt, x, dy, B, C, H, dS, dM, g_last; write ddt, dB, dC, the dA / ddt_bias partials
+        "bwd_chunk": (2 * U * (2 * cs * P * N + 2 * tri * N),
+                      4 * (E_dt + 2 * E_x + 2 * E_bc + 2 * E_cs + E_m + E_v + E_dt + 2 * E_bc + 2 * E_v)),
+        # reads dt, B, dy, x, dS, M; writes dx
+        "bwd_dx": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + 2 * E_x + E_cs + E_m + E_x)),
+        "state_passing_fwd": (0, 4 * (2 * E_cs + U * N + 2 * E_st)),
+        "state_passing_bwd": (0, 4 * (3 * E_cs + 2 * U * N + 2 * E_st)),
     }
+
+
+def stage_bound(flops, nbytes, us):
+    """The roofline that bounds a stage is the one with the longer minimum time; returns (bound, achieved in the
+    bound's unit, fraction of its peak, {mfma fraction, hbm fraction})."""
+    t = us * 1e-6
+    f_mfma = flops / t / (PEAK_FP32_MFMA_TFLOPS * 1e12)
+    f_hbm = nbytes / t / (PEAK_HBM_GBS * 1e9)
+    both = {"mfma_frac": round(f_mfma, 4), "hbm_frac": round(f_hbm, 4)}
+    if f_mfma >= f_hbm:
+        return "mfma", flops / t / 1e12, f_mfma, both
+    return "hbm", nbytes / t / 1e9, f_hbm, both
 
 
 def cpu_baseline(torch):
@@ -452,21 +473,14 @@ def main():
     stages = run.stage_times()
     work = stage_work(2)
     dom = max((k for k in stages if k in work), key=lambda k: stages[k])
-    bound, amount = work[dom]
-    if bound == "mfma":
-        achieved = amount / (stages[dom] * 1e-6) / 1e12
-        roof = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None, "kernel": dom}
-    else:
-        achieved = amount / (stages[dom] * 1e-6) / 1e9
-        roof = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBS, "traffic": None, "kernel": dom}
+    bound, achieved, frac, _ = stage_bound(*work[dom], stages[dom])
+    roof = {"bound": bound, "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS if bound == "mfma" else PEAK_HBM_GBS,
+            "unit": "TFLOP/s" if bound == "mfma" else "GB/s", "frac": frac, "traffic": None, "kernel": dom}
     roof["traffic"] = args.traffic if args.traffic is not None else MEASURED_TRAFFIC_BYTES.get(dom)
     per_stage = {}
-    for k, (b, amt) in work.items():
-        rate = amt / (stages[k] * 1e-6)
-        per_stage[k] = {"us": round(stages[k], 2), "bound": b,
-                        "frac": round(rate / (PEAK_FP32_MFMA_TFLOPS * 1e12 if b == "mfma" else PEAK_HBM_GBS * 1e9), 4)}
+    for k, (fl, nb) in work.items():
+        b, _, fr, both = stage_bound(fl, nb, stages[k])
+        per_stage[k] = {"us": round(stages[k], 2), "bound": b, "frac": round(fr, 4), **both}
     variants = {}
     if not args.no_variants:
         variants["headline_as_hip_graph_replay"] = round(run.time_graph_replays(args.steps, 5), 2)
