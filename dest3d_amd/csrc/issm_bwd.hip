@@ -142,25 +142,28 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
 // Block = (bt, h, 64 state columns); thread (pg = tid >> 4, nq = tid & 15) carries rows
 // p = pg, pg+16, ... of 4 adjacent columns.  dstates[c] holds dH_c on entry and dS_c (gradient
 // of the chunk-local end state) on exit.  g_last[c][n] = sum_p dS_c[p,n] * H_{c+1}[p,n].
+template <int NQ>
 __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __restrict__ states,
                                                         const float* __restrict__ cs_last,
                                                         float* __restrict__ dstates, float* __restrict__ g_last,
                                                         float* __restrict__ dh0_dir) {
-  __shared__ float red[16 * 64];
-  const int nsl = (p.N + 63) / 64;
+  // NQ column quads per workgroup: NCOL columns, PGN row groups, a thread carries rows pg, pg + PGN, ...
+  constexpr int NCOL = NQ * 4, PGN = NTHREADS / NQ, KR = (MAXP + PGN - 1) / PGN;
+  __shared__ float red[PGN * NCOL];
+  const int nsl = (p.N + NCOL - 1) / NCOL;
   int bid = blockIdx.x;
   const int ns = bid % nsl;
   bid /= nsl;
   const int h = bid % p.H;
   const int bt = bid / p.H;
   const int b = bt / p.ndir, dir = bt % p.ndir;
-  const int tid = threadIdx.x, pg = tid >> 4, nq = tid & 15;
-  const int n = ns * 64 + nq * 4;
+  const int tid = threadIdx.x, pg = tid / NQ, nq = tid % NQ;
+  const int n = ns * NCOL + nq * 4;
   const bool vec = ((p.N & 3) == 0) && (n + 3 < p.N);
-  float carry[4][4];
+  float carry[KR][4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int pp = pg + 16 * k;
+  for (int k = 0; k < KR; ++k) {
+    const int pp = pg + PGN * k;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const bool v = pp < p.P && n + j < p.N && p.dfinal[dir];
@@ -168,12 +171,12 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
     }
   }
   // operands of one chunk: decay exponent, H_{c+1} and dH_c of the thread's rows
-  auto load_chunk = [&](int c, float (&dec)[4], float (&hn)[4][4], float (&dh)[4][4]) {
+  auto load_chunk = [&](int c, float (&dec)[4], float (&hn)[KR][4], float (&dh)[KR][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) dec[j] = n + j < p.N ? cs_last[vec_off(p, bt, c, h) + n + j] : 0.0f;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int pp = pg + 16 * k;
+    for (int k = 0; k < KR; ++k) {
+      const int pp = pg + PGN * k;
       const float* hp = states + st_off(p, bt, c + 1, h) + (long)pp * p.N + n;
       const float* dd = dstates + dst_off(p, bt, c, h) + (long)pp * p.N + n;
       if (vec && pp < p.P) {
@@ -192,18 +195,18 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
   };
   // The operands of the next two chunks are always in flight (the loads do not depend on the carry), so the
   // recurrence never waits for memory and enough bytes are outstanding to keep HBM busy.
-  float dec[4], hn[4][4], dh[4][4], dec_1[4], hn_1[4][4], dh_1[4][4];
+  float dec[4], hn[KR][4], dh[KR][4], dec_1[4], hn_1[KR][4], dh_1[KR][4];
   load_chunk(p.nc - 1, dec, hn, dh);
   if (p.nc > 1) load_chunk(p.nc - 2, dec_1, hn_1, dh_1);
   for (int c = p.nc - 1; c >= 0; --c) {
     float gp[4] = {0, 0, 0, 0};
-    float dec_n[4], hn_n[4][4], dh_n[4][4];
+    float dec_n[4], hn_n[KR][4], dh_n[KR][4];
     if (c > 1) load_chunk(c - 2, dec_n, hn_n, dh_n);
 #pragma unroll
     for (int j = 0; j < 4; ++j) dec[j] = __expf(dec[j]);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int pp = pg + 16 * k;
+    for (int k = 0; k < KR; ++k) {
+      const int pp = pg + PGN * k;
       float* dd = dstates + dst_off(p, bt, c, h) + (long)pp * p.N + n;
       if (vec && pp < p.P) {
         *(f4*)dd = (f4){carry[k][0], carry[k][1], carry[k][2], carry[k][3]};
@@ -219,19 +222,25 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) red[pg * 64 + nq * 4 + j] = gp[j];
+    for (int j = 0; j < 4; ++j) red[pg * NCOL + nq * 4 + j] = gp[j];
     __syncthreads();
     if (tid < 64) {
+      // 64 lanes over NCOL columns: a lane sums every (64 / NCOL)-th row group of its column, then the lanes of a
+      // column (NCOL apart) are added
+      constexpr int PARTS = 64 / NCOL;
+      const int col = tid % NCOL, part = tid / NCOL;
       float sum = 0.0f;
 #pragma unroll
-      for (int k = 0; k < 16; ++k) sum += red[k * 64 + tid];
-      if (ns * 64 + tid < p.N) g_last[vec_off(p, bt, c, h) + ns * 64 + tid] = sum;
+      for (int k = 0; k < PGN / PARTS; ++k) sum += red[(k * PARTS + part) * NCOL + col];
+#pragma unroll
+      for (int d = NCOL; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
+      if (part == 0 && ns * NCOL + col < p.N) g_last[vec_off(p, bt, c, h) + ns * NCOL + col] = sum;
     }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < 4; ++j) { dec[j] = dec_1[j]; dec_1[j] = dec_n[j]; }
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
+    for (int k = 0; k < KR; ++k)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         hn[k][j] = hn_1[k][j]; dh[k][j] = dh_1[k][j];
@@ -239,13 +248,103 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
       }
   }
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int pp = pg + 16 * k;
+  for (int k = 0; k < KR; ++k) {
+    const int pp = pg + PGN * k;
     if (pp >= p.P) continue;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (n + j < p.N) dh0_dir[((((long)dir * p.B + b) * p.H + h) * p.P + pp) * p.N + n + j] = carry[k][j];
   }
+}
+
+// The same recurrence for complete shapes -- N a multiple of the slice width, P exactly KM rows per thread -- with
+// no conditional access anywhere: every load of the loop is issued on every path, so the compiler can count the
+// loads still in flight and the prefetched operands of the next two chunks stay in flight across the barriers
+// (with loads inside branches it waits for all of them before each store, which exposes the full memory latency
+// once per chunk; few workgroups walking many chunks -- batch 2, 256 chunks -- then run at that pace).
+template <int NQ, int KM>
+__global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* __restrict__ states,
+                                                             const float* __restrict__ cs_last,
+                                                             float* __restrict__ dstates, float* __restrict__ g_last,
+                                                             float* __restrict__ dh0_dir) {
+  constexpr int NCOL = NQ * 4, PGN = NTHREADS / NQ;
+  __shared__ __align__(16) float red[PGN * NCOL];
+  const int nsl = p.N / NCOL;
+  int bid = blockIdx.x;
+  const int ns = bid % nsl;
+  bid /= nsl;
+  const int h = bid % p.H;
+  const int bt = bid / p.H;
+  const int b = bt / p.ndir, dir = bt % p.ndir;
+  const int tid = threadIdx.x, pg = tid / NQ, nq = tid % NQ;
+  const int n = ns * NCOL + nq * 4;
+  const long row = (long)pg * p.N + n, kstep = (long)PGN * p.N;  // the thread's first row; from row block to row block
+  const long cstep = (long)p.H * p.P * p.N, vstep = (long)p.H * p.N;  // from chunk to chunk
+  f4 carry[KM];
+#pragma unroll
+  for (int k = 0; k < KM; ++k) {
+    carry[k] = (f4){0, 0, 0, 0};
+    if (p.dfinal[dir]) carry[k] = *(const f4*)(p.dfinal[dir] + ((long)b * p.H + h) * p.P * p.N + row + k * kstep);
+  }
+  const float* hp = states + st_off(p, bt, p.nc, h) + row;       // H_{c+1}, c = nc - 1
+  float* dd = dstates + dst_off(p, bt, p.nc - 1, h) + row;       // dH_c in, dS_c out
+  const float* cl = cs_last + vec_off(p, bt, p.nc - 1, h) + n;
+  float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;
+  // operands of chunks c, c - 1 in registers, those of c - 2 requested at the top of step c (the last two steps
+  // request chunk 0 again: in range, unused)
+  f4 dec = *(const f4*)cl, dec_1 = *(const f4*)(cl - (p.nc > 1 ? vstep : 0));
+  f4 hn[KM], dh[KM], hn_1[KM], dh_1[KM];
+  {
+    const long back = p.nc > 1 ? cstep : 0;
+#pragma unroll
+    for (int k = 0; k < KM; ++k) {
+      hn[k] = *(const f4*)(hp + k * kstep);
+      dh[k] = *(const f4*)(dd + k * kstep);
+      hn_1[k] = *(const f4*)(hp - back + k * kstep);
+      dh_1[k] = *(const f4*)(dd - back + k * kstep);
+    }
+  }
+  for (int c = p.nc - 1; c >= 0; --c) {
+    const long back = (long)min(c, 2) * cstep, vback = (long)min(c, 2) * vstep;
+    f4 dec_n = *(const f4*)(cl - vback), hn_n[KM], dh_n[KM];
+#pragma unroll
+    for (int k = 0; k < KM; ++k) {
+      hn_n[k] = *(const f4*)(hp - back + k * kstep);
+      dh_n[k] = *(const f4*)(dd - back + k * kstep);
+    }
+    f4 gp = {0, 0, 0, 0}, e;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) e[j] = __expf(dec[j]);
+#pragma unroll
+    for (int k = 0; k < KM; ++k) {
+      *(f4*)(dd + k * kstep) = carry[k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        gp[j] += hn[k][j] * carry[k][j];
+        carry[k][j] = e[j] * carry[k][j] + dh[k][j];
+      }
+    }
+    *(f4*)(red + pg * NCOL + nq * 4) = gp;
+    __syncthreads();
+    if (tid < 64) {
+      constexpr int PARTS = 64 / NCOL;
+      const int col = tid % NCOL, part = tid / NCOL;
+      float sum = 0.0f;
+#pragma unroll
+      for (int k = 0; k < PGN / PARTS; ++k) sum += red[(k * PARTS + part) * NCOL + col];
+#pragma unroll
+      for (int d = NCOL; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
+      if (part == 0) gl[col] = sum;
+    }
+    __syncthreads();
+    dec = dec_1; dec_1 = dec_n;
+#pragma unroll
+    for (int k = 0; k < KM; ++k) { hn[k] = hn_1[k]; dh[k] = dh_1[k]; hn_1[k] = hn_n[k]; dh_1[k] = dh_n[k]; }
+    hp -= cstep; dd -= cstep; cl -= vstep; gl -= vstep;
+  }
+#pragma unroll
+  for (int k = 0; k < KM; ++k)
+    *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + row + k * kstep) = carry[k];
 }
 
 // -------------------------------------------------------------- chunk backward
@@ -898,8 +997,28 @@ int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* d
 
 int launch_state_bwd(const KP& p, const float* states, const float* cs_last, float* dstates, float* g_last,
                      float* dh0_dir, hipStream_t st) {
-  const int blocks = p.B * p.ndir * p.H * ((p.N + 63) / 64);
-  hipLaunchKernelGGL(k_state_bwd, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last, dstates, g_last, dh0_dir);
+  // One workgroup walks the chunks of its columns one after the other.  Complete shapes take the variant without
+  // conditional accesses; with few (batch, head) pairs narrower column slices put more workgroups on the chip.
+  const int wide = p.B * p.ndir * p.H * ((p.N + 63) / 64);
+#define ISSM_STATE_BWD_FULL(NQ_, KM_)                                                                                   \
+  hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
+                     states, cs_last, dstates, g_last, dh0_dir)
+  if (wide < 256 && p.N % 32 == 0 && (p.P == 32 || p.P == 64)) {
+    if (p.P == 32) ISSM_STATE_BWD_FULL(8, 1); else ISSM_STATE_BWD_FULL(8, 2);
+  } else if (p.N % 64 == 0 && p.P % 16 == 0) {
+    switch (p.P / 16) {
+      case 1: ISSM_STATE_BWD_FULL(16, 1); break;
+      case 2: ISSM_STATE_BWD_FULL(16, 2); break;
+      case 3: ISSM_STATE_BWD_FULL(16, 3); break;
+      default: ISSM_STATE_BWD_FULL(16, 4); break;
+    }
+  } else if (wide < 256) {
+    const int blocks = p.B * p.ndir * p.H * ((p.N + 15) / 16);
+    hipLaunchKernelGGL(k_state_bwd<4>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last, dstates, g_last, dh0_dir);
+  } else {
+    hipLaunchKernelGGL(k_state_bwd<16>, dim3(wide), dim3(NTHREADS), 0, st, p, states, cs_last, dstates, g_last, dh0_dir);
+  }
+#undef ISSM_STATE_BWD_FULL
   return (int)hipGetLastError();
 }
 

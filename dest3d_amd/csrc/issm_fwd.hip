@@ -279,6 +279,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 // One thread carries 4 adjacent state columns of one (bt, h, p) through all chunks.
 // Slot c of `states` holds S_c on entry and H_c (state at the start of chunk c) on exit;
 // slot nc receives the final state.
+// D: chunks of operands a thread keeps in flight (2 when the launch has plenty of threads; 8 when a few threads walk
+// many chunks, e.g. batch 2 x 256 chunks, where memory latency and not bandwidth sets the pace)
+template <int D>
 __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict__ states,
                                                         const float* __restrict__ cs_last) {
   const int nq = (p.N + 3) >> 2;
@@ -303,7 +306,33 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
   const long cstride = (long)p.H * p.P * p.N;
   float* sp = states + st_off(p, bt, 0, h) + (long)pp * p.N + n;
   const float* cl = cs_last + vec_off(p, bt, 0, h) + n;
-  if (full) {
+  if (full && D > 2) {
+    const long dstride = (long)p.H * p.N;
+    f4 t[D], d[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      const int ci = min(i, p.nc - 1);
+      t[i] = *(const f4*)(sp + ci * cstride);
+      d[i] = *(const f4*)(cl + ci * dstride);
+    }
+    for (int c0 = 0; c0 < p.nc; c0 += D) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        if (c0 + i < p.nc) {  // uniform
+          const f4 tt = t[i], dd = d[i];
+          if (c0 + i + D < p.nc) {  // uniform: the slot's next occupant, D chunks ahead
+            t[i] = *(const f4*)(sp + D * cstride);
+            d[i] = *(const f4*)(cl + D * dstride);
+          }
+          *(f4*)sp = (f4){st[0], st[1], st[2], st[3]};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) st[j] = __expf(dd[j]) * st[j] + tt[j];
+          sp += cstride;
+          cl += dstride;
+        }
+      }
+    }
+  } else if (full) {
     // S_c and the chunk decay of the next two chunks are always in flight: the loads do not depend on
     // the running state, only the store into the slot just read does
     const long dstride = (long)p.H * p.N;
@@ -486,7 +515,10 @@ int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, 
 int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream_t st) {
   const long total = (long)p.B * p.ndir * p.H * p.P * ((p.N + 3) / 4);
   const int blocks = (int)((total + NTHREADS - 1) / NTHREADS);
-  hipLaunchKernelGGL(k_state_fwd, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+  if (total < (1L << 17) && p.nc >= 16)
+    hipLaunchKernelGGL(k_state_fwd<8>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+  else
+    hipLaunchKernelGGL(k_state_fwd<2>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
   return (int)hipGetLastError();
 }
 
