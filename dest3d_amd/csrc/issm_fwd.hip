@@ -279,6 +279,71 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 // One thread carries 4 adjacent state columns of one (bt, h, p) through all chunks.
 // Slot c of `states` holds S_c on entry and H_c (state at the start of chunk c) on exit;
 // slot nc receives the final state.
+// The recurrence for N a multiple of 4, without any conditional access: thread = 4 adjacent columns of one state row,
+// the operands of the next D chunks always requested (near the end the last chunk again: in range, unused), so the
+// compiler can count the loads in flight and never waits for all of them; with loads inside branches it did, once
+// per chunk.  D = 8 when few threads walk many chunks (memory latency sets the pace there), otherwise 4.
+template <int D>
+__global__ __launch_bounds__(NTHREADS) void k_state_fwd_full(KP p, float* __restrict__ states,
+                                                             const float* __restrict__ cs_last) {
+  const int nq = p.N >> 2;
+  const long total = (long)p.B * p.ndir * p.H * p.P * nq;
+  const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
+  if (id >= total) return;
+  const int q = id % nq;
+  long r = id / nq;
+  const int pp = r % p.P;
+  r /= p.P;
+  const int h = r % p.H;
+  const int bt = r / p.H;
+  const int b = bt / p.ndir, dir = bt % p.ndir;
+  const int n = q * 4;
+  f4 st = {0, 0, 0, 0};
+  if (p.h0.ptr) {
+    const long o = (long)b * p.h0.s0 + (long)h * p.h0.s1 + (long)pp * p.h0.s2 + n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) st[j] = ldv(p.h0.ptr, o + j, p.h0_dt);
+  }
+  const long cstride = (long)p.H * p.P * p.N, dstride = (long)p.H * p.N;
+  float* sp = states + st_off(p, bt, 0, h) + (long)pp * p.N + n;
+  const float* cl = cs_last + vec_off(p, bt, 0, h) + n;
+  // chunk c lives in slot c % D; the loop is unrolled over the D slots so that none is ever moved (a register copy
+  // would have to wait for the load that fills it)
+  const float* sp0 = sp;
+  const float* cl0 = cl;
+  f4 t[D], d[D];
+#pragma unroll
+  for (int i = 0; i < D; ++i) {
+    const int ci = min(i, p.nc - 1);
+    t[i] = *(const f4*)(sp0 + ci * cstride);
+    d[i] = *(const f4*)(cl0 + ci * dstride);
+  }
+  int c = 0;
+  for (; c + D <= p.nc; c += D) {
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      const f4 tt = t[i], dd = d[i];
+      const int cn = min(c + i + D, p.nc - 1);
+      t[i] = *(const f4*)(sp0 + cn * cstride);
+      d[i] = *(const f4*)(cl0 + cn * dstride);
+      *(f4*)sp = st;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) st[j] = __expf(dd[j]) * st[j] + tt[j];
+      sp += cstride;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i)
+    if (c + i < p.nc) {  // uniform: the last nc % D chunks
+      *(f4*)sp = st;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) st[j] = __expf(d[i][j]) * st[j] + t[i][j];
+      sp += cstride;
+    }
+  *(f4*)sp = st;  // slot nc keeps the final state for the backward pass
+  if (p.final_states[dir]) *(f4*)(p.final_states[dir] + (((long)b * p.H + h) * p.P + pp) * p.N + n) = st;
+}
+
 // D: chunks of operands a thread keeps in flight (2 when the launch has plenty of threads; 8 when a few threads walk
 // many chunks, e.g. batch 2 x 256 chunks, where memory latency and not bandwidth sets the pace)
 template <int D>
@@ -515,7 +580,12 @@ int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, 
 int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream_t st) {
   const long total = (long)p.B * p.ndir * p.H * p.P * ((p.N + 3) / 4);
   const int blocks = (int)((total + NTHREADS - 1) / NTHREADS);
-  if (total < (1L << 17) && p.nc >= 16)
+  if ((p.N & 3) == 0) {
+    if (total < (1L << 17) && p.nc >= 16)
+      hipLaunchKernelGGL(k_state_fwd_full<8>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+    else
+      hipLaunchKernelGGL(k_state_fwd_full<4>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+  } else if (total < (1L << 17) && p.nc >= 16)
     hipLaunchKernelGGL(k_state_fwd<8>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
   else
     hipLaunchKernelGGL(k_state_fwd<2>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
