@@ -290,38 +290,33 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   float* dd = dstates + dst_off(p, bt, p.nc - 1, h) + row;       // dH_c in, dS_c out
   const float* cl = cs_last + vec_off(p, bt, p.nc - 1, h) + n;
   float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;
-  // operands of chunks c, c - 1 in registers, those of c - 2 requested at the top of step c (the last two steps
-  // request chunk 0 again: in range, unused)
-  f4 dec = *(const f4*)cl, dec_1 = *(const f4*)(cl - (p.nc > 1 ? vstep : 0));
-  f4 hn[KM], dh[KM], hn_1[KM], dh_1[KM];
-  {
-    const long back = p.nc > 1 ? cstep : 0;
+  // Operands of three chunks in three register slots: the one being used, the next, and the one after that, which is
+  // requested at the top of a step (the last two steps request chunk 0 again: in range, unused).  Step j = nc-1-c
+  // uses slot j % 3; the loop is unrolled over the slots so that none is ever copied (a copy would wait for its load).
+  f4 dec[3], hn[3][KM], dh[3][KM];
+  auto request = [&](int slot, int back_chunks) {
+    const long back = (long)back_chunks * cstep;
+    dec[slot] = *(const f4*)(cl - (long)back_chunks * vstep);
 #pragma unroll
     for (int k = 0; k < KM; ++k) {
-      hn[k] = *(const f4*)(hp + k * kstep);
-      dh[k] = *(const f4*)(dd + k * kstep);
-      hn_1[k] = *(const f4*)(hp - back + k * kstep);
-      dh_1[k] = *(const f4*)(dd - back + k * kstep);
+      hn[slot][k] = *(const f4*)(hp - back + k * kstep);
+      dh[slot][k] = *(const f4*)(dd - back + k * kstep);
     }
-  }
-  for (int c = p.nc - 1; c >= 0; --c) {
-    const long back = (long)min(c, 2) * cstep, vback = (long)min(c, 2) * vstep;
-    f4 dec_n = *(const f4*)(cl - vback), hn_n[KM], dh_n[KM];
-#pragma unroll
-    for (int k = 0; k < KM; ++k) {
-      hn_n[k] = *(const f4*)(hp - back + k * kstep);
-      dh_n[k] = *(const f4*)(dd - back + k * kstep);
-    }
+  };
+  request(0, 0);
+  request(1, p.nc > 1 ? 1 : 0);
+  auto step = [&](int cur, int pre, int c) {
+    request(pre, min(c, 2));
     f4 gp = {0, 0, 0, 0}, e;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) e[j] = __expf(dec[j]);
+    for (int j = 0; j < 4; ++j) e[j] = __expf(dec[cur][j]);
 #pragma unroll
     for (int k = 0; k < KM; ++k) {
       *(f4*)(dd + k * kstep) = carry[k];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        gp[j] += hn[k][j] * carry[k][j];
-        carry[k][j] = e[j] * carry[k][j] + dh[k][j];
+        gp[j] += hn[cur][k][j] * carry[k][j];
+        carry[k][j] = e[j] * carry[k][j] + dh[cur][k][j];
       }
     }
     *(f4*)(red + pg * NCOL + nq * 4) = gp;
@@ -337,11 +332,16 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
       if (part == 0) gl[col] = sum;
     }
     __syncthreads();
-    dec = dec_1; dec_1 = dec_n;
-#pragma unroll
-    for (int k = 0; k < KM; ++k) { hn[k] = hn_1[k]; dh[k] = dh_1[k]; hn_1[k] = hn_n[k]; dh_1[k] = dh_n[k]; }
     hp -= cstep; dd -= cstep; cl -= vstep; gl -= vstep;
+  };
+  int c = p.nc - 1;
+  for (; c >= 2; c -= 3) {
+    step(0, 2, c);
+    step(1, 0, c - 1);
+    step(2, 1, c - 2);
   }
+  if (c >= 0) step(0, 2, c);      // uniform: the last nc % 3 chunks
+  if (c >= 1) step(1, 0, c - 1);
 #pragma unroll
   for (int k = 0; k < KM; ++k)
     *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + row + k * kstep) = carry[k];
