@@ -262,7 +262,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 // loads still in flight and the prefetched operands of the next two chunks stay in flight across the barriers
 // (with loads inside branches it waits for all of them before each store, which exposes the full memory latency
 // once per chunk; few workgroups walking many chunks -- batch 2, 256 chunks -- then run at that pace).
-template <int NQ, int KM>
+template <int NQ, int KM, int R>
 __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* __restrict__ states,
                                                              const float* __restrict__ cs_last,
                                                              float* __restrict__ dstates, float* __restrict__ g_last,
@@ -290,10 +290,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   float* dd = dstates + dst_off(p, bt, p.nc - 1, h) + row;       // dH_c in, dS_c out
   const float* cl = cs_last + vec_off(p, bt, p.nc - 1, h) + n;
   float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;
-  // Operands of three chunks in three register slots: the one being used, the next, and the one after that, which is
-  // requested at the top of a step (the last two steps request chunk 0 again: in range, unused).  Step j = nc-1-c
-  // uses slot j % 3; the loop is unrolled over the slots so that none is ever copied (a copy would wait for its load).
-  f4 dec[3], hn[3][KM], dh[3][KM];
+  // Operands of R chunks in R register slots: the one being used and the next R - 1, the last of which is requested
+  // at the top of a step (the final steps request chunk 0 again: in range, unused).  Step j = nc-1-c uses slot
+  // j % R; the loop is unrolled over the slots so that none is ever copied (a copy would wait for its load).
+  f4 dec[R], hn[R][KM], dh[R][KM];
   auto request = [&](int slot, int back_chunks) {
     const long back = (long)back_chunks * cstep;
     dec[slot] = *(const f4*)(cl - (long)back_chunks * vstep);
@@ -303,10 +303,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
       dh[slot][k] = *(const f4*)(dd - back + k * kstep);
     }
   };
-  request(0, 0);
-  request(1, p.nc > 1 ? 1 : 0);
+#pragma unroll
+  for (int i = 0; i < R - 1; ++i) request(i, min(i, p.nc - 1));
   auto step = [&](int cur, int pre, int c) {
-    request(pre, min(c, 2));
+    request(pre, min(c, R - 1));
     f4 gp = {0, 0, 0, 0}, e;
 #pragma unroll
     for (int j = 0; j < 4; ++j) e[j] = __expf(dec[cur][j]);
@@ -335,13 +335,13 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     hp -= cstep; dd -= cstep; cl -= vstep; gl -= vstep;
   };
   int c = p.nc - 1;
-  for (; c >= 2; c -= 3) {
-    step(0, 2, c);
-    step(1, 0, c - 1);
-    step(2, 1, c - 2);
+  for (; c >= R - 1; c -= R) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) step(i, (i + R - 1) % R, c - i);
   }
-  if (c >= 0) step(0, 2, c);      // uniform: the last nc % 3 chunks
-  if (c >= 1) step(1, 0, c - 1);
+#pragma unroll
+  for (int i = 0; i < R - 1; ++i)
+    if (c - i >= 0) step(i, (i + R - 1) % R, c - i);  // uniform: the last nc % R chunks
 #pragma unroll
   for (int k = 0; k < KM; ++k)
     *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + row + k * kstep) = carry[k];
@@ -1000,17 +1000,17 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
   // One workgroup walks the chunks of its columns one after the other.  Complete shapes take the variant without
   // conditional accesses; with few (batch, head) pairs narrower column slices put more workgroups on the chip.
   const int wide = p.B * p.ndir * p.H * ((p.N + 63) / 64);
-#define ISSM_STATE_BWD_FULL(NQ_, KM_)                                                                                   \
-  hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
+#define ISSM_STATE_BWD_FULL(NQ_, KM_, R_)                                                                                  \
+  hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_, R_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
                      states, cs_last, dstates, g_last, dh0_dir)
   if (wide < 256 && p.N % 32 == 0 && (p.P == 32 || p.P == 64)) {
-    if (p.P == 32) ISSM_STATE_BWD_FULL(8, 1); else ISSM_STATE_BWD_FULL(8, 2);
+    if (p.P == 32) ISSM_STATE_BWD_FULL(8, 1, 6); else ISSM_STATE_BWD_FULL(8, 2, 4);
   } else if (p.N % 64 == 0 && p.P % 16 == 0) {
     switch (p.P / 16) {
-      case 1: ISSM_STATE_BWD_FULL(16, 1); break;
-      case 2: ISSM_STATE_BWD_FULL(16, 2); break;
-      case 3: ISSM_STATE_BWD_FULL(16, 3); break;
-      default: ISSM_STATE_BWD_FULL(16, 4); break;
+      case 1: ISSM_STATE_BWD_FULL(16, 1, 3); break;
+      case 2: ISSM_STATE_BWD_FULL(16, 2, 3); break;
+      case 3: ISSM_STATE_BWD_FULL(16, 3, 3); break;
+      default: ISSM_STATE_BWD_FULL(16, 4, 3); break;
     }
   } else if (wide < 256) {
     const int blocks = p.B * p.ndir * p.H * ((p.N + 15) / 16);
