@@ -268,7 +268,8 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
                                                              float* __restrict__ dstates, float* __restrict__ g_last,
                                                              float* __restrict__ dh0_dir) {
   constexpr int NCOL = NQ * 4, PGN = NTHREADS / NQ;
-  __shared__ __align__(16) float red[PGN * NCOL];
+  __shared__ __align__(16) float red2[2][PGN * NCOL];  // two buffers, used in turn: one barrier per step
+  int par = 0;
   const int nsl = p.N / NCOL;
   int bid = blockIdx.x;
   const int ns = bid % nsl;
@@ -319,8 +320,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
         carry[k][j] = e[j] * carry[k][j] + dh[cur][k][j];
       }
     }
+    float* red = red2[par];
+    par ^= 1;
     *(f4*)(red + pg * NCOL + nq * 4) = gp;
-    __syncthreads();
+    __syncthreads();  // the buffer is written again two steps later, after the next step's barrier
     if (tid < 64) {
       constexpr int PARTS = 64 / NCOL;
       const int col = tid % NCOL, part = tid / NCOL;
@@ -331,7 +334,6 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
       for (int d = NCOL; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
       if (part == 0) gl[col] = sum;
     }
-    __syncthreads();
     hp -= cstep; dd -= cstep; cl -= vstep; gl -= vstep;
   };
   int c = p.nc - 1;
