@@ -257,11 +257,12 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
   }
 }
 
-// The same recurrence for complete shapes -- N a multiple of the slice width, P exactly KM rows per thread -- with
-// no conditional access anywhere: every load of the loop is issued on every path, so the compiler can count the
-// loads still in flight and the prefetched operands of the next two chunks stay in flight across the barriers
-// (with loads inside branches it waits for all of them before each store, which exposes the full memory latency
-// once per chunk; few workgroups walking many chunks -- batch 2, 256 chunks -- then run at that pace).
+// The same recurrence for N a multiple of the slice width, with no conditional access anywhere: every load of the
+// loop is issued on every path, so the compiler can count the loads still in flight and the prefetched operands of
+// the next chunks stay in flight across the barrier (with loads inside branches it waits for all of them before each
+// store, which exposes the full memory latency once per chunk; few workgroups walking many chunks -- batch 2, 256
+// chunks -- then run at that pace).  A thread owns KM rows, pg + PGN k; rows past the head dimension are replaced by
+// its last row: those threads compute and store exactly what the row's owner does, and stay out of the column sums.
 template <int NQ, int KM, int R>
 __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* __restrict__ states,
                                                              const float* __restrict__ cs_last,
@@ -279,16 +280,22 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   const int b = bt / p.ndir, dir = bt % p.ndir;
   const int tid = threadIdx.x, pg = tid / NQ, nq = tid % NQ;
   const int n = ns * NCOL + nq * 4;
-  const long row = (long)pg * p.N + n, kstep = (long)PGN * p.N;  // the thread's first row; from row block to row block
+  long rowk[KM];   // offsets of the thread's rows
+  float own[KM];   // 1 for a row of its own, 0 for a stand-in
+#pragma unroll
+  for (int k = 0; k < KM; ++k) {
+    rowk[k] = (long)min(pg + PGN * k, p.P - 1) * p.N + n;
+    own[k] = pg + PGN * k < p.P ? 1.0f : 0.0f;
+  }
   const long cstep = (long)p.H * p.P * p.N, vstep = (long)p.H * p.N;  // from chunk to chunk
   f4 carry[KM];
 #pragma unroll
   for (int k = 0; k < KM; ++k) {
     carry[k] = (f4){0, 0, 0, 0};
-    if (p.dfinal[dir]) carry[k] = *(const f4*)(p.dfinal[dir] + ((long)b * p.H + h) * p.P * p.N + row + k * kstep);
+    if (p.dfinal[dir]) carry[k] = *(const f4*)(p.dfinal[dir] + ((long)b * p.H + h) * p.P * p.N + rowk[k]);
   }
-  const float* hp = states + st_off(p, bt, p.nc, h) + row;       // H_{c+1}, c = nc - 1
-  float* dd = dstates + dst_off(p, bt, p.nc - 1, h) + row;       // dH_c in, dS_c out
+  const float* hp = states + st_off(p, bt, p.nc, h);      // H_{c+1}, c = nc - 1
+  float* dd = dstates + dst_off(p, bt, p.nc - 1, h);      // dH_c in, dS_c out
   const float* cl = cs_last + vec_off(p, bt, p.nc - 1, h) + n;
   float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;
   // Operands of R chunks in R register slots: the one being used and the next R - 1, the last of which is requested
@@ -300,8 +307,8 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     dec[slot] = *(const f4*)(cl - (long)back_chunks * vstep);
 #pragma unroll
     for (int k = 0; k < KM; ++k) {
-      hn[slot][k] = *(const f4*)(hp - back + k * kstep);
-      dh[slot][k] = *(const f4*)(dd - back + k * kstep);
+      hn[slot][k] = *(const f4*)(hp - back + rowk[k]);
+      dh[slot][k] = *(const f4*)(dd - back + rowk[k]);
     }
   };
 #pragma unroll
@@ -313,10 +320,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     for (int j = 0; j < 4; ++j) e[j] = __expf(dec[cur][j]);
 #pragma unroll
     for (int k = 0; k < KM; ++k) {
-      *(f4*)(dd + k * kstep) = carry[k];
+      *(f4*)(dd + rowk[k]) = carry[k];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        gp[j] += hn[cur][k][j] * carry[k][j];
+        gp[j] += own[k] * hn[cur][k][j] * carry[k][j];
         carry[k][j] = e[j] * carry[k][j] + dh[cur][k][j];
       }
     }
@@ -346,7 +353,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     if (c - i >= 0) step(i, (i + R - 1) % R, c - i);  // uniform: the last nc % R chunks
 #pragma unroll
   for (int k = 0; k < KM; ++k)
-    *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + row + k * kstep) = carry[k];
+    *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + rowk[k]) = carry[k];
 }
 
 // -------------------------------------------------------------- chunk backward
@@ -1005,10 +1012,10 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
 #define ISSM_STATE_BWD_FULL(NQ_, KM_, R_)                                                                                  \
   hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_, R_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
                      states, cs_last, dstates, g_last, dh0_dir)
-  if (wide < 256 && p.N % 32 == 0 && (p.P == 32 || p.P == 64)) {
-    if (p.P == 32) ISSM_STATE_BWD_FULL(8, 1, 6); else ISSM_STATE_BWD_FULL(8, 2, 4);
-  } else if (p.N % 64 == 0 && p.P % 16 == 0) {
-    switch (p.P / 16) {
+  if (wide < 256 && p.N % 32 == 0) {
+    if (p.P <= 32) ISSM_STATE_BWD_FULL(8, 1, 6); else ISSM_STATE_BWD_FULL(8, 2, 4);
+  } else if (p.N % 64 == 0) {
+    switch ((p.P + 15) / 16) {
       case 1: ISSM_STATE_BWD_FULL(16, 1, 3); break;
       case 2: ISSM_STATE_BWD_FULL(16, 2, 3); break;
       case 3: ISSM_STATE_BWD_FULL(16, 3, 3); break;
