@@ -190,8 +190,8 @@ class Runner:
 # plain 256 MiB copy of --calib-copy (fetch x2.000, write x1.000); the summary is kept under profiles/.
 # k_bwd_chunk is launched once per direction: the figure is per launch.  Override with --traffic.
 MEASURED_TRAFFIC_BYTES = {
-    "chunk_local": 275.0e6, "state_passing_fwd": 161.6e6, "chunk_scan": 260.6e6, "bwd_dstates": 274.0e6,
-    "state_passing_bwd": 214.0e6, "bwd_chunk": 301.3e6, "bwd_dx": 277.8e6,
+    "chunk_local": 208.0e6, "state_passing_fwd": 162.6e6, "chunk_scan": 210.2e6, "bwd_dstates": 206.6e6,
+    "state_passing_bwd": 214.0e6, "bwd_chunk": 301.3e6, "bwd_dx": 244.3e6,
 }
 
 

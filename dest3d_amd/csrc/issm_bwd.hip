@@ -2,7 +2,7 @@
 //
 //   k_bwd_gate      z-gate backward (elementwise)
 //   k_bwd_dstates   dH_c = dy^T (C*exp(cs))  and  dM = tril(dy x^T)
-//   k_state_bwd     reverse inter-chunk recurrence (HBM streaming)
+//   k_state_bwd_full / k_state_bwd   reverse inter-chunk recurrence (HBM streaming)
 //   k_bwd_chunk     per (chunk, group, 64-column slice), looping over the heads of the
 //                   group: ddt, dB, dC and the per-unit partial sums of dA / ddt_bias
 //   k_bwd_dx        dx and the per-unit partial sums of dD

@@ -2,7 +2,7 @@
 //
 //   k_chunk_local   dt transform + cumsum, chunk-local end states S_c and the intra-chunk
 //                   matrix M_c = "C.A.B^T" in one pass over dt
-//   k_state_fwd     inter-chunk recurrence (HBM streaming)
+//   k_state_fwd_full / k_state_fwd   inter-chunk recurrence (HBM streaming)
 //   k_chunk_scan    y = (C*exp(cs)) H^T + tril(M) x + D x, optional gate
 //
 // The decay exp(cs[l]-cs[s]) sits inside the contraction over the state index n, so
@@ -344,9 +344,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd_full(KP p, float* __rest
   if (p.final_states[dir]) *(f4*)(p.final_states[dir] + (((long)b * p.H + h) * p.P + pp) * p.N + n) = st;
 }
 
-// D: chunks of operands a thread keeps in flight (2 when the launch has plenty of threads; 8 when a few threads walk
-// many chunks, e.g. batch 2 x 256 chunks, where memory latency and not bandwidth sets the pace)
-template <int D>
+// The recurrence for any N (launched when N is not a multiple of 4): element-wise guards, scalar accesses.
 __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict__ states,
                                                         const float* __restrict__ cs_last) {
   const int nq = (p.N + 3) >> 2;
@@ -361,7 +359,6 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
   const int bt = r / p.H;
   const int b = bt / p.ndir, dir = bt % p.ndir;
   const int n = q * 4;
-  const bool full = (n + 3 < p.N) && ((p.N & 3) == 0);
   float st[4] = {0, 0, 0, 0};
   if (p.h0.ptr) {
     const long o = (long)b * p.h0.s0 + (long)h * p.h0.s1 + (long)pp * p.h0.s2 + n;
@@ -371,62 +368,18 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
   const long cstride = (long)p.H * p.P * p.N;
   float* sp = states + st_off(p, bt, 0, h) + (long)pp * p.N + n;
   const float* cl = cs_last + vec_off(p, bt, 0, h) + n;
-  if (full && D > 2) {
-    const long dstride = (long)p.H * p.N;
-    f4 t[D], d[D];
-#pragma unroll
-    for (int i = 0; i < D; ++i) {
-      const int ci = min(i, p.nc - 1);
-      t[i] = *(const f4*)(sp + ci * cstride);
-      d[i] = *(const f4*)(cl + ci * dstride);
+  for (int c = 0; c < p.nc; ++c) {
+    float sv[4], dv[4];
+    for (int j = 0; j < 4; ++j) {
+      const bool v = n + j < p.N;
+      sv[j] = v ? sp[j] : 0.0f;
+      dv[j] = v ? cl[j] : 0.0f;
+      if (v) sp[j] = st[j];
     }
-    for (int c0 = 0; c0 < p.nc; c0 += D) {
 #pragma unroll
-      for (int i = 0; i < D; ++i) {
-        if (c0 + i < p.nc) {  // uniform
-          const f4 tt = t[i], dd = d[i];
-          if (c0 + i + D < p.nc) {  // uniform: the slot's next occupant, D chunks ahead
-            t[i] = *(const f4*)(sp + D * cstride);
-            d[i] = *(const f4*)(cl + D * dstride);
-          }
-          *(f4*)sp = (f4){st[0], st[1], st[2], st[3]};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) st[j] = __expf(dd[j]) * st[j] + tt[j];
-          sp += cstride;
-          cl += dstride;
-        }
-      }
-    }
-  } else if (full) {
-    // S_c and the chunk decay of the next two chunks are always in flight: the loads do not depend on
-    // the running state, only the store into the slot just read does
-    const long dstride = (long)p.H * p.N;
-    f4 t0 = *(const f4*)sp, d0 = *(const f4*)cl, t1 = t0, d1 = d0;
-    if (p.nc > 1) { t1 = *(const f4*)(sp + cstride); d1 = *(const f4*)(cl + dstride); }
-    for (int c = 0; c < p.nc; ++c) {
-      f4 t2 = t1, d2 = d1;
-      if (c + 2 < p.nc) { t2 = *(const f4*)(sp + 2 * cstride); d2 = *(const f4*)(cl + 2 * dstride); }
-      *(f4*)sp = (f4){st[0], st[1], st[2], st[3]};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) st[j] = __expf(d0[j]) * st[j] + t0[j];
-      t0 = t1; d0 = d1; t1 = t2; d1 = d2;
-      sp += cstride;
-      cl += dstride;
-    }
-  } else {
-    for (int c = 0; c < p.nc; ++c) {
-      float sv[4], dv[4];
-      for (int j = 0; j < 4; ++j) {
-        const bool v = n + j < p.N;
-        sv[j] = v ? sp[j] : 0.0f;
-        dv[j] = v ? cl[j] : 0.0f;
-        if (v) sp[j] = st[j];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) st[j] = __expf(dv[j]) * st[j] + sv[j];
-      sp += cstride;
-      cl += (long)p.H * p.N;
-    }
+    for (int j = 0; j < 4; ++j) st[j] = __expf(dv[j]) * st[j] + sv[j];
+    sp += cstride;
+    cl += (long)p.H * p.N;
   }
   // slot nc keeps the final state for the backward pass
   for (int j = 0; j < 4; ++j)
@@ -585,10 +538,9 @@ int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream
       hipLaunchKernelGGL(k_state_fwd_full<8>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
     else
       hipLaunchKernelGGL(k_state_fwd_full<4>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
-  } else if (total < (1L << 17) && p.nc >= 16)
-    hipLaunchKernelGGL(k_state_fwd<8>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
-  else
-    hipLaunchKernelGGL(k_state_fwd<2>, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+  } else {
+    hipLaunchKernelGGL(k_state_fwd, dim3(blocks), dim3(NTHREADS), 0, st, p, states, cs_last);
+  }
   return (int)hipGetLastError();
 }
 
