@@ -96,37 +96,47 @@ __global__ __launch_bounds__(NTHREADS) void k_pgen_fwd(PGenP p) {
   float wk[KV];
 #pragma unroll
   for (int j = 0; j < KV; ++j) wk[j] = p.weights ? p.weights[t * p.K + k + j] : 1.0f;
+  // the token's biases, all requested before the row loop (a load per row inside it would be waited for row by
+  // row); bb: the reversed-order pair's bias of a B / C row
   const float* bias = p.bias + t * R;
-  for (int r = 0; r < R0; ++r) {
-    const float* w = p.W + r * PG_M;  // uniform: scalar loads
-    float s[KV], v[KV];
+  float bv[PG_MAXR0], bb[PG_MAXR0];
 #pragma unroll
-    for (int j = 0; j < KV; ++j) {
-      s[j] = 0.0f;
+  for (int r = 0; r < PG_MAXR0; ++r) {
+    bv[r] = bias[min(r, R - 1)];
+    bb[r] = bias[min(max(R0 + r - p.H, 0), R - 1)];
+  }
 #pragma unroll
-      for (int m = 0; m < PG_M; ++m) s[j] = fmaf(w[m], d[j][m], s[j]);
-      v[j] = s[j] + bias[r];
-    }
-    if (r < p.H) {
-      if (p.weights) {  // uniform: dt = softplus(raw) * weight, raw kept for the backward
-        if (BF) {
+  for (int r = 0; r < PG_MAXR0; ++r) {
+    if (r < R0) {  // uniform
+      const float* w = p.W + r * PG_M;  // uniform: scalar loads
+      float s[KV], v[KV];
 #pragma unroll
-          for (int j = 0; j < KV; ++j) v[j] = bf16_to_f(f_to_bf16(v[j]));  // the saved value is what the backward differentiates
-        }
-        stv<BF, KV>(p.dt_raw, (t * p.H + r) * p.K + k, v);
+      for (int j = 0; j < KV; ++j) {
+        s[j] = 0.0f;
 #pragma unroll
-        for (int j = 0; j < KV; ++j) v[j] = softplus_(v[j]) * wk[j];
+        for (int m = 0; m < PG_M; ++m) s[j] = fmaf(w[m], d[j][m], s[j]);
+        v[j] = s[j] + bv[r];
       }
-      stv<BF, KV>(p.dt, (t * p.H + r) * p.K + k, v);
-    } else {
-      const bool isB = r < p.H + p.G;
-      const int g = isB ? r - p.H : r - p.H - p.G;
-      stv<BF, KV>(isB ? p.Bm : p.Cm, (t * p.G + g) * p.K + k, v);
-      if (p.has_back) {
-        const float bb = bias[R0 + (isB ? 0 : p.G) + g];
+      if (r < p.H) {
+        if (p.weights) {  // uniform: dt = softplus(raw) * weight, raw kept for the backward
+          if (BF) {
 #pragma unroll
-        for (int j = 0; j < KV; ++j) v[j] = s[j] + bb;
-        stv<BF, KV>(isB ? p.Bb : p.Cb, (t * p.G + g) * p.K + k, v);
+            for (int j = 0; j < KV; ++j) v[j] = bf16_to_f(f_to_bf16(v[j]));  // the saved value is what the backward differentiates
+          }
+          stv<BF, KV>(p.dt_raw, (t * p.H + r) * p.K + k, v);
+#pragma unroll
+          for (int j = 0; j < KV; ++j) v[j] = softplus_(v[j]) * wk[j];
+        }
+        stv<BF, KV>(p.dt, (t * p.H + r) * p.K + k, v);
+      } else {
+        const bool isB = r < p.H + p.G;
+        const int g = isB ? r - p.H : r - p.H - p.G;
+        stv<BF, KV>(isB ? p.Bm : p.Cm, (t * p.G + g) * p.K + k, v);
+        if (p.has_back) {
+#pragma unroll
+          for (int j = 0; j < KV; ++j) v[j] = s[j] + bb[r];
+          stv<BF, KV>(isB ? p.Bb : p.Cb, (t * p.G + g) * p.K + k, v);
+        }
       }
     }
   }
