@@ -363,11 +363,16 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
 template <int PT>
 struct BwdChunkSmem {
   static constexpr int KW = 16 * PT;  // stored width; the K = 32 steps read missing columns as zero
+  // Four head tiles (P > 48): the dM tile takes the place of the x tile once the products over the head dimension
+  // are done, which keeps the workgroup under half of the CU's LDS (two workgroups per CU instead of one).
+  static constexpr bool DM_OVER_X = PT > 3;
   SplitTile<KW> xs;   // x tile [l][p] as bf16 (hi, lo)
   SplitTile<KW> dys;  // dy tile
-  float dms[CS * LDC];
+  float dms_own[DM_OVER_X ? 4 : CS * LDC];
   float dbc[32 * NTHREADS];  // per-lane dB / dC accumulators [k][tid]
+  __device__ __forceinline__ float* dms() { return DM_OVER_X ? reinterpret_cast<float*>(&xs) : dms_own; }
 };
+static_assert(sizeof(SplitTile<64>) >= CS * LDC * sizeof(float), "the dM tile must fit in the x tile's place");
 
 // F[l] = sum_{s<=l} dM[l,s] Bd[s] exp2(cs[l]-cs[s]) and G[s] = sum_{l>=s} dM[l,s] C[l] exp2(cs[l]-cs[s]) per state
 // column, accumulated into x2 (F) and e1 (G).  A pair (l > s) is handled at the level w = highest set
@@ -580,6 +585,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     const float gl = (g4 == 3 && vn) ? g_last[vec_off(p, u.bt, u.c, u.h) + n] : 0.0f;
     lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
     lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
+    f4 mkeep[SM::DM_OVER_X ? 4 : 1];  // the thread's part of the dM tile until the x tile's place is free
     {
       float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
       f4 mv[4];
@@ -591,7 +597,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       __syncthreads();  // the previous head no longer reads the LDS tiles
       lp_store_split<PT, LDS_>(dv, s.dys.hi, s.dys.lo, tq);
       lp_store_split<PT, LDS_>(xv, s.xs.hi, s.xs.lo, tq);
-      tril_store(mv, s.dms, tq);
+      if constexpr (!SM::DM_OVER_X) tril_store(mv, s.dms(), tq);
+      else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) mkeep[v] = mv[v];
+      }
     }
     __syncthreads();
 
@@ -674,23 +684,30 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
       }
     }
 
+    if constexpr (SM::DM_OVER_X) {
+      __syncthreads();  // every wave is done with the x tile
+      int tq = tid;
+      asm volatile("" : "+v"(tq));
+      tril_store(mkeep, s.dms(), tq);
+      __syncthreads();
+    }
     // ---- hierarchy levels of F and G; scheduling barriers keep one level's operands live at a time
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level<5>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_big_level<5>(cs, Bd, Cv, s.dms(), e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level<4>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_big_level<4>(cs, Bd, Cv, s.dms(), e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level<3>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_mid_level<3>(cs, Bd, Cv, s.dms(), e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level<2>(cs, Bd, Cv, s.dms, e1, x2, cq, gq);
+    bwd_mid_level<2>(cs, Bd, Cv, s.dms(), e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
@@ -698,7 +715,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     float old[16];
     if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_small_levels(cs, Bd, Cv, s.dms, e1, x2, gq);
+    bwd_small_levels(cs, Bd, Cv, s.dms(), e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase: everything below is local to the lane except the scans over rows
