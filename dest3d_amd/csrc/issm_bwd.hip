@@ -1029,7 +1029,7 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
 #define ISSM_STATE_BWD_FULL(NQ_, KM_, R_)                                                                                  \
   hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_, R_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
                      states, cs_last, dstates, g_last, dh0_dir)
-  if (wide < 256 && p.N % 32 == 0) {
+  if (p.N % 32 == 0 && (wide < 256 || p.N % 64 != 0)) {
     if (p.P <= 32) ISSM_STATE_BWD_FULL(8, 1, 6); else ISSM_STATE_BWD_FULL(8, 2, 4);
   } else if (p.N % 64 == 0) {
     switch ((p.P + 15) / 16) {

@@ -110,6 +110,7 @@ CASES = [
     (1, 64 * 37, 2, 20, 64, 1, dict()),
     (1, 64 * 7 - 5, 1, 40, 96, 1, dict(D="hp")),          # two rows per thread, four slots, ragged last chunk
     (4, 64 * 5, 8, 36, 256, 1, dict(softplus=False)),    # 64-column slices, three slots, 5 chunks, P = 36
+    (16, 70, 8, 16, 96, 1, dict()),                      # many workgroups, N a multiple of 32 but not of 64
 ]
 
 
