@@ -492,6 +492,19 @@ def main():
             variants[name] = round(r.time_steps(max(args.steps // 2, 5), 5), 2)
             del r
         SHAPE["P"] = 32
+        # the other scan configurations of the baseline: long sequence (B 2, L 16384, bf16, one direction) and
+        # large state (B 16, L 2048, H 16, P 64, N 512, fp32, both directions)
+        keep = dict(SHAPE)
+        for name, shp, nd, dt in (("long_sequence_B2_L16384_uni_bf16", dict(B=2, L=16384), 1, torch.bfloat16),
+                                  ("large_state_B16_L2048_H16_P64_N512_bidir_fp32",
+                                   dict(B=16, L=2048, H=16, P=64, N=512), 2, torch.float32)):
+            SHAPE.update(shp)
+            r = Runner(torch, nd, dt)
+            variants[name] = round(r.time_steps(5, 2), 2)
+            del r
+            torch.cuda.empty_cache()
+            SHAPE.clear()
+            SHAPE.update(keep)
         variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
         variants["detector_layer_bf16_fwd_bwd_as_hip_graph"] = round(time_module_layer(torch, as_graph=True), 2)
         variants["detector_layer_fp32_fwd_bwd"] = round(time_module_layer(torch, dtype=torch.float32), 2)
