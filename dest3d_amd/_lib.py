@@ -108,6 +108,7 @@ class DwConvArgs(C.Structure):
         ("dbias", C.c_void_p), ("stream", C.c_void_p),
         ("split", C.c_int32), ("y_tail", C.c_void_p), ("dy_tail", C.c_void_p * 2),
         ("du_batch_stride", C.c_int64), ("du_token_stride", C.c_int64),
+        ("chain", C.c_int32),
     ]
 
 

@@ -18,9 +18,15 @@ FLAGS = [
 ]
 
 
+# Sources whose results are integers decided by a floating-point quotient: compiled with IEEE division (no
+# reciprocal-multiply rewriting), so that a point exactly on a cell boundary lands in the same cell as on the host.
+EXACT_DIVISION = {"hilbert.hip"}
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    flags = [f for f in FLAGS if f not in ("-ffast-math", "-fno-finite-math-only")] if src in EXACT_DIVISION else FLAGS
+    cmd = [HIPCC, *flags, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -43,19 +49,5 @@ def build(verbose: bool = True) -> str:
     return LIB
 
 
-def build_probe() -> str:
-    """Stand-alone issue-rate probe (matrix vs vector instructions); not part of the library."""
-    out = os.path.join(HERE, "probe_mfma_valu")
-    cmd = [HIPCC, *[f for f in FLAGS if f != "-fPIC"], os.path.join(CSRC, "probe_mfma_valu.hip"), "-o", out]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed for the probe:\n{r.stderr}")
-    print(f"built {out}")
-    return out
-
-
 if __name__ == "__main__":
-    if "--probe" in sys.argv[1:]:
-        build_probe()
-    else:
-        build()
+    build()

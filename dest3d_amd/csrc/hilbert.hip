@@ -50,7 +50,10 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_codes(HilbertP p) {
   const int cap = (1 << p.bits) - 1;
 #pragma unroll
   for (int i = 0; i < 3; ++i) {
-    const float v = truncf((q[i] - mn[i]) / p.cell);  // a true division, as torch.div(..., rounding_mode="trunc")
+    // a correctly rounded division, as torch.div(..., rounding_mode="trunc") performs on the host: this file is built
+    // without fast-math, which would turn it into a multiplication by an approximate reciprocal and move points that
+    // sit exactly on a cell boundary into the neighbouring cell
+    const float v = truncf((q[i] - mn[i]) / p.cell);
     int c = v >= (float)cap ? cap : (int)v;
     g[i] = (unsigned)(c < 0 ? 0 : c);
   }

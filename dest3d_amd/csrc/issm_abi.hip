@@ -482,6 +482,7 @@ static int dwconv_params(const issm_dwconv_args* a, DwConvP* p, bool bwd) {
   if (a->batch < 0 || a->seqlen < 0 || a->channels < 1) return fail(ISSM_E_SHAPE, "dwconv: bad shape");
   if (a->taps != 7) return fail(ISSM_E_UNSUPPORTED, "dwconv: %d taps (only 7 is built)", a->taps);
   if (a->nsets < 1 || a->nsets > 2) return fail(ISSM_E_UNSUPPORTED, "dwconv: nsets = %d (1 or 2)", a->nsets);
+  if (a->chain && a->nsets != 2) return fail(ISSM_E_SHAPE, "dwconv: chain needs nsets = 2, got %d", a->nsets);
   if (a->dtype != ISSM_F32 && a->dtype != ISSM_BF16) return fail(ISSM_E_DTYPE, "dwconv: dtype %d", a->dtype);
   if (!a->u || !a->w || !a->pre) return fail(ISSM_E_NULL, "dwconv: u/w/pre is NULL");
   if (a->u_token_stride < a->channels || a->u_batch_stride < 0)
@@ -489,6 +490,7 @@ static int dwconv_params(const issm_dwconv_args* a, DwConvP* p, bool bwd) {
   if (!bwd && (!a->bias || !a->y)) return fail(ISSM_E_NULL, "dwconv: bias/y is NULL");
   if (bwd && (!a->partial || !a->dw || !a->dbias)) return fail(ISSM_E_NULL, "dwconv bwd: partial/dw/dbias is NULL");
   p->B = a->batch; p->L = a->seqlen; p->C = a->channels; p->nsets = a->nsets; p->dtype = a->dtype;
+  p->chain = a->chain ? 1 : 0;
   p->u = a->u; p->u_bs = a->u_batch_stride; p->u_ls = a->u_token_stride;
   if (a->split < 0 || a->split >= a->channels) return fail(ISSM_E_SHAPE, "dwconv: split %d outside [0, channels)", a->split);
   if (a->split > 0 && !bwd && !a->y_tail) return fail(ISSM_E_NULL, "dwconv: y_tail is NULL");

@@ -111,6 +111,7 @@ struct BoxDistP {
 // parameters of the depthwise conv + SiLU kernels (dwconv_silu.hip)
 struct DwConvP {
   int B, L, C, nsets, dtype;
+  int chain;           // nsets == 2: set 1 convolves set 0's output instead of u
   const void* u;       // (B, L, C) io dtype, element strides u_bs (batch), u_ls (token), channels contiguous
   long u_bs, u_ls;
   const float* w;      // (nsets, C, 7) fp32

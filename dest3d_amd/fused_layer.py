@@ -1,7 +1,8 @@
 """The core of MultiHeadISSMScan as one autograd node.
 
 Between the input projections and the output projections, MultiHeadISSMScan.forward (models/dest_module.py:528-581)
-is a fixed chain: depthwise conv + SiLU of both branches, generation of dt / B / C from the distance encoding, the
+is a fixed chain: depthwise conv + SiLU of both branches (the reversed-order branch convolves the forward-order
+branch's output, dest_module.py:530,534), generation of dt / B / C from the distance encoding, the
 bidirectional scan, the average of the two directions, the gated RMSNorm.  Run as separate autograd Functions and
 PyTorch ops that is some forty small operations forward and as many autograd nodes backward, and at the detector's
 layer shape the host cannot issue them as fast as the GPU finishes them.  ``fused_scan_core`` makes the same calls
@@ -78,6 +79,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             a = _dw._args(xbc, 2)
             a.w, a.bias, a.y, a.pre = cw.data_ptr(), cb.data_ptr(), x.data_ptr(), pre.data_ptr()
             a.split, a.y_tail = di, tail.data_ptr()
+            a.chain = 1                                                      # key_conv_back reads key_conv's output
             L.check(lib.issm_dwconv_silu_fwd(C.byref(a)), "issm_dwconv_silu_fwd")
             x_f, x_b = x[0], x[1]
             # 2. dt / B / C (and the reversed-order B / C) from the distance encoding
@@ -178,7 +180,7 @@ class FusedScanCoreFn(torch.autograd.Function):
             dcb = torch.empty((2, Cc), dtype=torch.float32, device=dev)
             a = _dw._args(xbc, 2)
             a.w, a.pre = cw.data_ptr(), pre.data_ptr()
-            a.split = di
+            a.split, a.chain = di, 1
             a.dy[0], a.dy[1] = dxs[0].data_ptr(), dxs[1].data_ptr()
             a.dy_tail[0], a.dy_tail[1] = dtail[0].data_ptr(), dtail[1].data_ptr()
             a.du = dzx.data_ptr() + di * dzx.element_size()

@@ -204,6 +204,10 @@ class ISSMChunkScanCombinedFn(torch.autograd.Function):
         prob = _Problem([x], dt, A, [B], [C], chunk_size, D, [z], dt_bias, initial_states, seq_idx, dt_softplus,
                         dt_limit)
         outs, finals, ws = _scan_fwd(prob, return_final_states)
+        # The caller's tensors go through save_for_backward (issm_combined.py:42 does the same): `prob` holds detached
+        # views of the same storage, and reading ctx.saved_tensors in backward is what makes PyTorch raise when one of
+        # them was modified in place between forward and backward instead of returning gradients of changed data.
+        ctx.save_for_backward(x, dt, A, B, C, D, z, dt_bias, initial_states)
         ctx.prob = prob
         ctx.ws = ws
         ctx.return_final_states = return_final_states
@@ -213,6 +217,7 @@ class ISSMChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *args):
+        ctx.saved_tensors  # version check of the inputs
         prob = ctx.prob
         x, dt, A, B, C, D, z, dt_bias, h0 = ctx.refs
         dfinal = args[0] if ctx.return_final_states else None
@@ -256,6 +261,7 @@ class ISSMBiScanFn(torch.autograd.Function):
         prob = _Problem([x_f, x_b], dt, A, [B_f, B_b], [C_f, C_b], chunk_size, D, [None, None], dt_bias,
                         initial_states, None, dt_softplus, dt_limit)
         outs, finals, ws = _scan_fwd(prob, True)
+        ctx.save_for_backward(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D, dt_bias, initial_states)  # see ISSMChunkScanCombinedFn
         ctx.prob = prob
         ctx.ws = ws
         ctx.refs = _dtypes(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D, dt_bias, initial_states)
@@ -264,6 +270,7 @@ class ISSMBiScanFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy_f, dy_b, dl_f, dl_b):
+        ctx.saved_tensors  # version check of the inputs
         prob = ctx.prob
         x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D, dt_bias, h0 = ctx.refs
         dxs, ddt, dA, dBs, dCs, dD, _, dbias, dh0 = _scan_bwd(prob, ctx.ws, [dy_f, dy_b], [dl_f, dl_b], want_dz=False)

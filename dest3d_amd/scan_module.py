@@ -37,13 +37,21 @@ class _LinearTokens(torch.autograd.Function):
     batched GEMM and the slices' results are summed (24 us)."""
 
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, x, w):
+        # under autocast F.linear runs in the autocast dtype; what is saved must be in that dtype too, or the
+        # backward's `dy @ w` would mix dtypes
+        if torch.is_autocast_enabled("cuda"):
+            adt = torch.get_autocast_dtype("cuda")
+            x, w = x.to(adt), w.to(adt)
         ctx.save_for_backward(x, w)
         return F.linear(x, w)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dy):
         x, w = ctx.saved_tensors
+        dy = dy.to(x.dtype)
         dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = dy @ w
@@ -132,9 +140,10 @@ class MultiHeadISSMScan(nn.Module):
         zxbcdt = _linear(self.key_proj, in_key)
         z, xbc, dt_tok = torch.split(zxbcdt, [self.d_inner, self.d_inner + 2 * G, H], dim=-1)
         if self.use_biscan:
-            # both convolutions read xbc once (dest_module.py:531,548)
+            # key_conv_back runs on key_conv's OUTPUT (dest_module.py:530 reassigns xbc before :534 uses it):
+            # one chained pass, xbc_b = silu(conv_back(silu(conv(xbc))))
             convs = (self.key_conv.dwconv, self.key_conv_back.dwconv)
-            xbc_f, xbc_b = dwconv_silu(xbc, [c.weight for c in convs], [c.bias for c in convs])
+            xbc_f, xbc_b = dwconv_silu(xbc, [c.weight for c in convs], [c.bias for c in convs], chain=True)
         else:
             xbc_f = self.key_conv(key_xyz, xbc)
         x, b_bias, c_bias = torch.split(xbc_f, [self.d_inner, G, G], dim=-1)

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define ISSM_ABI_VERSION 1
+#define ISSM_ABI_VERSION 2
 #define ISSM_CHUNK 64 /* tokens per internal chunk */
 
 typedef enum issm_status {
@@ -278,9 +278,11 @@ int issm_param_gen_bwd(const issm_pgen_args* args);
 /* ---- depthwise 7-tap convolution along the token order + SiLU -------------------------
  * PointLiteConv (models/dest_module.py:400-423): nn.Conv1d(C, C, 7, padding=3, groups=C) on
  * feature.transpose(1, 2), then SiLU, transposed back.  Here on (B, L, C) as it lies, for up to two
- * weight sets at once (MultiHeadISSMScan applies key_conv and key_conv_back to the same tensor,
- * dest_module.py:531,548):
- *   pre[s][b][l][c] = bias[s][c] + sum_j w[s][c][j] u[b][l+j-3][c]   (zero outside [0, L)),  y = silu(pre).
+ * weight sets in one pass:
+ *   pre[s][b][l][c] = bias[s][c] + sum_j w[s][c][j] in_s[b][l+j-3][c]   (zero outside [0, L)),  y[s] = silu(pre[s]).
+ * chain = 0: in_s = u for every set.  chain = 1 (nsets = 2): in_0 = u and in_1 = y[0] (as stored, i.e. rounded to
+ * `dtype`) -- MultiHeadISSMScan's pair: dest_module.py:530 reassigns xbc = key_conv(xbc), and :534 applies
+ * key_conv_back to that result, not to the key_proj output; du is then the gradient through both convolutions.
  * u: `dtype`, channels contiguous, element strides u_batch_stride / u_token_stride.  w (nsets, C, 7) and
  * bias (nsets, C): fp32 contiguous.  y and pre: (nsets, B, L, C) contiguous in `dtype`; pre is the
  * convolution output before SiLU, which the backward reads.  With 0 < split < C the output is written as two dense
@@ -311,6 +313,7 @@ typedef struct issm_dwconv_args {
   const void* dy_tail[2];
   /* element strides of du (0, 0 = contiguous (B, L, C)): lets the gradient land inside a wider row */
   int64_t du_batch_stride, du_token_stride;
+  int32_t chain; /* 1: set 1 convolves set 0's output (needs nsets = 2) */
 } issm_dwconv_args;
 
 int issm_dwconv_partial_rows(int32_t batch, int32_t seqlen);

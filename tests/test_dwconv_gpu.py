@@ -60,6 +60,68 @@ def test_dwconv_silu_matches_fp64(case):
         assert _rel(bs[s].grad, b64[s].grad) <= gtol
 
 
+CHAIN_CASES = [
+    # B, L, C, dtype, strided input
+    (2, 100, 290, torch.float32, True),
+    (3, 16, 64, torch.float32, False),
+    (2, 1, 8, torch.float32, False),
+    (1, 5, 33, torch.float32, False),
+    (1, 23, 40, torch.float32, False),
+    (2, 257, 290, torch.bfloat16, True),
+]
+
+
+@pytest.mark.parametrize("case", CHAIN_CASES, ids=lambda c: "B%d_L%d_C%d_%s_%s" % (*c[:3], str(c[3])[6:], "view" if c[4] else "dense"))
+def test_dwconv_chain_matches_fp64(case):
+    """chain=True: the second set convolves the first set's result (models/dest_module.py:530,534), forward and every
+    gradient -- du and the first set's weight gradient collect what flows back through the second convolution."""
+    from dest3d_amd.dwconv import dwconv_silu
+    B, L, C, dtype, strided = case
+    print(f"[case] dwconv chain B={B} L={L} C={C} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(91 + L + C)
+    full = torch.randn(B, L, C + 24, generator=g).to(dtype)
+    base = full.cuda().requires_grad_()
+    u = base[..., 8:8 + C] if strided else base[..., :C].contiguous()
+    ws = [(0.4 * torch.randn(C, 1, 7, generator=g)).cuda().requires_grad_() for _ in range(2)]
+    bs = [(0.2 * torch.randn(C, generator=g)).cuda().requires_grad_() for _ in range(2)]
+    ys = dwconv_silu(u, ws, bs, chain=True)
+    u64 = (full[..., 8:8 + C] if strided else full[..., :C]).double().requires_grad_()
+    w64 = [w.detach().double().cpu().requires_grad_() for w in ws]
+    b64 = [b.detach().double().cpu().requires_grad_() for b in bs]
+    r0 = _ref(u64, w64[:1], b64[:1])[0]
+    r1 = _ref(r0, w64[1:], b64[1:])[0]
+    ftol, gtol = (1e-5, 1e-4) if dtype == torch.float32 else (1.5e-2, 4e-2)
+    for y, r in zip(ys, (r0, r1)):
+        assert y.shape == (B, L, C) and y.dtype == dtype
+        assert _rel(y, r) <= ftol
+    gy = [torch.randn(B, L, C, generator=g).to(dtype) for _ in range(2)]
+    torch.autograd.backward(list(ys), [t.cuda() for t in gy])
+    torch.autograd.backward([r0, r1], [t.double() for t in gy])
+    got_du = base.grad[..., 8:8 + C] if strided else base.grad[..., :C]
+    assert _rel(got_du, u64.grad) <= gtol
+    for s in range(2):
+        assert _rel(ws[s].grad, w64[s].grad) <= gtol
+        assert _rel(bs[s].grad, b64[s].grad) <= gtol
+
+
+def test_dwconv_chain_only_second_gradient():
+    """Only the second output has a gradient: it still reaches u and the first set's parameters through the chain."""
+    from dest3d_amd.dwconv import dwconv_silu
+    g = torch.Generator().manual_seed(6)
+    u = torch.randn(2, 50, 40, generator=g).cuda().requires_grad_()
+    ws = [(0.4 * torch.randn(40, 7, generator=g)).cuda().requires_grad_() for _ in range(2)]
+    bs = [(0.2 * torch.randn(40, generator=g)).cuda().requires_grad_() for _ in range(2)]
+    _, y1 = dwconv_silu(u, ws, bs, chain=True)
+    y1.sum().backward()
+    u64 = u.detach().double().cpu().requires_grad_()
+    w64 = [w.detach().double().cpu().requires_grad_() for w in ws]
+    b64 = [b.detach().double().cpu().requires_grad_() for b in bs]
+    r1 = _ref(_ref(u64, w64[:1], b64[:1])[0], w64[1:], b64[1:])[0]
+    r1.sum().backward()
+    assert _rel(u.grad, u64.grad) <= 1e-4
+    assert _rel(ws[0].grad, w64[0].grad.reshape(40, 7)) <= 1e-4 and _rel(bs[0].grad, b64[0].grad) <= 1e-4
+
+
 def test_dwconv_one_absent_gradient():
     from dest3d_amd.dwconv import dwconv_silu
     g = torch.Generator().manual_seed(5)
@@ -86,6 +148,8 @@ def test_dwconv_rejects_unbuilt_shapes():
     assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -5
     a.nsets = 1
     assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -1
+    a.chain = 1                               # a chain needs two sets
+    assert lib.issm_dwconv_silu_fwd(C.byref(a)) == -2
 
 
 def test_dwconv_split_outputs_equal_the_slices():

@@ -258,6 +258,29 @@ def test_stage_entry_points_match_oracle_intermediates():
         _check(name, t, ref[k], BWD32)
 
 
+def test_inplace_edit_between_forward_and_backward_raises():
+    """The operator saves its inputs for the backward as the reference does (issm_combined.py:42): changing one of them
+    in place before backward must raise PyTorch's version-counter error, not return gradients of other data."""
+    from dest3d_amd import ISSM_chunk_scan_combined
+    from dest3d_amd.issm_combined import ISSM_biscan_combined
+    print("[case] in-place edit of a saved input", flush=True)
+    I = R.make_inputs(1, 70, 2, 16, 32, G=1, seed=3)
+    for name in ("x", "dt_raw", "B", "C"):
+        g = {k: I[k].cuda().requires_grad_() for k in ("x", "dt_raw", "A", "B", "C")}
+        w = {k: v * 1.0 for k, v in g.items()}              # non-leaf copies that may be edited in place
+        y = ISSM_chunk_scan_combined(w["x"], w["dt_raw"], w["A"], w["B"], w["C"], 64, dt_softplus=True)
+        w[name].mul_(2.0)
+        with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+            y.sum().backward()
+    g = {k: I[k].cuda().requires_grad_() for k in ("x", "dt_raw", "A", "B", "C")}
+    w = {k: v * 1.0 for k, v in g.items()}
+    yf, yb, _, _ = ISSM_biscan_combined(w["x"], w["x"], w["dt_raw"], w["A"], w["B"], w["B"], w["C"], w["C"], 64,
+                                        dt_softplus=True)
+    w["dt_raw"].add_(1.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        (yf.sum() + yb.sum()).backward()
+
+
 def test_error_codes_do_not_abort():
     from dest3d_amd import _lib as L
     _say("error codes")

@@ -5,9 +5,6 @@ import sys
 
 import pytest
 import torch
-import torch.nn.functional as F
-
-from oracle import issm_ref as R
 
 pytestmark = pytest.mark.gpu
 FWD32, BWD32, FWD16 = 1e-4, 1e-3, 2e-2
@@ -27,46 +24,10 @@ def _check(name, a, b, tol):
 
 
 def _module_ref(sd, cfg, in_key, in_query, dist, mask):
-    """dest_module.py:528-585 in the reference's own order of operations (transposed views, flipped
-    copies, two scans), in fp64, with the scan and the gated norm taken from the oracle."""
-    H, G, d_inner = cfg["nheads"], cfg["ngroups"], cfg["d_inner"]
-    P, K = d_inner // H, cfg["d_state"]
-
-    def conv(prefix, t):
-        w, b = sd[prefix + ".dwconv.weight"], sd[prefix + ".dwconv.bias"]
-        return F.silu(F.conv1d(t.transpose(1, 2), w, b, padding=3, groups=w.shape[0])).transpose(1, 2)
-
-    zxbcdt = in_key @ sd["key_proj.weight"].T
-    z, xbc, dt_tok = torch.split(zxbcdt, [d_inner, d_inner + 2 * G, H], dim=-1)
-    x, b_bias, c_bias = torch.split(conv("key_conv", xbc), [d_inner, G, G], dim=-1)
-    h0 = (in_query @ sd["query_proj.weight"].T).reshape(in_query.shape[0], K, H, P).permute(0, 2, 3, 1)
-    A = (-torch.exp(sd["A_log"]))[:, None].expand(H, K)
-    bc = dist @ sd["bc_proj.weight"].T
-    b_base, c_base = torch.split(bc, [G, G], dim=-1)
-    Bm = b_base.transpose(-1, -2) + b_bias.unsqueeze(-1)
-    Cm = c_base.transpose(-1, -2) + c_bias.unsqueeze(-1)
-    dt = F.softplus((dist @ sd["dt_proj.weight"].T).transpose(-1, -2) + dt_tok.unsqueeze(-1)
-                    + sd["dt_bias"].reshape(1, 1, -1, 1))
-    if mask is not None:
-        if mask.dtype == torch.bool:
-            dt = dt.masked_fill(mask.unsqueeze(2), 0.0)
-        else:
-            dt = dt * mask.unsqueeze(2).double()
-    hp = lambda t: t.reshape(*t.shape[:2], H, P)
-    scan = lambda x_, dt_, B_, C_: R.issm_scan_sequential(hp(x_), dt_, A, B_, C_, D=sd["D"], initial_states=h0)
-    key, last = scan(x, dt, Bm, Cm)
-    if cfg["use_biscan"]:
-        x_b, bb, cb = torch.split(conv("key_conv_back", xbc), [d_inner, G, G], dim=-1)
-        fl = lambda t: torch.flip(t, dims=[1])
-        key_b, last_b = scan(fl(x_b), fl(dt), fl(b_base.transpose(-1, -2) + bb.unsqueeze(-1)),
-                             fl(c_base.transpose(-1, -2) + cb.unsqueeze(-1)))
-        key = (key + fl(key_b)) / 2
-        last = (last + last_b) / 2
-    key = R.gated_rmsnorm_ref(key.flatten(-2), sd["key_norm.weight"], z=z, eps=1e-5, norm_before_gate=False)
-    out_key = key @ sd["out_key_proj.weight"].T
-    last = last.permute(0, 3, 1, 2).flatten(-2)
-    last = F.layer_norm(last, (d_inner,), sd["query_norm.weight"], sd["query_norm.bias"], 1e-5)
-    return out_key, last @ sd["out_query_proj.weight"].T
+    """dest_module.py:528-585 in the reference's own order of operations (oracle/module_ref.py; the order of the two
+    convolutions is pinned in tests/test_module_cpu.py)."""
+    from oracle.module_ref import multi_head_issm_scan_ref
+    return multi_head_issm_scan_ref(sd, cfg, in_key, in_query, dist, mask)
 
 
 @pytest.mark.parametrize("biscan,mask_kind", [(True, None), (True, "float"), (True, "bool"), (False, "bool"), (False, "float")])
@@ -108,6 +69,25 @@ def test_module_matches_fp64_evaluation(biscan, mask_kind):
         _check("d" + k, gin[k].grad, rin[k].grad, BWD32)
     for k, p in m.named_parameters():
         _check("d" + k, p.grad, sd[k].grad, BWD32)
+
+
+def test_token_linear_under_autocast():
+    """The projections' autograd node under torch.autocast: forward in bf16, and the backward's products see operands
+    of one dtype (fp32 parameters and input, bf16 output gradient)."""
+    from dest3d_amd.scan_module import _LinearTokens
+    print("[case] _LinearTokens under autocast", flush=True)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2048, 72, generator=g).cuda().requires_grad_()
+    w = (0.1 * torch.randn(40, 72, generator=g)).cuda().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = _LinearTokens.apply(x, w)
+        assert y.dtype == torch.bfloat16
+        y.float().square().mean().backward()
+    x64, w64 = x.detach().double().cpu().requires_grad_(), w.detach().double().cpu().requires_grad_()
+    (x64 @ w64.T).square().mean().backward()
+    assert x.grad.dtype == torch.float32 and w.grad.dtype == torch.float32
+    _check("dx", x.grad, x64.grad, 3e-2)
+    _check("dw", w.grad, w64.grad, 3e-2)
 
 
 def test_six_layer_stack_bf16_at_detector_shape():

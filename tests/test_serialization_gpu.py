@@ -21,6 +21,26 @@ def test_codes_match_oracle(order, bit):
     assert (code == R.hilbert_distance(g, bit)).all()
 
 
+def test_points_on_cell_boundaries_land_where_the_host_division_puts_them():
+    """Points whose offset from the sample minimum is the float nearest to k * cell: the quotient is then within an
+    ulp of the integer k, and whether trunc gives k or k - 1 depends on the division being correctly rounded.  The
+    kernel must agree with torch.div(..., rounding_mode="trunc") on the CPU for every one of them
+    (models/dest_module.py:326-329)."""
+    from dest3d_amd.serialization import hilbert_codes
+    cell = np.float32(1.0 / 50.0)
+    k = np.arange(512, dtype=np.float32)
+    pts = np.zeros((1, 3 * 512 + 1, 3), np.float32)           # row 0 stays at the origin: the sample minimum
+    for ax in range(3):
+        pts[0, 1 + ax * 512:1 + (ax + 1) * 512, ax] = k * cell
+    t = torch.from_numpy(pts)
+    want_grid = torch.div(t - t.min(1, keepdim=True)[0], float(cell), rounding_mode="trunc").long().clamp_max(511).numpy()
+    assert (R.grid_coords(pts, 9) == want_grid).all()        # the oracle is the host division
+    code = hilbert_codes(t.cuda(), "xyz", 9).cpu().numpy()
+    assert (code == R.hilbert_distance(want_grid, 9)).all()
+    # the case is not vacuous: some quotients do fall short of their integer
+    assert (want_grid[0, 1:513, 0] != np.arange(512)).any()
+
+
 def test_whole_cube_is_a_unit_step_walk():
     from dest3d_amd.serialization import Serialization
     s = Serialization(order=["xyz"], bit=4)
