@@ -24,6 +24,7 @@ EXPORTS = [
     "issm_stage_chunk_scan", "issm_stage_bwd_gate", "issm_stage_bwd_dstates",
     "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_stage_bwd_dx", "issm_stage_bwd_reduce",
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
+    "issm_gated_rmsnorm_bwd_noalloc",
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
     "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
@@ -174,6 +175,7 @@ def load() -> C.CDLL:
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]
     lib.issm_gated_rmsnorm_fwd.argtypes = [P(NormArgs)]
     lib.issm_gated_rmsnorm_bwd.argtypes = [P(NormArgs)]
+    lib.issm_gated_rmsnorm_bwd_noalloc.argtypes = [P(NormArgs)]
     lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
     lib.issm_hilbert_codes.argtypes = [P(HilbertArgs)]
     lib.issm_transpose_states.argtypes = [P(TransposeArgs)]

@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "../../include/issm.h"
 #include "issm_dev.h"
 
@@ -430,6 +432,61 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* a) {
   int rc = norm_params(a, &p, true);
   if (rc) return rc;
   return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd");
+}
+
+}  // extern "C"
+
+// ---- the same backward on a scratch buffer that belongs to the library: no allocation by anyone
+// The per-block partial sums of dw (nblocks x ncols floats) normally arrive as args->dw_partial.  For callers that
+// cannot allocate, they go into this array instead; every GPU the library runs on holds its own copy (8 MiB) at
+// its own address until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and kept, and it is that pointer -- never
+// the name -- that the kernels receive.  (No `used` attribute on the array: the compiler gives a file-scope device
+// variable that host code refers to an external symbol, which is what the runtime's lookup needs; `used` keeps it local
+// and the lookup then aborts the process.)
+static __device__ __align__(256) float g_norm_scratch[ISSM_NORM_SCRATCH_FLOATS];
+static constexpr int kMaxDevices = 64;
+static std::mutex g_norm_scratch_mutex;
+static float* g_norm_scratch_ptr[kMaxDevices];  // [device]: address of that device's copy, once looked up
+
+static int norm_scratch_ptr(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(ISSM_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(ISSM_E_UNSUPPORTED, "device index %d outside 0..%d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_norm_scratch_mutex);
+  if (!g_norm_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_norm_scratch));  // of the current device's copy
+    if (e != hipSuccess || !ptr)
+      return fail(ISSM_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_norm_scratch_ptr[dev] = (float*)ptr;
+  }
+  *out = g_norm_scratch_ptr[dev];
+  return ISSM_OK;
+}
+
+extern "C" {
+
+int issm_gated_rmsnorm_bwd_noalloc(const issm_norm_args* a) {
+  if (!a) return fail(ISSM_E_NULL, "args is NULL");
+  issm_norm_args b = *a;
+  float* scratch = nullptr;
+  // sizes are checked before anything touches the device
+  if (b.rows > 0 && b.ncols > 0 &&
+      (int64_t)issm_rmsnorm_bwd_blocks(b.rows) * b.ncols > (int64_t)ISSM_NORM_SCRATCH_FLOATS)
+    return fail(ISSM_E_WORKSPACE,
+                "rmsnorm bwd without allocation: %d row blocks x %d columns = %lld floats of partial sums exceed the "
+                "library's %d-float scratch array; use issm_gated_rmsnorm_bwd with a dw_partial buffer",
+                issm_rmsnorm_bwd_blocks(b.rows), b.ncols, (long long)issm_rmsnorm_bwd_blocks(b.rows) * b.ncols,
+                (int)ISSM_NORM_SCRATCH_FLOATS);
+  b.dw_partial = (float*)(uintptr_t)256;  // placeholder so that the shared validation sees a buffer; replaced below
+  NormP p;
+  int rc = norm_params(&b, &p, true);
+  if (rc) return rc;
+  if ((rc = norm_scratch_ptr(&scratch))) return rc;
+  p.dw_partial = scratch;  // every launched block writes its whole row of partials before the sum reads it
+  return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd_noalloc");
 }
 
 static int pgen_params(const issm_pgen_args* a, PGenP* p, bool bwd) {

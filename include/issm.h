@@ -232,6 +232,18 @@ int issm_rmsnorm_bwd_blocks(int64_t rows);
 int issm_gated_rmsnorm_fwd(const issm_norm_args* args);
 int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
 
+/* issm_gated_rmsnorm_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and the same
+ * results, bit for bit, as issm_gated_rmsnorm_bwd, except that args->dw_partial is ignored: the per-block partial
+ * sums of dw go into a scratch array inside the library (ISSM_NORM_SCRATCH_FLOATS floats = 8 MiB per GPU the library
+ * runs on, held until the process ends).  Problems with issm_rmsnorm_bwd_blocks(rows) * ncols >
+ * ISSM_NORM_SCRATCH_FLOATS return ISSM_E_WORKSPACE (rows of up to 1024 columns always fit).  The function calls no
+ * hipMalloc / hipFree or other allocating routine.  All calls on one GPU share that GPU's array: two calls that
+ * overlap in time on one GPU (different streams or host threads) race; calls on one stream are ordered and safe.
+ * Nothing in the array has to be cleared between calls (every partial that is read was written by the same call). */
+#define ISSM_NORM_SCRATCH_FLOATS (2048 * 1024)
+int issm_gated_rmsnorm_bwd_noalloc(const issm_norm_args* args);
+
 /* ---- generation of the scan parameters from the distance encoding -------------------
  * Replaces the bc_proj / dt_proj Linear layers, their transposes and the broadcast bias
  * additions of MultiHeadISSMScan.forward (models/dest_module.py:541-553) by one pass:
