@@ -261,8 +261,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 // loop is issued on every path, so the compiler can count the loads still in flight and the prefetched operands of
 // the next chunks stay in flight across the barrier (with loads inside branches it waits for all of them before each
 // store, which exposes the full memory latency once per chunk; few workgroups walking many chunks -- batch 2, 256
-// chunks -- then run at that pace).  A thread owns KM rows, pg + PGN k; rows past the head dimension are replaced by
-// its last row: those threads compute and store exactly what the row's owner does, and stay out of the column sums.
+// chunks -- then run at that pace).  A thread owns KM rows, pg + PGN k; for rows past the head dimension it stands in
+// for the head's last row: it issues the same loads (so that every load of the loop is unconditional) but stores
+// nothing and adds nothing to the column sums -- what a stand-in computes is never used, so it does not matter that
+// the row's owner overwrites dH with dS while the stand-in's prefetches of that row are in flight.
 template <int NQ, int KM, int R>
 __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* __restrict__ states,
                                                              const float* __restrict__ cs_last,
@@ -281,11 +283,11 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   const int tid = threadIdx.x, pg = tid / NQ, nq = tid % NQ;
   const int n = ns * NCOL + nq * 4;
   long rowk[KM];   // offsets of the thread's rows
-  float own[KM];   // 1 for a row of its own, 0 for a stand-in
+  bool own[KM];    // a row of its own (stores, takes part in the column sums) or a stand-in (loads only)
 #pragma unroll
   for (int k = 0; k < KM; ++k) {
     rowk[k] = (long)min(pg + PGN * k, p.P - 1) * p.N + n;
-    own[k] = pg + PGN * k < p.P ? 1.0f : 0.0f;
+    own[k] = pg + PGN * k < p.P;
   }
   const long cstep = (long)p.H * p.P * p.N, vstep = (long)p.H * p.N;  // from chunk to chunk
   f4 carry[KM];
@@ -320,10 +322,10 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     for (int j = 0; j < 4; ++j) e[j] = __expf(dec[cur][j]);
 #pragma unroll
     for (int k = 0; k < KM; ++k) {
-      *(f4*)(dd + rowk[k]) = carry[k];
+      if (own[k]) *(f4*)(dd + rowk[k]) = carry[k];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        gp[j] += own[k] * hn[cur][k][j] * carry[k][j];
+        gp[j] += own[k] ? hn[cur][k][j] * carry[k][j] : 0.0f;
         carry[k][j] = e[j] * carry[k][j] + dh[cur][k][j];
       }
     }
@@ -353,7 +355,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
     if (c - i >= 0) step(i, (i + R - 1) % R, c - i);  // uniform: the last nc % R chunks
 #pragma unroll
   for (int k = 0; k < KM; ++k)
-    *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + rowk[k]) = carry[k];
+    if (own[k]) *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + rowk[k]) = carry[k];
 }
 
 // -------------------------------------------------------------- chunk backward
