@@ -200,6 +200,8 @@ static KP make_kp(const issm_scan_args* a) {
   p.io_dt = a->io_dtype; p.dt_dt = a->dt_dtype; p.h0_dt = a->h0_dtype;
   p.flags = ((a->flags & ISSM_FLAG_DT_SOFTPLUS) ? F_SOFTPLUS : 0u) | ((a->flags & ISSM_FLAG_D_HAS_HDIM) ? F_D_HDIM : 0u);
   p.dt_min = a->dt_min; p.dt_max = a->dt_max;
+  // softplus is positive: limits of (<= 0, >= 3e38 or inf) cannot act on it
+  if ((p.flags & F_SOFTPLUS) && a->dt_min <= 0.0f && a->dt_max >= 3.0e38f) p.flags |= F_NOCLAMP;
   for (int i = 0; i < 2; ++i) {
     p.x[i] = td(a->x[i]); p.Bm[i] = td(a->Bm[i]); p.Cm[i] = td(a->Cm[i]); p.z[i] = td(a->z[i]);
     p.out[i] = td(a->out[i]); p.dout[i] = td(a->dout[i]); p.dx[i] = td(a->dx[i]); p.dB[i] = td(a->dB[i]);

@@ -96,10 +96,27 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
       f4 acc = {0, 0, 0, 0};
 #pragma unroll
       for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
+      if (IOB) {
+        // bf16 inputs: the block goes out as two bf16 copies in the same 16 KB, dM[l][s] at [l][s] of the first half
+        // and at [s][l] of the second, which is what k_bwd_chunk_bf's matrix operands read (blocks above the diagonal
+        // are not written and never read)
+        uint16_t* mb = reinterpret_cast<uint16_t*>(m);
+        const int sc = j * 16 + cm, l0 = wave * 16 + 4 * g4;
+        float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int l = wave * 16 + 4 * g4 + r, sc = j * 16 + cm;
-        m[l * CS + sc] = sc <= l ? acc[r] : 0.0f;
+        for (int r = 0; r < 4; ++r) v[r] = sc <= l0 + r ? acc[r] : 0.0f;
+        const unsigned w0 = pack_bf16(v[0], v[1]), w1 = pack_bf16(v[2], v[3]);
+        mb[(l0 + 0) * CS + sc] = (uint16_t)w0;
+        mb[(l0 + 1) * CS + sc] = (uint16_t)(w0 >> 16);
+        mb[(l0 + 2) * CS + sc] = (uint16_t)w1;
+        mb[(l0 + 3) * CS + sc] = (uint16_t)(w1 >> 16);
+        *(uint2*)(mb + CS * CS + sc * CS + l0) = make_uint2(w0, w1);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int l = wave * 16 + 4 * g4 + r, sc = j * 16 + cm;
+          m[l * CS + sc] = sc <= l ? acc[r] : 0.0f;
+        }
       }
     }
   }
@@ -794,6 +811,404 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   }
 }
 
+// ------------------------------------------------- chunk backward, bf16 inputs
+// The same computation for bf16 x / B / C / dy: every matrix product runs on v_mfma_f32_16x16x32_bf16 with operands
+// rounded once to bf16 (the reference casts its dot operands to the input dtype as well, issm_cabt_bmm.py:42-43;
+// running sums, decays, states and all accumulation stay fp32).  x and dy are bf16 already, so their tiles are exact;
+// dM arrives from k_bwd_dstates as two bf16 copies, row-major and transposed, because the F sums contract over the
+// columns of dM and the G sums over its rows, and a lane's operand must be contiguous in LDS.
+template <int PT>
+struct BwdChunkBfSmem {
+  static constexpr int KW = 16 * PT, LDP = KW + 8;  // x / dy tiles [l][p]
+  static constexpr int LDM = CS + 8;                // dM tiles [row][col]
+  uint16_t xs[CS * LDP], dys[CS * LDP];
+  uint16_t dmr[CS * LDM];  // dM[l][s]
+  uint16_t dmt[CS * LDM];  // dM[s][l] stored at [l][s]: the transpose
+  float dbc[32 * NTHREADS];
+};
+
+__device__ __forceinline__ bf8 pack_bf8(const float (&v)[8]) {
+  bf8 r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (__bf16)v[j];
+  return r;
+}
+// four values in k-slots 0..3, zeros in 4..7
+__device__ __forceinline__ bf8 pack_bf4_lo(float a, float b, float c, float d) {
+  bf8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+  r[0] = (__bf16)a; r[1] = (__bf16)b; r[2] = (__bf16)c; r[3] = (__bf16)d;
+  return r;
+}
+__device__ __forceinline__ bf8 frag4_lo(const uint16_t* q, bool keep = true) {
+  uint2 w = *(const uint2*)q;
+  if (!keep) w = make_uint2(0u, 0u);
+  const bf4 a = __builtin_bit_cast(bf4, w);
+  const bf4 z = {0, 0, 0, 0};
+  return __builtin_shufflevector(a, z, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <int LDM, int LV>
+__device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+                                                 const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
+                                                 float (&e1)[16], float (&x2)[16], int cm, int g4) {
+  float op[16], ee[16];
+  const float ref_a = __shfl(LV == 4 ? cs[3] : cs[7], cm + 48, 64);
+  const float ref_b = LV == 4 ? __shfl(cs[11], cm + 48, 64) : ref_a;
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    const float ref = (J & 2) ? ref_b : ref_a;
+    const bool upper = LV == 4 ? (J & 1) : (J & 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * J + j;
+      const float e = ex2(upper ? cs[k] - ref : ref - cs[k]);
+      ee[k] = e;
+      op[k] = (upper ? Cv[k] : Bv[k] * dtp[k]) * e;
+    }
+  }
+  if (LV == 5) {
+    float lo8[8], hi8[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { lo8[j] = op[j]; hi8[j] = op[8 + j]; }
+    const bf8 blo = pack_bf8(lo8), bhi = pack_bf8(hi8);
+    // all four operand fragments first, then the products
+    const bf8 a2 = split_frag<LDM>(dmr, 32 + cm, g4, 0), a3 = split_frag<LDM>(dmr, 48 + cm, g4, 0);
+    const bf8 a0 = split_frag<LDM>(dmt, cm, g4, 1), a1 = split_frag<LDM>(dmt, 16 + cm, g4, 1);
+    const f4 z = {0, 0, 0, 0};
+    const f4 f2 = mfma_bf(a2, blo, z), f3 = mfma_bf(a3, blo, z);   // F: rows of tiles 2, 3 gather from tiles 0, 1
+    const f4 g0 = mfma_bf(a0, bhi, z), g1 = mfma_bf(a1, bhi, z);   // G: rows of tiles 0, 1 gather from tiles 2, 3
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      e1[rr] += ee[rr] * g0[rr];
+      e1[4 + rr] += ee[4 + rr] * g1[rr];
+      x2[8 + rr] += ee[8 + rr] * f2[rr];
+      x2[12 + rr] += ee[12 + rr] * f3[rr];
+    }
+  } else {
+    bf8 a[4], b[4];
+#pragma unroll
+    for (int I = 0; I < 4; ++I) {
+      const int K = (I & 1) ? I - 1 : I + 1;  // the tile contracted over
+      a[I] = frag4_lo(((I & 1) ? dmr : dmt) + (I * 16 + cm) * LDM + K * 16 + 4 * g4);
+      b[I] = pack_bf4_lo(op[4 * K], op[4 * K + 1], op[4 * K + 2], op[4 * K + 3]);
+    }
+    const f4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int I = 0; I < 4; ++I) {
+      const f4 acc = mfma_bf(a[I], b[I], z);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        if (I & 1) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+        else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+      }
+    }
+  }
+}
+
+template <int LDM, int LV>
+__device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+                                                 const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
+                                                 float (&e1)[16], float (&x2)[16], int cm, int g4) {
+  const bool up = LV == 2 ? (g4 & 1) : (g4 & 2);  // role of the lane's rows 4 g4 + j
+  const float upf = up ? 1.0f : 0.0f, lof = up ? 0.0f : 1.0f, sg = up ? 1.0f : -1.0f;
+  // A operand: row i = cm of T_w (see bwd_mid_level), columns 4 g4 + jj; non-zero only where (i, kk) is a level-w pair
+  const int cg = cm >> 2;
+  const bool iup = LV == 2 ? (cg & 1) : (cg & 2);
+  const bool nz = LV == 2 ? (g4 == (cg ^ 1)) : ((g4 >> 1) != (cg >> 1));
+  const uint16_t* abase = (iup ? dmr : dmt) + cm * LDM + 4 * g4;
+  float op[16], ee[16], refs[4];
+#pragma unroll
+  for (int J = 0; J < 4; ++J)
+    refs[J] = LV == 2 ? __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64) : __shfl(cs[4 * J + 3], cm + 16, 64);
+  bf8 a[4];
+#pragma unroll
+  for (int I = 0; I < 4; ++I) a[I] = frag4_lo(abase + I * (16 * LDM + 16), nz);
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const float e = ex2(sg * (cs[k] - refs[k >> 2]));
+    ee[k] = e;
+    op[k] = (up ? Cv[k] : Bv[k] * dtp[k]) * e;
+  }
+  const f4 z = {0, 0, 0, 0};
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    const f4 acc = mfma_bf(a[I], pack_bf4_lo(op[4 * I], op[4 * I + 1], op[4 * I + 2], op[4 * I + 3]), z);
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const float v = ee[4 * I + rr] * acc[rr];
+      x2[4 * I + rr] = fmaf(v, upf, x2[4 * I + rr]);
+      e1[4 * I + rr] = fmaf(v, lof, e1[4 * I + rr]);
+    }
+  }
+}
+
+template <int LDM>
+__device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+                                                    const uint16_t* __restrict__ dmr, float (&e1)[16], float (&x2)[16],
+                                                    int g4) {
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    const uint16_t* blk = dmr + (16 * J + 4 * g4) * LDM + 16 * J + 4 * g4;  // dM[row jl][col js] of the group
+    uint2 m[4];
+#pragma unroll
+    for (int jl = 0; jl < 4; ++jl) m[jl] = *(const uint2*)(blk + jl * LDM);
+    float Bd[4];
+#pragma unroll
+    for (int jl = 0; jl < 4; ++jl) Bd[jl] = Bv[4 * J + jl] * dtp[4 * J + jl];
+    auto at = [&](int jl, int js) {
+      const unsigned w = js < 2 ? m[jl].x : m[jl].y;
+      return __uint_as_float((js & 1) ? (w & 0xffff0000u) : (w << 16));
+    };
+#pragma unroll
+    for (int jl = 0; jl < 4; ++jl) {
+      const int kl = 4 * J + jl;
+      const float d = at(jl, jl);
+      e1[kl] = fmaf(d, Cv[kl], e1[kl]);
+      x2[kl] = fmaf(d, Bd[jl], x2[kl]);
+#pragma unroll
+      for (int js = 0; js < jl; ++js) {
+        const int ks = 4 * J + js;
+        const float wgt = at(jl, js) * ex2(cs[kl] - cs[ks]);
+        e1[ks] = fmaf(wgt, Cv[kl], e1[ks]);
+        x2[kl] = fmaf(wgt, Bd[js], x2[kl]);
+      }
+    }
+  }
+}
+
+// a (64 x 16 PT) register tile (layout of lp_load) as bf16 into LDS dst[l][p]
+template <int PT, int LD>
+__device__ __forceinline__ void lp_store_bf(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* dst, int tid) {
+  constexpr int G4 = 4 * PT;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS;
+    *(uint2*)(dst + (e4 / G4) * LD + (e4 % G4) * 4) =
+        make_uint2(pack_bf16(v[4 * i], v[4 * i + 1]), pack_bf16(v[4 * i + 2], v[4 * i + 3]));
+  }
+}
+
+template <int PT, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws,
+                                                              const float* __restrict__ states,
+                                                              const float* __restrict__ dstates,
+                                                              const float* __restrict__ dm,
+                                                              const float* __restrict__ g_last,
+                                                              float* __restrict__ partA, float* __restrict__ partBias) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  typedef BwdChunkBfSmem<PT> SM;
+  SM& s = *reinterpret_cast<SM*>(smem_raw);
+  constexpr int LDP = SM::LDP, LDM = SM::LDM, KT = (PT + 1) / 2;
+  constexpr int KP_ = PT * 4;  // dS / H values per lane
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cm = lane & 15, g4 = lane >> 4;
+  const int nsl = (p.N + NS - 1) / NS;
+  Unit u;
+  int id = xcd_remap(blockIdx.x, gridDim.x);
+  const int ns = id % nsl;
+  id /= nsl;
+  u.g = id % p.G;
+  id /= p.G;
+  u.c = id % p.nc;
+  u.b = id / p.nc;
+  u.dir = p.dir0;
+  u.bt = u.b * p.ndir + u.dir;
+  u.h = u.g * p.hpg;
+  const int n = ns * NS + wave * 16 + cm;
+  const bool vn = FULL || n < p.N;
+  const RowMap rm = make_rowmap<FULL>(p, u, g4, ns * NS);
+  const int lim = vn ? rm.nvalid - 4 * g4 : 0;
+  auto rowk = [&](int k) { return 16 * (k >> 2) + (k & 3); };
+  const bool pn_full = FULL && p.P == PT * 16;
+
+  float Bv[16], Cv[16];
+  lane_load_ln<true>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, Bv);
+  lane_load_ln<true>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, Cv);
+#pragma unroll
+  for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
+
+  for (int hh = 0; hh < p.hpg; ++hh) {
+    // the reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
+    // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first
+    u.h = u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh);
+    // ---- global loads of this head
+    float raw[16], dsv[KP_], hv[KP_];
+    lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+    const Coef cf = lane_coef(p, u.h, n, vn);
+    const float gl = (g4 == 3 && vn) ? g_last[vec_off(p, u.bt, u.c, u.h) + n] : 0.0f;
+    lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
+    lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
+    {
+      float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
+      int tq = tid;
+      asm volatile("" : "+v"(tq));
+      dy_load<true, PT, FULL>(p, u, dy_ws, dv, tq);
+      lp_load<true, PT, FULL>(p, u, p.x[u.dir], xv, tq);
+      // both bf16 copies of dM: 2 x (64 x 64) halves, 16 bytes per access
+      const uint16_t* dmb = reinterpret_cast<const uint16_t*>(dm + sq_off(p, u.bt, u.c, u.h));
+      // (thread tq: row tq >> 3 and row 32 + (tq >> 3), columns 8 (tq & 7) .. + 7 of either copy)
+      const int mrow = tq >> 3, mcol = (tq & 7) * 8;
+      const uint4 mr0 = *(const uint4*)(dmb + mrow * CS + mcol), mr1 = *(const uint4*)(dmb + (32 + mrow) * CS + mcol);
+      const uint4 mt0 = *(const uint4*)(dmb + CS * CS + mrow * CS + mcol);
+      const uint4 mt1 = *(const uint4*)(dmb + CS * CS + (32 + mrow) * CS + mcol);
+      __syncthreads();  // the previous head no longer reads the LDS tiles
+      lp_store_bf<PT, LDP>(dv, s.dys, tq);
+      lp_store_bf<PT, LDP>(xv, s.xs, tq);
+      *(uint4*)(s.dmr + mrow * LDM + mcol) = mr0;
+      *(uint4*)(s.dmr + (32 + mrow) * LDM + mcol) = mr1;
+      *(uint4*)(s.dmt + mrow * LDM + mcol) = mt0;
+      *(uint4*)(s.dmt + (32 + mrow) * LDM + mcol) = mt1;
+    }
+    __syncthreads();
+
+    const float An = cf.A;
+    float dtp[16], cs[16], dfac[16];
+    const float last = lane_prep<true>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dfac);
+    pin16(cs);
+
+    int cq = cm, gq = g4;
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    float e1[16], x2[16];
+    {
+      // Q = x . dS and R = dy . H over the head dimension, K = 32 per step; k-slot s of step t <-> lane value 8 t + s.
+      // x and dy are exact in bf16; dS and H are fp32 states and enter as (hi, lo) pairs -- two instructions per step:
+      // the last row's Bd . E1 cancels against the state term g = sum_p dS H_next in d/d(cs), and a dS rounded to 8
+      // bits would leave that difference with a relative error far above the bf16 level.
+      bf8 dsh[KT], dsl[KT], hh_[KT], hl_[KT];
+#pragma unroll
+      for (int t = 0; t < KT; ++t) {
+        float a[8], b[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          a[j] = 8 * t + j < KP_ ? dsv[(8 * t + j) % KP_] : 0.0f;
+          b[j] = 8 * t + j < KP_ ? hv[(8 * t + j) % KP_] : 0.0f;
+        }
+        split8(a, dsh[t], dsl[t]);
+        split8(b, hh_[t], hl_[t]);
+      }
+#pragma unroll
+      for (int I = 0; I < 4; ++I) {
+        f4 q = {0, 0, 0, 0}, r = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+          const bool half = (PT & 1) && t == KT - 1;
+          const bf8 xf = half ? split_frag<LDP, true>(s.xs, I * 16 + cq, gq, t) : split_frag<LDP>(s.xs, I * 16 + cq, gq, t);
+          const bf8 yf = half ? split_frag<LDP, true>(s.dys, I * 16 + cq, gq, t) : split_frag<LDP>(s.dys, I * 16 + cq, gq, t);
+          q = mfma_bf(xf, dsl[t], q);
+          r = mfma_bf(yf, hl_[t], r);
+          q = mfma_bf(xf, dsh[t], q);
+          r = mfma_bf(yf, hh_[t], r);
+        }
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          e1[4 * I + rr] = ex2(last - cs[4 * I + rr]) * q[rr];
+          x2[4 * I + rr] = ex2(cs[4 * I + rr]) * r[rr];
+        }
+      }
+    }
+
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 5>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 4>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 3>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    // the second direction adds to the first one's ddt: fetch it while the last levels run
+    float old[16];
+    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
+    __builtin_amdgcn_sched_barrier(0);
+    bwd_small_levels_bf<LDM>(cs, Bv, dtp, Cv, s.dmr, e1, x2, gq);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- column phase (as in k_bwd_chunk)
+    pin16(e1); pin16(x2);
+    float dcs[16], val[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float E1 = e1[k], X2 = x2[k];
+      s.dbc[k * NTHREADS + tid] += dtp[k] * E1;
+      s.dbc[(16 + k) * NTHREADS + tid] += X2;
+      val[k] = Bv[k] * E1;
+      dcs[k] = Cv[k] * X2 - Bv[k] * dtp[k] * E1;
+    }
+    dcs[15] += gl;
+    {
+      float c[4], v[4], t[4];
+#pragma unroll
+      for (int J = 3; J >= 0; --J) {
+        float a = 0.0f;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+          a += dcs[4 * J + j];
+          dcs[4 * J + j] = a;
+        }
+        c[J] = a;
+      }
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl_down(c[J], 16, 64);
+#pragma unroll
+      for (int J = 0; J < 4; ++J) v[J] = g4 <= 2 ? c[J] + t[J] : c[J];
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl_down(v[J], 32, 64);
+#pragma unroll
+      for (int J = 0; J < 4; ++J) v[J] = g4 <= 1 ? v[J] + t[J] : v[J];
+#pragma unroll
+      for (int J = 0; J < 4; ++J) t[J] = __shfl(v[J], cm, 64);
+      float carry = 0.0f;
+#pragma unroll
+      for (int J = 3; J >= 0; --J) {
+        const float add = carry + (v[J] - c[J]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dcs[4 * J + j] += add;
+        carry += t[J];
+      }
+    }
+    float sumA = 0.0f, sumB = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float da = dcs[k];
+      sumA += da * dtp[k];
+      val[k] = (val[k] + da * An) * dfac[k];
+      if (rm.full || rowk(k) < lim) sumB += val[k];
+    }
+    if (p.dir0 > 0 && p.ddt.ptr) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) val[k] += old[k];
+    }
+    if (p.ddt.ptr) lane_store_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, val);
+    sumA = scan_g_incl(sumA, g4);
+    sumB = scan_g_incl(sumB, g4);
+    if (g4 == 3 && vn) {
+      partA[vec_off(p, u.bt, u.c, u.h) + n] = sumA;
+      partBias[vec_off(p, u.bt, u.c, u.h) + n] = sumB;
+    }
+  }
+
+  {
+    float vb[16], vc[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      vb[k] = s.dbc[k * NTHREADS + tid];
+      vc[k] = s.dbc[(16 + k) * NTHREADS + tid];
+    }
+    if (p.dB[u.dir].ptr) lane_store_ln<true>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, vb);
+    if (p.dC[u.dir].ptr) lane_store_ln<true>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
+  }
+}
+
 // ------------------------------------------------------------------------- dx
 template <int PT>
 struct BwdDxSmem {
@@ -1050,14 +1465,29 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
   return (int)hipGetLastError();
 }
 
+template <int PT, bool IOB, bool DTB, bool FULL>
+static int launch_bwd_chunk_t(const KP& p, int blocks, const float* dy_ws, const float* states, const float* dstates,
+                              const float* dm, const float* g_last, float* partA, float* partBias, hipStream_t st) {
+  if constexpr (IOB) {  // bf16 inputs: every product on the bf16 matrix instructions
+    const size_t sm = sizeof(BwdChunkBfSmem<PT>);
+    if (int e = set_lds(k_bwd_chunk_bf<PT, DTB, FULL>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk_bf<PT, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm,
+                       g_last, partA, partBias);
+  } else {
+    const size_t sm = sizeof(BwdChunkSmem<PT>);
+    if (int e = set_lds(k_bwd_chunk<PT, false, DTB, FULL>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk<PT, false, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
+                       dm, g_last, partA, partBias);
+  }
+  return 0;
+}
+
 int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
                      const float* g_last, float* partA, float* partBias, hipStream_t st) {
   const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
   ISSM_DISPATCH(p, {
-    const size_t sm = sizeof(BwdChunkSmem<PT_>);
-    if (int e = set_lds(k_bwd_chunk<PT_, IOB_, DTB_, FULL_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_chunk<PT_, IOB_, DTB_, FULL_>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
-                       dm, g_last, partA, partBias);
+    if (int e = launch_bwd_chunk_t<PT_, IOB_, DTB_, FULL_>(p, blocks, dy_ws, states, dstates, dm, g_last, partA, partBias, st))
+      return e;
   });
   return (int)hipGetLastError();
 }

@@ -56,7 +56,7 @@ struct KP {
   const float* dfinal[2];
 };
 
-enum : unsigned { F_SOFTPLUS = 1u, F_D_HDIM = 2u };
+enum : unsigned { F_SOFTPLUS = 1u, F_D_HDIM = 2u, F_NOCLAMP = 4u };
 
 // Parameter block of the gated RMSNorm kernels.
 struct NormP {
@@ -165,6 +165,8 @@ __device__ __forceinline__ uint16_t f_to_bf16(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
   return (uint16_t)(u >> 16);
 }
+// a float rounded to bf16 (nearest even) and back
+__device__ __forceinline__ float bf16_round(float f) { return (float)(__bf16)f; }
 // runtime-dtype element access (used only outside hot loops)
 __device__ __forceinline__ float ldv(const void* p, long i, int dt) {
   return dt ? bf16_to_f(((const uint16_t*)p)[i]) : ((const float*)p)[i];
@@ -343,7 +345,7 @@ __device__ __forceinline__ void lp_store_split(const float (&v)[CS * PT * 16 / N
 
 // Same register tile stored transposed, [p][l] (rows = head dimension, KW = CS columns), for products that
 // contract over the rows of the chunk.
-template <int PT, int LD>
+template <int PT, int LD, bool SPLIT = true>
 __device__ __forceinline__ void lp_store_split_t(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* hi,
                                                  uint16_t* lo, int tid = threadIdx.x) {
   constexpr int G4 = 4 * PT;
@@ -356,14 +358,15 @@ __device__ __forceinline__ void lp_store_split_t(const float (&v)[CS * PT * 16 /
       const __bf16 h = (__bf16)w;
       const __bf16 lw = (__bf16)(w - (float)h);
       hi[(p4 + j) * LD + l] = __builtin_bit_cast(uint16_t, h);
-      lo[(p4 + j) * LD + l] = __builtin_bit_cast(uint16_t, lw);
+      if (SPLIT) lo[(p4 + j) * LD + l] = __builtin_bit_cast(uint16_t, lw);
     }
   }
 }
 // acc[pt] += (tile^T)(16 pt .. +15, :) . b  for a product over the 64 chunk rows whose B operand is the lane's
 // 16 column-lane values (k = 4J + j <-> row 16J + 4 g4 + j): two K = 32 steps, step t <-> values 8t .. 8t+7.
 // `b(k)` yields the lane's value k (evaluated step by step, so that only eight are live at a time).
-template <int PT, int LD, typename F>
+// (SPLIT = false: the operands are used as rounded to bf16 -- one instruction per step instead of three.)
+template <int PT, int LD, bool SPLIT = true, typename F>
 __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t* thi, const uint16_t* tlo, F b,
                                                    int cm, int g4) {
 #pragma unroll
@@ -372,11 +375,21 @@ __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t
 #pragma unroll
     for (int j = 0; j < 8; ++j) w[j] = b(8 * t + j);
     bf8 bh, bl;
-    split8(w, bh, bl);
+    if (SPLIT) {
+      split8(w, bh, bl);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bh[j] = (__bf16)w[j];
+    }
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) {
-      const bf8 ah = split_frag<LD>(thi, pt * 16 + cm, g4, t), al = split_frag<LD>(tlo, pt * 16 + cm, g4, t);
-      acc[pt] = mfma_split(ah, al, bh, bl, acc[pt]);
+      const bf8 ah = split_frag<LD>(thi, pt * 16 + cm, g4, t);
+      if (SPLIT) {
+        const bf8 al = split_frag<LD>(tlo, pt * 16 + cm, g4, t);
+        acc[pt] = mfma_split(ah, al, bh, bl, acc[pt]);
+      } else {
+        acc[pt] = mfma_bf(ah, bh, acc[pt]);
+      }
     }
   }
 }
@@ -559,19 +572,35 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
                                            float (&dfac)[16]) {
   const float A2 = cf.A * LOG2E;
   const float bias = cf.bias;
+  // softplus and its derivative share one exponential: with t = e^pre, softplus = log(1 + t) and sigmoid = t / (1 + t);
+  // above the reference's threshold of 20 both are replaced (identity, 1).  F_NOCLAMP: the limits are (0, inf) and
+  // softplus is on, so the clamp and its mask cannot act and are skipped.
   if (p.flags & F_SOFTPLUS) {
+    if (p.flags & F_NOCLAMP) {
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const float pre = raw[k] + bias;
-      const float sp = softplus_(pre);
-      dtp[k] = fminf(fmaxf(sp, p.dt_min), p.dt_max);
-      if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : (pre <= 20.0f ? sigmoidf_(pre) : 1.0f);
+      for (int k = 0; k < 16; ++k) {
+        const float pre = raw[k] + bias;
+        const float t = ex2(pre * LOG2E), u = 1.0f + t;
+        const bool big = pre > 20.0f;
+        dtp[k] = big ? pre : LN2 * __builtin_amdgcn_logf(u);
+        if (WANT_DFAC) dfac[k] = big ? 1.0f : t * __builtin_amdgcn_rcpf(u);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float pre = raw[k] + bias;
+        const float t = ex2(pre * LOG2E), u = 1.0f + t;
+        const bool big = pre > 20.0f;
+        const float sp = big ? pre : LN2 * __builtin_amdgcn_logf(u);
+        dtp[k] = __builtin_amdgcn_fmed3f(sp, p.dt_min, p.dt_max);
+        if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : (big ? 1.0f : t * __builtin_amdgcn_rcpf(u));
+      }
     }
   } else {
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       const float sp = raw[k] + bias;
-      dtp[k] = fminf(fmaxf(sp, p.dt_min), p.dt_max);
+      dtp[k] = __builtin_amdgcn_fmed3f(sp, p.dt_min, p.dt_max);
       if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : 1.0f;
     }
   }

@@ -24,53 +24,19 @@
 
 namespace issm {
 
-template <int PT>
+// Shared memory of k_chunk_local.  Operands of the matrix instructions are bf16 tiles with the contraction index
+// (the state column) contiguous: a lane's operand of one K = 32 step is 8 adjacent columns = one 16-byte read.
+// SPLIT (fp32 inputs): every operand is kept as a (hi, lo) pair and a product is hi.hi + hi.lo + lo.hi; the four
+// operand tiles then hold two levels at a time and a slice takes two passes.  Otherwise (bf16 inputs) one bf16
+// rounding per operand is inside the bf16 tolerance and the four tiles hold the four levels.
+template <int PT, bool SPLIT>
 struct FwdLocalSmem {
-  SplitTile<CS> xt;     // x tile transposed, [p][l], as bf16 (hi, lo)
-  float cs[CS * LDN];   // running sum of dt'*A*log2e [l][n] of the current slice
-  float bd[CS * LDN];   // B*dt' [l][n]
-  float cc[CS * LDN];   // C [l][n]
+  static constexpr int LDK = NS + 8;   // row stride of an operand tile, bf16 elements (conflict-free 16-byte fragment reads)
+  static constexpr int LDT = CS + 8;   // row stride of the transposed x tile
+  uint16_t xt_hi[PT * 16 * LDT];       // x tile transposed, [p][l]
+  uint16_t xt_lo[SPLIT ? PT * 16 * LDT : 8];
+  uint16_t op[4][CS * LDK];            // level operands [l][n]
 };
-
-// Row-lane fragments of 16 rows x 64 columns: lane (cm, g4) holds row cm, columns 16kb + 4g4 + j.
-struct Frag {
-  f4 v[4];
-};
-__device__ __forceinline__ Frag frag_rows(const float* tile, int row0, int cm, int g4) {
-  Frag f;
-#pragma unroll
-  for (int kb = 0; kb < 4; ++kb) f.v[kb] = *(const f4*)(tile + (row0 + cm) * LDN + kb * 16 + 4 * g4);
-  return f;
-}
-__device__ __forceinline__ Frag frag_row_bcast(const float* tile, int row, int g4) {
-  Frag f;
-#pragma unroll
-  for (int kb = 0; kb < 4; ++kb) f.v[kb] = *(const f4*)(tile + row * LDN + kb * 16 + 4 * g4);
-  return f;
-}
-
-// Level 8 (LV = 3) or 4 (LV = 2) of the wave's diagonal block, operands built in registers from the wave's
-// own row fragments; the reference row of lane row cm is another row of the same block.
-template <int LV>
-__device__ __forceinline__ void m_mid_level(f4& acc, const Frag& cs, const Frag& cc, const Frag& bd, int cm,
-                                            int g4) {
-  constexpr int w = 1 << LV;
-  const int src = ((cm & ~(2 * w - 1)) + w - 1) + 16 * g4;
-  const bool upper = (cm & w) != 0;
-#pragma unroll
-  for (int kb = 0; kb < 4; ++kb) {
-    float ref[4], t[4];  // four cross-lane fetches in flight together
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ref[j] = __shfl(cs.v[kb][j], src, 64);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float d = cs.v[kb][j] - ref[j];
-      t[j] = (upper ? cc.v[kb][j] : bd.v[kb][j]) * ex2(upper ? d : -d);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc = mfma4(t[j], t[j], acc);
-  }
-}
 
 // sum over the 16 lanes of a row (lanes sharing g4); the total is valid in the lane with cm == 15
 __device__ __forceinline__ float row_sum16(float v) {
@@ -84,13 +50,35 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
+// the lane's 16 values of one operand -> column `col` of a [64][LDK] bf16 tile (hi, and lo if wanted)
+template <int LDK, bool SPLIT>
+__device__ __forceinline__ void op_store(const float (&v)[16], uint16_t* hi, uint16_t* lo, int g4, int col) {
+#pragma unroll
+  for (int k = 0; k < 16; k += 2) {
+    const unsigned h2 = pack_bf16(v[k], v[k + 1]);
+    const int o0 = lane_row(k, g4) * LDK + col, o1 = lane_row(k + 1, g4) * LDK + col;
+    hi[o0] = (uint16_t)h2;
+    hi[o1] = (uint16_t)(h2 >> 16);
+    if (SPLIT) {
+      const unsigned l2 = pack_bf16(v[k] - __uint_as_float(h2 << 16), v[k + 1] - __uint_as_float(h2 & 0xffff0000u));
+      lo[o0] = (uint16_t)l2;
+      lo[o1] = (uint16_t)(l2 >> 16);
+    }
+  }
+}
+template <int LDK>
+__device__ __forceinline__ bf8 op_frag(const uint16_t* tile, int row, int g4, int t) {
+  return *(const bf8*)(tile + row * LDK + 32 * t + 8 * g4);
+}
+
 template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __restrict__ states,
                                                           float* __restrict__ cs_last, float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  typedef FwdLocalSmem<PT> SM;
+  constexpr bool SPLIT = !IOB;
+  typedef FwdLocalSmem<PT, SPLIT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDT = SplitTile<CS>::LD;
+  constexpr int LDT = SM::LDT, LDK = SM::LDK;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -108,23 +96,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
   {
     float xv[CS * PT * 16 / NTHREADS];
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
-    lp_store_split_t<PT, LDT>(xv, s.xt.hi, s.xt.lo);
+    lp_store_split_t<PT, LDT, SPLIT>(xv, s.xt_hi, s.xt_lo);
   }
-  // accumulators of M.  od: the six off-diagonal blocks (1,0) (3,2) | (2,0) (2,1) (3,0) (3,1), each wave
-  // summing over its own 16 columns of every slice; a8 / a4: levels 8 and 4 of the wave's diagonal
-  // block; sp: the lane's in-group pairs (J, jl >= js) of its own column.
-  f4 od[6], a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0};
-#pragma unroll
-  for (int b = 0; b < 6; ++b) od[b] = (f4){0, 0, 0, 0};
+  // Accumulators of M.  od: the off-diagonal 16x16 blocks (I, J) this wave owns -- (1,0) and (3,0) in wave 0, (3,2)
+  // and (3,1) in wave 1, (2,0) in wave 2, (2,1) in wave 3; a8 / a4: levels 8 and 4 of the wave's diagonal block; sp:
+  // the lane's in-group pairs (J, jl >= js) of its own column.
+  f4 od[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, a8 = {0, 0, 0, 0}, a4 = {0, 0, 0, 0};
   float sp[40];
 #pragma unroll
   for (int i = 0; i < 40; ++i) sp[i] = 0.0f;
+  // roles of the lane's rows at the two levels that pair rows of one 16-row tile (the lane's rows are 4 g4 + j of
+  // every tile): upper half of the 16-row block / of the 8-row block
+  const bool up8 = (g4 & 2) != 0, up4 = (g4 & 1) != 0;
+  const float sg8 = up8 ? 1.0f : -1.0f, sg4 = up4 ? 1.0f : -1.0f;
 
   __syncthreads();  // x tile complete
   for (int n0 = 0; n0 < p.N; n0 += NS) {
-    // ---- column-lane phase, registers only (overlaps other waves still in the previous slice's row-lane phase)
-    // B and C of this slice are requested here and first used after the dt transform, which covers their
-    // latency; only dt is prefetched across the row-lane phase (fewer registers live there)
+    // ---- column-lane phase, registers only
     lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, vn, g4, rm, bv);
     lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, vn, g4, rm, cv);
     float dtp[16], cs[16], dummy[16];
@@ -133,17 +121,24 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 #pragma unroll
     for (int k = 0; k < 16; ++k) bd[k] = bv[k] * dtp[k];
     if (g4 == 0 && vn) cs_last[vec_off(p, u.bt, u.c, u.h) + n] = last * LN2;
+    if (n0 + NS < p.N) {  // the next slice's dt is requested as soon as this slice's has been consumed
+      n = n0 + NS + wave * 16 + cm;
+      vn = FULL || n < p.N;
+      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
+      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
+      cf = lane_coef(p, u.h, n, vn);
+    }
 
     if (want_s) {
-      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers,
-      // split-bf16 product over the 64 rows
+      // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-      rows_product_split<PT, LDT>(acc, s.xt.hi, s.xt.lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
+      rows_product_split<PT, LDT, SPLIT>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
+      const int nn = n0 + wave * 16 + cm;
       if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
-        float* d0 = dst + (4 * g4) * p.N + n;
+        float* d0 = dst + (4 * g4) * p.N + nn;
 #pragma unroll
         for (int pt = 0; pt < PT; ++pt)
 #pragma unroll
@@ -154,7 +149,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int pp = pt * 16 + 4 * g4 + r;
-            if (pp < p.P && vn) dst[(long)pp * p.N + n] = acc[pt][r];
+            if (pp < p.P && nn < p.N) dst[(long)pp * p.N + nn] = acc[pt][r];
           }
       }
     }
@@ -171,91 +166,99 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
             const float cb = cv[kl] * bd[ks];
             sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * ex2(cs[kl] - cs[ks]);
           }
-      if (n0 > 0) __syncthreads();  // every wave has finished reading the previous slice's LDS tiles
+      // reference rows of the four levels: cross-lane fetches, all issued before the first is used
+      const float r15 = __shfl(cs[3], cm + 48, 64), r31 = __shfl(cs[7], cm + 48, 64), r47 = __shfl(cs[11], cm + 48, 64);
+      float ref8[4], ref4[4];
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const int o = lane_row(k, g4) * LDN + wave * 16 + cm;
-        s.cs[o] = cs[k];
-        s.bd[o] = bd[k];
-        s.cc[o] = cv[k];
-      }
-    }
-    if (n0 + NS < p.N) {  // prefetch the next slice's dt into the registers that have just been consumed
-      n = n0 + NS + wave * 16 + cm;
-      vn = FULL || n < p.N;
-      rm = make_rowmap<FULL>(p, u, g4, n0 + NS);
-      lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
-      cf = lane_coef(p, u.h, n, vn);
-    }
-
-    if (want_m) {
-      __syncthreads();  // the slice's LDS tiles are complete
-      // ---- row-lane phase, levels 8 and 4: this wave's diagonal block from its own row fragments
-      {
-        const Frag fc = frag_rows(s.cs, wave * 16, cm, g4);
-        const Frag fcc = frag_rows(s.cc, wave * 16, cm, g4);
-        const Frag fbd = frag_rows(s.bd, wave * 16, cm, g4);
-        m_mid_level<3>(a8, fc, fcc, fbd, cm, g4);
-        pin4(a8);
-        m_mid_level<2>(a4, fc, fcc, fbd, cm, g4);
-        pin4(a4);
-      }
-      // levels 16 and 32: all six off-diagonal blocks over this wave's 16 columns (4 MFMA steps each)
-      {
-        const int co = wave * 16 + 4 * g4;
-        auto rows = [&](const float* tile, int T) { return *(const f4*)(tile + (T * 16 + cm) * LDN + co); };
-        auto ref = [&](int R) { return *(const f4*)(s.cs + R * LDN + co); };
-        const f4 r15 = ref(15), r31 = ref(31), r47 = ref(47);
-        const f4 c0 = rows(s.cs, 0), c1 = rows(s.cs, 1), c2 = rows(s.cs, 2), c3 = rows(s.cs, 3);
-        const f4 b0 = rows(s.bd, 0), b1 = rows(s.bd, 1), b2 = rows(s.bd, 2);
-        const f4 q1 = rows(s.cc, 1), q2 = rows(s.cc, 2), q3 = rows(s.cc, 3);
+      for (int J = 0; J < 4; ++J) ref8[J] = __shfl(cs[4 * J + 3], cm + 16, 64);               // row 16 J + 7
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float A1 = q1[j] * ex2(c1[j] - r15[j]), B0 = b0[j] * ex2(r15[j] - c0[j]);    // level 16, rows 0..31
-          const float A3 = q3[j] * ex2(c3[j] - r47[j]), B2 = b2[j] * ex2(r47[j] - c2[j]);    // level 16, rows 32..63
-          const float A2w = q2[j] * ex2(c2[j] - r31[j]), A3w = q3[j] * ex2(c3[j] - r31[j]);  // level 32
-          const float B0w = b0[j] * ex2(r31[j] - c0[j]), B1w = b1[j] * ex2(r31[j] - c1[j]);
-          od[0] = mfma4(A1, B0, od[0]);
-          od[1] = mfma4(A3, B2, od[1]);
-          od[2] = mfma4(A2w, B0w, od[2]);
-          od[3] = mfma4(A2w, B1w, od[3]);
-          od[4] = mfma4(A3w, B0w, od[4]);
-          od[5] = mfma4(A3w, B1w, od[5]);
+      for (int J = 0; J < 4; ++J) ref4[J] = __shfl(cs[4 * J + 3], cm + 16 * (g4 & 2), 64);    // row 16 J + 8 (g4 / 2) + 3
+      const int col = wave * 16 + cm;
+      float v[16];
+      // levels 16 and 32 pair rows of different tiles: the role of a row is fixed by its tile
+      auto big16 = [&]() {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const int J = k >> 2;
+          const float ref = (J & 2) ? r47 : r15;
+          v[k] = (J & 1) ? cv[k] * ex2(cs[k] - ref) : bd[k] * ex2(ref - cs[k]);
         }
+      };
+      auto big32 = [&]() {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) v[k] = (k >> 3) ? cv[k] * ex2(cs[k] - r31) : bd[k] * ex2(r31 - cs[k]);
+      };
+      auto mid = [&](const float (&ref)[4], bool up, float sg) {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) v[k] = (up ? cv[k] : bd[k]) * ex2(sg * (cs[k] - ref[k >> 2]));
+      };
+      // products of one pass: T16 / T32 / T8 / T4 name the (hi, lo) tiles holding that level (nullptr = not in this pass)
+      auto products = [&](const uint16_t* h16, const uint16_t* l16, const uint16_t* h32, const uint16_t* l32,
+                          const uint16_t* h8, const uint16_t* l8, const uint16_t* h4, const uint16_t* l4) {
+        auto prod = [&](f4& acc, const uint16_t* th, const uint16_t* tl, int ra, int rb) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const bf8 ah = op_frag<LDK>(th, ra + cm, g4, t), bh = op_frag<LDK>(th, rb + cm, g4, t);
+            if (SPLIT) {
+              const bf8 al = op_frag<LDK>(tl, ra + cm, g4, t), bl = op_frag<LDK>(tl, rb + cm, g4, t);
+              acc = mfma_bf(al, bh, acc);
+              acc = mfma_bf(ah, bl, acc);
+            }
+            acc = mfma_bf(ah, bh, acc);
+          }
+        };
+        if (h8) prod(a8, h8, l8, wave * 16, wave * 16);
+        if (h4) prod(a4, h4, l4, wave * 16, wave * 16);
+        if (h16 && wave < 2) prod(od[0], h16, l16, wave ? 48 : 16, wave ? 32 : 0);       // (1,0) | (3,2)
+        if (h32) {
+          if (wave < 2) prod(od[1], h32, l32, 48, wave ? 16 : 0);                         // (3,0) | (3,1)
+          else prod(od[0], h32, l32, 32, wave == 2 ? 0 : 16);                             // (2,0) | (2,1)
+        }
+      };
+      if (n0 > 0) __syncthreads();  // every wave has finished reading the previous slice's tiles
+      if (SPLIT) {
+        big16(); op_store<LDK, true>(v, s.op[0], s.op[1], g4, col);
+        big32(); op_store<LDK, true>(v, s.op[2], s.op[3], g4, col);
+        __syncthreads();
+        products(s.op[0], s.op[1], s.op[2], s.op[3], nullptr, nullptr, nullptr, nullptr);
+        __syncthreads();
+        mid(ref8, up8, sg8); op_store<LDK, true>(v, s.op[0], s.op[1], g4, col);
+        mid(ref4, up4, sg4); op_store<LDK, true>(v, s.op[2], s.op[3], g4, col);
+        __syncthreads();
+        products(nullptr, nullptr, nullptr, nullptr, s.op[0], s.op[1], s.op[2], s.op[3]);
+      } else {
+        big16(); op_store<LDK, false>(v, s.op[0], nullptr, g4, col);
+        big32(); op_store<LDK, false>(v, s.op[1], nullptr, g4, col);
+        mid(ref8, up8, sg8); op_store<LDK, false>(v, s.op[2], nullptr, g4, col);
+        mid(ref4, up4, sg4); op_store<LDK, false>(v, s.op[3], nullptr, g4, col);
+        __syncthreads();
+        products(s.op[0], nullptr, s.op[1], nullptr, s.op[2], nullptr, s.op[3], nullptr);
       }
     }
   }
 
   if (want_m) {
+    float* m = cabt + sq_off(p, u.bt, u.c, u.h);
+    // off-diagonal blocks: complete in the wave that owns them; accumulator r <-> (row 4 g4 + r, column cm)
+    {
+      const int I0 = wave == 0 ? 1 : wave == 1 ? 3 : 2, J0 = wave == 0 ? 0 : wave == 1 ? 2 : wave == 2 ? 0 : 1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) m[(I0 * 16 + 4 * g4 + r) * CS + J0 * 16 + cm] = od[0][r];
+      if (wave < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m[(48 + 4 * g4 + r) * CS + wave * 16 + cm] = od[1][r];
+      }
+    }
     __syncthreads();  // all waves are done with the last slice's tiles
-    // combine the waves' partial sums through LDS (the slice tiles are free now)
-    static_assert(4 * 6 * 4 * 64 + 4 * 4 * 40 <= 3 * CS * LDN, "reduction scratch must fit in the slice tiles");
-    float* red_od = s.cs;                    // [wave][block][r][lane], runs on into the bd / cc tiles
-    float* red_sp = s.cs + 4 * 6 * 4 * 64;   // [wave][g4][40]
-#pragma unroll
-    for (int b = 0; b < 6; ++b)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) red_od[((wave * 6 + b) * 4 + r) * 64 + lane] = od[b][r];
+    // the in-lane pairs are sums over columns: over the 16 lanes of a row, then over the waves through LDS
+    float* red_sp = reinterpret_cast<float*>(s.op[0]);   // [wave][g4][40]
+    static_assert(4 * 4 * 40 * sizeof(float) <= sizeof(s.op[0]), "reduction scratch must fit in an operand tile");
 #pragma unroll
     for (int i = 0; i < 40; ++i) {
       const float t = row_sum16(sp[i]);
       if (cm == 15) red_sp[(wave * 4 + g4) * 40 + i] = t;
     }
     __syncthreads();
-    float* m = cabt + sq_off(p, u.bt, u.c, u.h);
-    // off-diagonal blocks: thread tid owns entry (r, lane) = (tid >> 6, tid & 63) of each block
-    {
-      const int r = tid >> 6, ln = tid & 63, row = 4 * (ln >> 4) + r, col = ln & 15;
-#pragma unroll
-      for (int b = 0; b < 6; ++b) {
-        float v = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) v += red_od[((w * 6 + b) * 4 + r) * 64 + ln];
-        const int I = b == 0 ? 1 : b == 1 ? 3 : b < 4 ? 2 : 3;
-        const int J = b == 0 ? 0 : b == 1 ? 2 : (b & 1) ? 1 : 0;
-        m[(I * 16 + row) * CS + J * 16 + col] = v;
-      }
-    }
     // diagonal block of this wave: row l = 4 g4 + r, column sc = cm
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -523,7 +526,7 @@ static int set_lds(K kernel, size_t bytes) {
 int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
-    const size_t sm = sizeof(FwdLocalSmem<PT_>);
+    const size_t sm = sizeof(FwdLocalSmem<PT_, !IOB_>);
     if (int e = set_lds(k_chunk_local<PT_, IOB_, DTB_, FULL_>, sm)) return e;
     hipLaunchKernelGGL((k_chunk_local<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
   });
