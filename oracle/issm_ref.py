@@ -21,18 +21,20 @@ What each function restates (paths relative to the reference checkout):
                               per-chunk states, inter-chunk recurrence, state->output),
                               evaluated per (batch, head) so that the exp(segsum) tensor
                               stays small.  This is the CPU baseline that is timed.
-* ``issm_chunk_scan_combined_ref``  operator-level semantics of
-                              issm_triton/issm_combined.py:16-92 (argument meaning,
-                              output dtypes) on top of the sequential recurrence
+* ``issm_biscan_ref``         the module's bidirectional use of the scan,
+                              models/dest_module.py:565-575
 * ``issm_bwd_closed_form``    closed-form gradients of the chunked algorithm (the sums
                               evaluated by issm_combined.py:95-179 and the kernels it
-                              calls), used to cross-check autograd and to debug kernels
+                              calls), used to cross-check autograd and to debug kernels;
+                              its per-chunk intermediates (S, states, M, dM, dH, dS,
+                              g_next, y) are what the GPU stage tests compare with
 * ``gated_rmsnorm_ref``       issm_triton/layernorm_gated.py:8-29
 
 Pinning status: every function here is pinned by tests/test_oracle.py against an
 independent brute-force numpy loop on tiny shapes, against closed forms (A=0, dt=0,
-B=0, N=P=1 by hand), by chunk-size invariance, by time-reversal symmetry and by
-torch.autograd.gradcheck.  The reference holds no golden vectors for this path
+B=0, N=P=1 by hand), by chunk-size invariance, by time-reversal symmetry, by
+torch.autograd.gradcheck, and -- the per-chunk intermediates -- by a chunk-by-chunk
+evaluation of the token recurrence with autograd and scalar loops.  The reference holds no golden vectors for this path
 (test_issm.py prints errors, asserts nothing, ships no data).
 """
 from __future__ import annotations
@@ -164,23 +166,6 @@ def issm_scan_chunked(x, dtp, A, B, C, chunk, initial_states=None):
             y[b, :, h] = (y_diag + y_off).reshape(L, P)
             final[b, h] = Hprev[-1]
     return y, final
-
-
-def issm_chunk_scan_combined_ref(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None,
-                                 initial_states=None, seq_idx=None, dt_softplus=False,
-                                 dt_limit=(0.0, INF), return_final_states=False,
-                                 dtype=torch.float64):
-    """Operator-level oracle with the signature of issm_combined.py:16.
-
-    ``chunk_size`` does not change the mathematical result; it is accepted for
-    signature parity.  Output ``out`` is cast to x.dtype, final states stay fp32+
-    (issm_state_passing.py:17) -- here they are returned in ``dtype``.
-    """
-    assert seq_idx is None, "seq_idx is not used by DEST (dest_module.py:600-611)"
-    y, fin = issm_scan_sequential(x, dt, A, B, C, D=D, z=z, dt_bias=dt_bias,
-                                  initial_states=initial_states, dt_softplus=dt_softplus,
-                                  dt_limit=dt_limit, dtype=dtype)
-    return (y, fin) if return_final_states else y
 
 
 def issm_biscan_ref(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, D=None, initial_states=None,

@@ -356,6 +356,81 @@ def test_properties_at_benchmark_shape():
         _check("d" + k, gi[k].grad, ins[k].grad, BWD32)
 
 
+def test_benchmark_shape_bf16_bidirectional():
+    """configs[1] with bf16 inputs (x, B, C, dt bf16; A, D fp32; fp32 states), both directions fused, at full size
+    (B=8, L=1024, H=8, P=32, N=256): the fused call against two single-direction calls on flipped copies (outputs bit
+    for bit; gradients as the sum of the parts), run-to-run reproducibility, and the fp64 oracle on one (batch, head)
+    through the fused call -- forward and every gradient inside the bf16 tolerances."""
+    from dest3d_amd import ISSM_biscan_combined, ISSM_chunk_scan_combined as op
+    _say("benchmark shape bf16 bidirectional B=8 L=1024 H=8 P=32 N=256")
+    dev = "cuda"
+    I = R.make_inputs(8, 1024, 8, 32, 256, seed=1235, h0_std=0.1)
+    g2 = torch.Generator().manual_seed(1236)
+    bf = lambda v: v.to(dev, torch.bfloat16)
+    t = dict(x=bf(I["x"]), x_b=bf(torch.randn(I["x"].shape, generator=g2)), dt=bf(I["dt_raw"]), B=bf(I["B"]),
+             B_b=bf(torch.randn(I["B"].shape, generator=g2) / 16.0), C=bf(I["C"]),
+             C_b=bf(torch.randn(I["C"].shape, generator=g2) / 16.0), A=I["A"].to(dev), D=I["D"].to(dev),
+             h0=I["h0"].to(dev))
+    dy, dy_b = I["dy"].to(dev), torch.randn(I["x"].shape, generator=g2).to(dev)
+    df, df_b = I["dfinal"].to(dev), torch.randn(I["dfinal"].shape, generator=g2).to(dev)
+    names = ("x", "x_b", "dt", "A", "B", "B_b", "C", "C_b", "D", "h0")
+
+    def fused():
+        g = {k: t[k].detach().clone().requires_grad_() for k in names}
+        o = ISSM_biscan_combined(g["x"], g["x_b"], g["dt"], g["A"], g["B"], g["B_b"], g["C"], g["C_b"], 64, D=g["D"],
+                                 initial_states=g["h0"], dt_softplus=True)
+        ((o[0].float() * dy).sum() + (o[1].float() * dy_b).sum() + (o[2] * df).sum() + (o[3] * df_b).sum()).backward()
+        torch.cuda.synchronize()
+        return o, g
+
+    o, g = fused()
+    o2, g2_ = fused()
+    for a, b in zip(o, o2):
+        assert torch.equal(a, b)
+    for k in names:
+        assert torch.equal(g[k].grad, g2_[k].grad), f"d{k} differs between two runs"
+    # two single-direction calls, the second on flipped copies
+    fl = lambda v: torch.flip(v, dims=[1]).contiguous()
+    a = {k: t[k].detach().clone().requires_grad_() for k in ("x", "dt", "A", "B", "C", "D", "h0")}
+    y1, l1 = op(a["x"], a["dt"], a["A"], a["B"], a["C"], 64, D=a["D"], initial_states=a["h0"], dt_softplus=True,
+                return_final_states=True)
+    ((y1.float() * dy).sum() + (l1 * df).sum()).backward()
+    r = {k: t[k].detach().clone().requires_grad_() for k in ("x_b", "dt", "A", "B_b", "C_b", "D", "h0")}
+    y2, l2 = op(fl(r["x_b"]), fl(r["dt"]), r["A"], fl(r["B_b"]), fl(r["C_b"]), 64, D=r["D"], initial_states=r["h0"],
+                dt_softplus=True, return_final_states=True)
+    ((y2.float() * fl(dy_b)).sum() + (l2 * df_b).sum()).backward()
+    torch.cuda.synchronize()
+    assert torch.equal(o[0], y1) and torch.equal(o[2], l1)
+    assert torch.equal(o[1], torch.flip(y2, dims=[1])) and torch.equal(o[3], l2)
+    for k, part in (("x", a["x"]), ("B", a["B"]), ("C", a["C"]), ("x_b", r["x_b"]), ("B_b", r["B_b"]), ("C_b", r["C_b"])):
+        assert torch.equal(g[k].grad, part.grad), f"d{k}: fused != single direction"
+    for k in ("A", "D", "h0"):
+        _check(f"d{k} fused vs sum of parts", g[k].grad, a[k].grad + r[k].grad, 1e-5)
+    # ddt leaves in bf16: the fused call rounds the first direction's part before the second is added
+    _check("ddt fused vs sum of parts", g["dt"].grad, a["dt"].grad.float() + r["dt"].grad.float(), 1e-2)
+    del o2, g2_, a, r, y1, y2
+    # oracle on (b, h) = (5, 3), both directions through the fused call on strided views
+    b0, hh = 5, 3
+    sl = {k: (t[k][b0:b0 + 1, :, hh:hh + 1] if k in ("x", "x_b", "dt") else
+              t[k][hh:hh + 1] if k in ("A", "D") else
+              t[k][b0:b0 + 1, hh:hh + 1] if k == "h0" else t[k][b0:b0 + 1]) for k in names}
+    w = [v.double().cpu() for v in (dy[b0:b0 + 1, :, hh:hh + 1], dy_b[b0:b0 + 1, :, hh:hh + 1],
+                                     df[b0:b0 + 1, hh:hh + 1], df_b[b0:b0 + 1, hh:hh + 1])]
+    ref = {k: v.detach().double().cpu().clone().requires_grad_() for k, v in sl.items()}
+    o_ref = R.issm_biscan_ref(ref["x"], ref["x_b"], ref["dt"], ref["A"], ref["B"], ref["B_b"], ref["C"], ref["C_b"],
+                              D=ref["D"], initial_states=ref["h0"], dt_softplus=True)
+    sum((oi * wi).sum() for oi, wi in zip(o_ref, w)).backward()
+    gg = {k: v.detach().requires_grad_() for k, v in sl.items()}
+    og = ISSM_biscan_combined(gg["x"], gg["x_b"], gg["dt"], gg["A"], gg["B"], gg["B_b"], gg["C"], gg["C_b"], 64,
+                              D=gg["D"], initial_states=gg["h0"], dt_softplus=True)
+    sum((oi.float() * wi.to(dev).float()).sum() for oi, wi in zip(og, w)).backward()
+    torch.cuda.synchronize()
+    for name, ai, bi in zip(("y_f", "y_b", "last_f", "last_b"), og, o_ref):
+        _check(name, ai, bi, FWD16)
+    for k in ref:
+        _check("d" + k, gg[k].grad, ref[k].grad, BWD16)
+
+
 def _split_sequence_check(t, dtype, Lh, tol_sum):
     """scan(whole sequence) must equal scan(first part) followed by scan(rest) started from the first part's
     final state, forward and backward (the backward chains d(initial_states) of the second call into

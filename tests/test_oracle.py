@@ -184,6 +184,64 @@ def test_closed_form_backward_matches_autograd(L, chunk, softplus):
         assert (g["ddt"] == 0).any()
 
 
+def test_closed_form_intermediates_against_chunk_by_chunk_autograd():
+    """The per-chunk quantities that issm_bwd_closed_form(intermediates=True) returns -- and that the GPU stage tests
+    compare the kernels with -- derived independently: the sequence is scanned chunk by chunk with the token-by-token
+    recurrence, each chunk started from the previous chunk's final state, with a zero "extra log-decay" leaf eps_c[n]
+    multiplying the state handed to the next chunk.  Then, by autograd alone,
+      states[c]  = state entering chunk c              S[c]   = final state of chunk c scanned from a zero state
+      y          = concatenated chunk outputs          dS[c]  = dL / d(state handed over after chunk c)
+      dH[c]      = dL / d(state entering chunk c) holding later states fixed  (= grad through chunk c's outputs only)
+      g_next[c]  = dL / d eps_c   (= sum_p dS[c] * states[c + 1]: what reaches the chunk's total decay via the states)
+    and M, dM from their definitions with scalar loops."""
+    chunk, L = 4, 11                                     # ragged last chunk
+    x, dt, A, B, C, D, h0 = _rand_problem(L=L, seed=11)
+    Bsz, _, H, P = x.shape
+    N = dt.shape[-1]
+    dy, dfin = torch.randn_like(x), torch.randn_like(h0)
+    out = R.issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=dfin, D=None, initial_states=h0, intermediates=True)
+    nc = math.ceil(L / chunk)
+    states, eps, ys, handed = [h0.clone().requires_grad_()], [], [], []
+    for c in range(nc):
+        sl = slice(c * chunk, min(L, (c + 1) * chunk))
+        y_c, fin_c = R.issm_scan_sequential(x[:, sl], dt[:, sl], A, B[:, sl], C[:, sl], initial_states=states[-1])
+        e = torch.zeros(Bsz, H, N, dtype=torch.float64, requires_grad=True)
+        nxt = fin_c * torch.exp(e)[:, :, None, :]
+        nxt.retain_grad()
+        eps.append(e); ys.append(y_c); handed.append(nxt)
+        states.append(nxt)
+    y = torch.cat(ys, dim=1)
+    ((y * dy).sum() + (states[-1] * dfin).sum()).backward()
+    close = lambda a, b, name: torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-10, msg=lambda m: f"{name}: {m}")
+    close(out["y"], y.detach(), "y")
+    close(out["states"], torch.stack([t.detach() for t in states], dim=1), "states")
+    close(out["dS"], torch.stack([t.grad for t in handed], dim=1), "dS")
+    close(out["g_next"], torch.stack([e.grad for e in eps], dim=1), "g_next")
+    close(out["dinitial_states"], states[0].grad, "dh0")
+    for c in range(nc):
+        sl = slice(c * chunk, min(L, (c + 1) * chunk))
+        # chunk-local end state: the chunk scanned from nothing
+        _, s_c = R.issm_scan_sequential(x[:, sl], dt[:, sl], A, B[:, sl], C[:, sl])
+        close(out["S"][:, c], s_c, f"S[{c}]")
+        # dH[c]: gradient of this chunk's outputs alone with respect to its entry state
+        hin = states[c].detach().clone().requires_grad_()
+        y_c, _ = R.issm_scan_sequential(x[:, sl], dt[:, sl], A, B[:, sl], C[:, sl], initial_states=hin)
+        (y_c * dy[:, sl]).sum().backward()
+        close(out["dH"][:, c], hin.grad, f"dH[{c}]")
+    # M[l][s] = sum_n C[l,n] B[s,n] dt[s,n] exp(sum_{s<k<=l} dt[k,n] A[n]) and dM = tril(dy x^T), scalar loops on (b=1, h=2)
+    b, h, g = 1, 2, 2 // (H // B.shape[2])
+    a = (dt * A[None, None]).numpy()
+    for c in range(nc):
+        lo, hi = c * chunk, min(L, (c + 1) * chunk)
+        for l in range(lo, hi):
+            for s_ in range(lo, l + 1):
+                m = sum(C[b, l, g, n].item() * B[b, s_, g, n].item() * dt[b, s_, h, n].item()
+                        * math.exp(a[b, s_ + 1:l + 1, h, n].sum()) for n in range(N))
+                assert abs(out["M"][b, c, h, l - lo, s_ - lo].item() - m) < 1e-10
+                dm = sum(dy[b, l, h, p].item() * x[b, s_, h, p].item() for p in range(P))
+                assert abs(out["dM"][b, c, h, l - lo, s_ - lo].item() - dm) < 1e-10
+
+
 def test_gated_rmsnorm_closed_form_and_grad():
     x = torch.randn(3, 5, 8, dtype=torch.float64)
     z = torch.randn(3, 5, 8, dtype=torch.float64)
