@@ -47,12 +47,16 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_gate(KP p, const float* __rest
 }
 
 // ------------------------------------------------------------ dstates and dM
-template <int PT>
+// BF (bf16 inputs): the dy and x tiles are kept as bf16 (exact) and every product runs on the bf16 matrix instruction.
+template <int PT, bool BF>
 struct BwdStSmem {
   static constexpr int LDPT = PT * 16 + 4;
-  float dys[CS * LDPT];
-  float xs[CS * LDPT];
-  SplitTile<CS> dyt;  // dy tile transposed, [p][l], as bf16 (hi, lo): operand of dH
+  static constexpr int LDP = PT * 16 + 8;   // bf16 tiles [l][p]
+  static constexpr int LDT = CS + 8;        // transposed dy tile [p][l]
+  typename std::conditional<BF, uint16_t, float>::type dys[CS * (BF ? LDP : LDPT)];
+  typename std::conditional<BF, uint16_t, float>::type xs[CS * (BF ? LDP : LDPT)];
+  uint16_t dyt_hi[PT * 16 * LDT];             // dy tile transposed, [p][l]: operand of dH
+  uint16_t dyt_lo[BF ? 8 : PT * 16 * LDT];
 };
 
 // dH[p][n] = sum_l dy[l][p] * C[l][n] exp2(cs[l][n]): contraction over rows, so the B operand
@@ -62,9 +66,9 @@ template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __restrict__ dy_ws,
                                                           float* __restrict__ dstates, float* __restrict__ dm) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  typedef BwdStSmem<PT> SM;
+  typedef BwdStSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT;
+  constexpr int LDPT = SM::LDPT, LDP = SM::LDP, LDT = SM::LDT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -84,9 +88,14 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     float dv[CS * PT * 16 / NTHREADS], xv[CS * PT * 16 / NTHREADS];
     dy_load<IOB, PT, FULL>(p, u, dy_ws, dv);
     lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv);
-    lp_store<PT>(dv, s.dys, LDPT);
-    lp_store<PT>(xv, s.xs, LDPT);
-    if (dstates) lp_store_split_t<PT, SplitTile<CS>::LD>(dv, s.dyt.hi, s.dyt.lo);
+    if constexpr (IOB) {
+      lp_store_bf<PT, LDP>(dv, s.dys, tid);
+      lp_store_bf<PT, LDP>(xv, s.xs, tid);
+    } else {
+      lp_store<PT>(dv, s.dys, LDPT);
+      lp_store<PT>(xv, s.xs, LDPT);
+    }
+    if (dstates) lp_store_split_t<PT, LDT, !IOB>(dv, s.dyt_hi, s.dyt_lo);
   }
   __syncthreads();
 
@@ -94,8 +103,19 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     float* m = dm + sq_off(p, u.bt, u.c, u.h);
     for (int j = 0; j <= wave; ++j) {
       f4 acc = {0, 0, 0, 0};
+      if constexpr (IOB) {
+        constexpr int KT = (PT + 1) / 2;
 #pragma unroll
-      for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
+        for (int t = 0; t < KT; ++t) {
+          const bool half = (PT & 1) && t == KT - 1;  // an odd number of 16-column tiles: the last step is half full
+          const bf8 a = half ? split_frag<LDP, true>(s.dys, wave * 16 + cm, g4, t) : split_frag<LDP>(s.dys, wave * 16 + cm, g4, t);
+          const bf8 b = half ? split_frag<LDP, true>(s.xs, j * 16 + cm, g4, t) : split_frag<LDP>(s.xs, j * 16 + cm, g4, t);
+          acc = mfma_bf(a, b, acc);
+        }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
+      }
       if (IOB) {
         // bf16 inputs: the block goes out as two bf16 copies in the same 16 KB, dM[l][s] at [l][s] of the first half
         // and at [s][l] of the second, which is what k_bwd_chunk_bf's matrix operands read (blocks above the diagonal
@@ -143,7 +163,7 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
     f4 acc[PT];
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-    rows_product_split<PT, SplitTile<CS>::LD>(acc, s.dyt.hi, s.dyt.lo, [&](int k) { return ct[k]; }, cm, g4);
+    rows_product_split<PT, LDT, IOB ? 2 : 1>(acc, s.dyt_hi, s.dyt_lo, [&](int k) { return ct[k]; }, cm, g4);
     float* dst = dstates + dst_off(p, u.bt, u.c, u.h);
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt)
@@ -976,18 +996,6 @@ __device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const
   }
 }
 
-// a (64 x 16 PT) register tile (layout of lp_load) as bf16 into LDS dst[l][p]
-template <int PT, int LD>
-__device__ __forceinline__ void lp_store_bf(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* dst, int tid) {
-  constexpr int G4 = 4 * PT;
-#pragma unroll
-  for (int i = 0; i < PT; ++i) {
-    const int e4 = tid + i * NTHREADS;
-    *(uint2*)(dst + (e4 / G4) * LD + (e4 % G4) * 4) =
-        make_uint2(pack_bf16(v[4 * i], v[4 * i + 1]), pack_bf16(v[4 * i + 2], v[4 * i + 3]));
-  }
-}
-
 template <int PT, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws,
                                                               const float* __restrict__ states,
@@ -1210,13 +1218,32 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float*
 }
 
 // ------------------------------------------------------------------------- dx
-template <int PT>
+// BF (bf16 inputs): the operands of the product over the state index are bf16 tiles read as matrix fragments of 8
+// adjacent columns; otherwise fp32 tiles.  `prod` (the dy * x products of the skip gradient) is its own small tile.
+template <int PT, bool BF>
 struct BwdDxSmem {
   static constexpr int LDPT = PT * 16 + 4;
+  static constexpr int LDK = NS + 8;
   float dys[CS * LDPT];
-  float bt[CS * LDN];       // B dt' exp2(last - cs) [m][n]; later dy*x products
-  float dss[PT * 16 * LDN]; // dS [p][n]
+  typename std::conditional<BF, uint16_t, float>::type bt[CS * (BF ? LDK : LDN)];        // B dt' exp2(last - cs) [m][n]
+  typename std::conditional<BF, uint16_t, float>::type dss[PT * 16 * (BF ? LDK : LDN)];  // dS [p][n]
+  float prod_own[BF ? CS * LDPT : 4];  // dy * x; with fp32 tiles it takes the place of `bt`
+  __device__ __forceinline__ float* prod() { return BF ? prod_own : reinterpret_cast<float*>(bt); }
+  static constexpr int LDPROD = BF ? LDPT : LDN;
 };
+template <int PT, int LD>
+__device__ __forceinline__ void pn_store_bf16(const PnRegs<PT>& r, uint16_t* dst, int tid = threadIdx.x) {
+  typedef PnRegs<PT> R;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    if (e < R::TOT) *(uint2*)(dst + pp * LD + c4) = make_uint2(pack_bf16(r.v[i][0], r.v[i][1]), pack_bf16(r.v[i][2], r.v[i][3]));
+  }
+}
+template <int LD>
+__device__ __forceinline__ bf8 frag8(const uint16_t* tile, int row, int g4, int t) {
+  return *(const bf8*)(tile + row * LD + 32 * t + 8 * g4);
+}
 
 // partD: (Bt*nc*H, P) per-unit sums over rows of dy*x
 template <int PT, bool IOB, bool DTB, bool FULL>
@@ -1224,9 +1251,9 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
                                                      const float* __restrict__ dstates,
                                                      const float* __restrict__ cabt, float* __restrict__ partD) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  typedef BwdDxSmem<PT> SM;
+  typedef BwdDxSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT;
+  constexpr int LDPT = SM::LDPT, LDK = SM::LDK, LDPR = SM::LDPROD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -1272,11 +1299,24 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
     {
       float dtp[16], cs[16], dummy[16];
       const float last = lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
+      if constexpr (IOB) {
+        float btv[16];
 #pragma unroll
-      for (int k = 0; k < 16; ++k)
-        s.bt[lane_row(k, g4) * LDN + wave * 16 + cm] = bv[k] * dtp[k] * ex2(last - cs[k]);
+        for (int k = 0; k < 16; k += 2) {
+          btv[k] = bv[k] * dtp[k] * ex2(last - cs[k]);
+          btv[k + 1] = bv[k + 1] * dtp[k + 1] * ex2(last - cs[k + 1]);
+          const unsigned h2 = pack_bf16(btv[k], btv[k + 1]);
+          s.bt[lane_row(k, g4) * LDK + wave * 16 + cm] = (uint16_t)h2;
+          s.bt[lane_row(k + 1, g4) * LDK + wave * 16 + cm] = (uint16_t)(h2 >> 16);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+          s.bt[lane_row(k, g4) * LDN + wave * 16 + cm] = bv[k] * dtp[k] * ex2(last - cs[k]);
+      }
     }
-    pn_store<PT>(sv, s.dss);
+    if constexpr (IOB) pn_store_bf16<PT, LDK>(sv, s.dss);
+    else pn_store<PT>(sv, s.dss);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
       vn = FULL || n < p.N;
@@ -1287,10 +1327,19 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
       pn_load<PT>(p, ds, n0 + NS, sv);
     }
     __syncthreads();
+    if constexpr (IOB) {
 #pragma unroll
-    for (int kb = 0; kb < NS; kb += 16)
+      for (int t = 0; t < 2; ++t) {
+        const bf8 a = frag8<LDK>(s.bt, wave * 16 + cm, g4, t);
 #pragma unroll
-      for (int pt = 0; pt < PT; ++pt) mma16_mm(acc[pt], s.bt, LDN, wave * 16, s.dss, LDN, pt * 16, kb, lane);
+        for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma_bf(a, frag8<LDK>(s.dss, pt * 16 + cm, g4, t), acc[pt]);
+      }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < NS; kb += 16)
+#pragma unroll
+        for (int pt = 0; pt < PT; ++pt) mma16_mm(acc[pt], s.bt, LDN, wave * 16, s.dss, LDN, pt * 16, kb, lane);
+    }
     __syncthreads();
   }
   // dx[m][p] += sum_{l>=m} M[l][m] dy[l][p]
@@ -1307,7 +1356,7 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
 
   const TensorD& tx = p.x[u.dir];
   const TensorD& tdx = p.dx[u.dir];
-  float* prod = s.bt;  // [64][LDN] holds at least [64][16 PT]
+  float* prod = s.prod();  // [64][LDPR]
 #pragma unroll
   for (int pt = 0; pt < PT; ++pt) {
     int ox[4], odx[4];
@@ -1328,7 +1377,7 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
       const int l = wave * 16 + 4 * g4 + r, pp = pt * 16 + cm;
       const float dyv = s.dys[l * LDPT + pp];
       v[r] = fmaf(dcoef, dyv, acc[pt][r]);
-      prod[l * LDN + pp] = dyv * xv[r];
+      prod[l * LDPR + pp] = dyv * xv[r];
     }
     gstore<IOB, 4>(const_cast<void*>(tdx.ptr), (long)u.b * tdx.s0 + (long)u.h * tdx.s2, odx, v);
   }
@@ -1336,7 +1385,7 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
     __syncthreads();
     if (tid < PT * 16) {
       float sum = 0.0f;
-      for (int l = 0; l < CS; ++l) sum += prod[l * LDN + tid];
+      for (int l = 0; l < CS; ++l) sum += prod[l * LDPR + tid];
       if (tid < p.P) partD[(((long)u.bt * p.nc + u.c) * p.H + u.h) * p.P + tid] = sum;
     }
   }
@@ -1431,7 +1480,7 @@ int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t s
 int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* dm, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
-    const size_t sm = sizeof(BwdStSmem<PT_>);
+    const size_t sm = sizeof(BwdStSmem<PT_, IOB_>);
     if (int e = set_lds(k_bwd_dstates<PT_, IOB_, DTB_, FULL_>, sm)) return e;
     hipLaunchKernelGGL((k_bwd_dstates<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
   });
@@ -1496,7 +1545,7 @@ int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const f
                   hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
-    const size_t sm = sizeof(BwdDxSmem<PT_>);
+    const size_t sm = sizeof(BwdDxSmem<PT_, IOB_>);
     if (int e = set_lds(k_bwd_dx<PT_, IOB_, DTB_, FULL_>, sm)) return e;
     hipLaunchKernelGGL((k_bwd_dx<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
   });

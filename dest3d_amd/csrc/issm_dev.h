@@ -365,8 +365,9 @@ __device__ __forceinline__ void lp_store_split_t(const float (&v)[CS * PT * 16 /
 // acc[pt] += (tile^T)(16 pt .. +15, :) . b  for a product over the 64 chunk rows whose B operand is the lane's
 // 16 column-lane values (k = 4J + j <-> row 16J + 4 g4 + j): two K = 32 steps, step t <-> values 8t .. 8t+7.
 // `b(k)` yields the lane's value k (evaluated step by step, so that only eight are live at a time).
-// (SPLIT = false: the operands are used as rounded to bf16 -- one instruction per step instead of three.)
-template <int PT, int LD, bool SPLIT = true, typename F>
+// MODE 1: both operands as (hi, lo) pairs, three instructions per step.  MODE 0: both operands rounded to bf16, one
+// instruction.  MODE 2: the tile is exact in bf16 (bf16 inputs), only b is split: two instructions.
+template <int PT, int LD, int MODE = 1, typename F>
 __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t* thi, const uint16_t* tlo, F b,
                                                    int cm, int g4) {
 #pragma unroll
@@ -375,7 +376,7 @@ __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t
 #pragma unroll
     for (int j = 0; j < 8; ++j) w[j] = b(8 * t + j);
     bf8 bh, bl;
-    if (SPLIT) {
+    if (MODE != 0) {
       split8(w, bh, bl);
     } else {
 #pragma unroll
@@ -384,13 +385,28 @@ __device__ __forceinline__ void rows_product_split(f4 (&acc)[PT], const uint16_t
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) {
       const bf8 ah = split_frag<LD>(thi, pt * 16 + cm, g4, t);
-      if (SPLIT) {
+      if (MODE == 1) {
         const bf8 al = split_frag<LD>(tlo, pt * 16 + cm, g4, t);
         acc[pt] = mfma_split(ah, al, bh, bl, acc[pt]);
+      } else if (MODE == 2) {
+        acc[pt] = mfma_bf(ah, bl, acc[pt]);
+        acc[pt] = mfma_bf(ah, bh, acc[pt]);
       } else {
         acc[pt] = mfma_bf(ah, bh, acc[pt]);
       }
     }
+  }
+}
+
+// a (64 x 16 PT) register tile (layout of lp_load) as bf16 into LDS dst[l][p]
+template <int PT, int LD>
+__device__ __forceinline__ void lp_store_bf(const float (&v)[CS * PT * 16 / NTHREADS], uint16_t* dst, int tid) {
+  constexpr int G4 = 4 * PT;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS;
+    *(uint2*)(dst + (e4 / G4) * LD + (e4 % G4) * 4) =
+        make_uint2(pack_bf16(v[4 * i], v[4 * i + 1]), pack_bf16(v[4 * i + 2], v[4 * i + 3]));
   }
 }
 

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-      rows_product_split<PT, LDT, SPLIT>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
+      rows_product_split<PT, LDT, SPLIT ? 1 : 2>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
       const int nn = n0 + wave * 16 + cm;
       if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
@@ -395,21 +395,44 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
 }
 
 // ------------------------------------------------------------------ chunk scan
-template <int PT>
+// BF (bf16 inputs): the operands of the product over the state index are bf16 tiles read as matrix fragments of 8
+// adjacent columns; otherwise fp32 tiles.
+template <int PT, bool BF>
 struct FwdScanSmem {
   static constexpr int LDPT = PT * 16 + 4;
-  float xs[CS * LDPT];      // x [s][p]
-  float ct[CS * LDN];       // C * exp2(cs) [l][n]
-  float hs[PT * 16 * LDN];  // H [p][n]
+  static constexpr int LDK = NS + 8;  // row stride of the bf16 tiles
+  float xs[CS * LDPT];                                          // x [s][p]
+  typename std::conditional<BF, uint16_t, float>::type ct[CS * (BF ? LDK : LDN)];       // C * exp2(cs) [l][n]
+  typename std::conditional<BF, uint16_t, float>::type hs[PT * 16 * (BF ? LDK : LDN)];  // H [p][n]
 };
+// a (16 PT x 64) slab of fp32 values (layout of pn_load) rounded to bf16 into LDS dst[p][col], row stride LD
+template <int PT, int LD>
+__device__ __forceinline__ void pn_store_bf(const PnRegs<PT>& r, uint16_t* dst, int tid = threadIdx.x) {
+  typedef PnRegs<PT> R;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    if (e < R::TOT) *(uint2*)(dst + pp * LD + c4) = make_uint2(pack_bf16(r.v[i][0], r.v[i][1]), pack_bf16(r.v[i][2], r.v[i][3]));
+  }
+}
+// the lane's 16 values of one column -> column `col` of a [64][LD] bf16 tile
+template <int LD>
+__device__ __forceinline__ void col_store_bf(const float (&v)[16], uint16_t* dst, int g4, int col) {
+#pragma unroll
+  for (int k = 0; k < 16; k += 2) {
+    const unsigned h2 = pack_bf16(v[k], v[k + 1]);
+    dst[lane_row(k, g4) * LD + col] = (uint16_t)h2;
+    dst[lane_row(k + 1, g4) * LD + col] = (uint16_t)(h2 >> 16);
+  }
+}
 
 template <int PT, bool IOB, bool DTB, bool FULL>
 __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states,
                                                          const float* __restrict__ cabt, float* __restrict__ out_x) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  typedef FwdScanSmem<PT> SM;
+  typedef FwdScanSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT;
+  constexpr int LDPT = SM::LDPT, LDK = SM::LDK;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -453,10 +476,18 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     {
       float dtp[16], cs[16], dummy[16];
       lane_prep<false>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dummy);
+      if constexpr (IOB) {
+        float ctv[16];
 #pragma unroll
-      for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
+        for (int k = 0; k < 16; ++k) ctv[k] = cv[k] * ex2(cs[k]);
+        col_store_bf<LDK>(ctv, s.ct, g4, wave * 16 + cm);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
+      }
     }
-    pn_store<PT>(hv, s.hs);
+    if constexpr (IOB) pn_store_bf<PT, LDK>(hv, s.hs);
+    else pn_store<PT>(hv, s.hs);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
       vn = FULL || n < p.N;
@@ -469,10 +500,21 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     __syncthreads();
     // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows.  (fp32 product: both operands change with
     // every slice and are used once or twice, so a bf16 split costs more vector work than it saves -- measured)
+    if constexpr (IOB) {
+      // bf16 inputs: one rounding of C exp(cs) and of the entry state to bf16 (the reference stores the entry states
+      // in the input dtype and casts its dot operands, issm_combined.py:87, issm_chunk_scan.py:149-190)
 #pragma unroll
-    for (int kb = 0; kb < NS; kb += 16)
+      for (int t = 0; t < 2; ++t) {
+        const bf8 a = op_frag<LDK>(s.ct, wave * 16 + cm, g4, t);
 #pragma unroll
-      for (int pt = 0; pt < PT; ++pt) mma16_mm(acc[pt], s.ct, LDN, wave * 16, s.hs, LDN, pt * 16, kb, lane);
+        for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma_bf(a, op_frag<LDK>(s.hs, pt * 16 + cm, g4, t), acc[pt]);
+      }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < NS; kb += 16)
+#pragma unroll
+        for (int pt = 0; pt < PT; ++pt) mma16_mm(acc[pt], s.ct, LDN, wave * 16, s.hs, LDN, pt * 16, kb, lane);
+    }
     __syncthreads();
   }
   // y[l][p] += sum_{s<=l} M[l][s] x[s][p]; rows of this wave only need s < 16(wave+1)
@@ -550,7 +592,7 @@ int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream
 int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float* out_x, hipStream_t st) {
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
-    const size_t sm = sizeof(FwdScanSmem<PT_>);
+    const size_t sm = sizeof(FwdScanSmem<PT_, IOB_>);
     if (int e = set_lds(k_chunk_scan<PT_, IOB_, DTB_, FULL_>, sm)) return e;
     hipLaunchKernelGGL((k_chunk_scan<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
   });
