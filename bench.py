@@ -7,11 +7,17 @@ A / D / initial states), fp32 inputs, synthetic seeded data already resident in 
 One "step" = one forward + backward call of the operator.  `value` is microseconds per step.
 
 Besides the driver's JSON contract the line carries
-  roofline      the dominant kernel's achieved fraction of its bound (live HIP-event timing)
-  cpu_baseline  the oracle's chunked pure-PyTorch formulation timed on the host cores
-  stages_us     average duration of every kernel of the step
-  variants_us   fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants (also at the
-                detector's head dimension 36), and of one whole detector layer around the scan
+  roofline           the dominant kernel's achieved fraction of its bound (live HIP-event timing); `traffic` is read
+                     from the committed rocprofv3 summary under profiles/
+  cpu_baseline       the oracle's chunked pure-PyTorch formulation timed on the host cores (fwd+bwd sample scaled to
+                     the workload, and configs[0]'s own forward-only B=2 figure)
+  stages_us, stage_roofline, step_roofline   every kernel of the step against the roofline that bounds it, and the
+                     whole step against its compulsory traffic and FLOPs
+  variants_us        fwd+bwd time of the unidirectional fp32 / bf16 and bidirectional bf16 variants (also at the
+                     detector's head dimension 36), of configs[3] (long sequence) and configs[4] (large state), and
+                     of one whole detector layer around the scan
+  variant_rooflines  the same per-kernel and whole-step rooflines for the bf16 headline variant, configs[3], configs[4]
+`--workload NAME` runs one scan workload alone (the command the kernel traces under profiles/ are taken with).
 """
 import argparse
 import ctypes as C
@@ -25,14 +31,30 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 SHAPE = dict(B=8, L=1024, H=8, P=32, N=256, G=1, cs=64)
 
 
-def make_problem(torch, ndir, dtype, seed=1235):
+# The scan workloads this script can time: the headline (configs[1], fp32), its variants, and the baseline's other scan
+# configurations (configs[3]: long sequence; configs[4]: large state).  shape overrides SHAPE.
+WORKLOADS = {
+    "headline": dict(shape={}, ndir=2, dtype="float32"),
+    "uni_fp32": dict(shape={}, ndir=1, dtype="float32"),
+    "uni_bf16": dict(shape={}, ndir=1, dtype="bfloat16"),
+    "bidir_bf16": dict(shape={}, ndir=2, dtype="bfloat16"),
+    "bidir_bf16_headdim36": dict(shape=dict(P=36), ndir=2, dtype="bfloat16"),   # the detector's head size
+    "long_sequence_B2_L16384_uni_bf16": dict(shape=dict(B=2, L=16384), ndir=1, dtype="bfloat16"),
+    "large_state_B16_L2048_H16_P64_N512_bidir_fp32": dict(shape=dict(B=16, L=2048, H=16, P=64, N=512), ndir=2,
+                                                          dtype="float32", h0_std=0.1),
+}
+
+
+def make_problem(torch, shape, ndir, dtype, seed=1235, h0_std=0.0):
     from oracle.issm_ref import make_inputs   # data generator only (shared with the tests)
-    I = make_inputs(SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed)
+    SHAPE = shape
+    I = make_inputs(SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed, h0_std=h0_std)
     g = torch.Generator().manual_seed(seed + 1)
     dev = "cuda"
     t = dict(x=[I["x"]], B=[I["B"]], C=[I["C"]], dy=[I["dy"]], dfinal=[I["dfinal"]])
@@ -46,7 +68,7 @@ def make_problem(torch, ndir, dtype, seed=1235):
     out["dt"] = torch.nn.functional.softplus(I["dt_raw"]).to(dev, dtype)   # module call pattern: dt already softplus'ed
     out["A"] = I["A"].to(dev)
     out["D"] = I["D"].to(dev)
-    out["h0"] = torch.zeros(SHAPE["B"], SHAPE["H"], SHAPE["P"], SHAPE["N"], device=dev)
+    out["h0"] = I["h0"].to(dev)
     return out
 
 
@@ -54,12 +76,14 @@ class Runner:
     """Forward + backward through the C ABI with preallocated buffers (no autograd, no allocation
     in the timed region): exactly the kernels ISSMChunkScanCombinedFn launches."""
 
-    def __init__(self, torch, ndir, dtype):
+    def __init__(self, torch, ndir, dtype, shape=None, h0_std=0.0):
         from dest3d_amd import _lib as L
         from dest3d_amd.issm_combined import _Problem
         self.torch, self.L, self.lib = torch, L, L.load()
         self.ndir = ndir
-        t = self.t = make_problem(torch, ndir, dtype)
+        SHAPE = self.shape = dict(globals()["SHAPE"], **(shape or {}))
+        self.elt = 2 if dtype == torch.bfloat16 else 4
+        t = self.t = make_problem(torch, SHAPE, ndir, dtype, h0_std=h0_std)
         self.prob = _Problem(t["x"], t["dt"], t["A"], t["B"], t["C"], SHAPE["cs"], t["D"], [None] * ndir, None,
                              t["h0"], None, False, (0.0, float("inf")))
         a = self.a = self.prob.args()
@@ -152,7 +176,7 @@ class Runner:
         back-to-back launches of that kernel."""
         torch, lib, a = self.torch, self.lib, self.a
         nd = self.ndir
-        B_, L_, H, P, N = (SHAPE[k] for k in ("B", "L", "H", "P", "N"))
+        B_, L_, H, P, N = (self.shape[k] for k in ("B", "L", "H", "P", "N"))
         nc = math.ceil(L_ / 64)
         Bt = B_ * nd
         f = lambda *s: torch.zeros(*s, device="cuda")
@@ -185,52 +209,96 @@ class Runner:
         return res
 
 
-# Memory traffic per launch at the headline workload, from two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the
-# plain 256 MiB copy of --calib-copy (fetch x2.000, write x1.000); the summary is kept under profiles/.
-# k_bwd_chunk is launched once per direction: the figure is per launch.  Override with --traffic.
-MEASURED_TRAFFIC_BYTES = {
-    "chunk_local": 208.0e6, "state_passing_fwd": 162.6e6, "chunk_scan": 210.2e6, "bwd_dstates": 206.6e6,
-    "state_passing_bwd": 214.0e6, "bwd_chunk": 301.3e6, "bwd_dx": 244.3e6,
-}
+KERNEL_OF_STAGE = {"chunk_local": "k_chunk_local", "state_passing_fwd": "k_state_fwd_full", "chunk_scan": "k_chunk_scan",
+                   "bwd_dstates": "k_bwd_dstates", "state_passing_bwd": "k_state_bwd_full", "bwd_chunk": "k_bwd_chunk",
+                   "bwd_dx": "k_bwd_dx", "bwd_reduce": "k_bwd_reduce"}
 
 
-def stage_work(ndir):
+def measured_traffic(stage):
+    """HBM bytes per launch of a stage's kernel at the headline workload, as the committed profile summary holds it
+    (profiles/issm_fwd_bwd_bidir_fp32_hbm_traffic.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled by
+    the same counters on a plain copy; last column of the kernel's row); None if the summary has no such row."""
+    import re
+    path = os.path.join(ROOT, "profiles", "issm_fwd_bwd_bidir_fp32_hbm_traffic.md")
+    pat = re.compile(KERNEL_OF_STAGE.get(stage, stage) + r"\b")
+    try:
+        for row in open(path):
+            cells = [c.strip() for c in row.strip().strip("|").split("|")]
+            if len(cells) >= 4 and pat.search(cells[0]):
+                return float(cells[-1]) * 1e6
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def stage_work(ndir, shape=None, elt=4):
     """Algorithmic FLOPs (2*MAC; exps not counted) and algorithmic bytes (every operand read once, every result
-    written once, in the run's 4-byte types; dt counted once for both directions) per launch of each kernel."""
-    B_, L_, H, P, N, G, cs = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "G", "cs"))
+    written once; caller tensors in their `elt`-byte type, intermediates fp32; dt counted once for both directions)
+    per launch of each kernel, and the same for the whole step ("step": compulsory bytes only -- inputs read once in
+    each pass, outputs and gradients written once)."""
+    SHAPE_ = dict(SHAPE, **(shape or {}))
+    B_, L_, H, P, N, G = (SHAPE_[k] for k in ("B", "L", "H", "P", "N", "G"))
+    cs = 64
     U = B_ * ndir * H * math.ceil(L_ / cs)
     tri = cs * (cs + 1) // 2
     E_cs, E_st = U * P * N, B_ * ndir * H * P * N          # chunk states; initial / final states
     E_x, E_bc = ndir * B_ * L_ * H * P, ndir * B_ * L_ * G * N   # x / y / dy / dx; B, C and their gradients
     E_dt, E_m, E_v = B_ * L_ * H * N, U * cs * cs, U * N   # dt / ddt; intra-chunk matrix M / dM; per-chunk vectors
-    return {
+    s = elt
+    w = {
         # reads dt, x, B, C; writes chunk-local end states S, M, the chunks' total decay
-        "chunk_local": (2 * U * (cs * P * N + tri * N), 4 * (E_dt + E_x + 2 * E_bc + E_cs + E_m + E_v)),
+        "chunk_local": (2 * U * (cs * P * N + tri * N), s * (E_dt + E_x + 2 * E_bc) + 4 * (E_cs + E_m + E_v)),
         # reads dt, C, x, states H, M; writes y
-        "chunk_scan": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + E_x + E_cs + E_m + E_x)),
+        "chunk_scan": (2 * U * (cs * P * N + tri * P), s * (E_dt + E_bc + 2 * E_x) + 4 * (E_cs + E_m)),
         # reads dt, C, dy, x; writes dH, dM
-        "bwd_dstates": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + 2 * E_x + E_cs + E_m)),
-        # both launches: read dt, x, dy, B, C, H, dS, dM, g_last; write ddt, dB, dC, the dA / ddt_bias partials
+        "bwd_dstates": (2 * U * (cs * P * N + tri * P), s * (E_dt + E_bc + 2 * E_x) + 4 * (E_cs + E_m)),
+        # all launches: read dt, x, dy, B, C, H, dS, dM, g_last; write ddt, dB, dC, the dA / ddt_bias partials
         "bwd_chunk": (2 * U * (2 * cs * P * N + 2 * tri * N),
-                      4 * (E_dt + 2 * E_x + 2 * E_bc + 2 * E_cs + E_m + E_v + E_dt + 2 * E_bc + 2 * E_v)),
+                      s * (2 * E_dt + 2 * E_x + 4 * E_bc) + 4 * (2 * E_cs + E_m + 3 * E_v)),
         # reads dt, B, dy, x, dS, M; writes dx
-        "bwd_dx": (2 * U * (cs * P * N + tri * P), 4 * (E_dt + E_bc + 2 * E_x + E_cs + E_m + E_x)),
+        "bwd_dx": (2 * U * (cs * P * N + tri * P), s * (E_dt + E_bc + 3 * E_x) + 4 * (E_cs + E_m)),
         "state_passing_fwd": (0, 4 * (2 * E_cs + U * N + 2 * E_st)),
         "state_passing_bwd": (0, 4 * (3 * E_cs + 2 * U * N + 2 * E_st)),
     }
+    # whole step, compulsory traffic only: every caller tensor read once per pass, every output and gradient written
+    # once, each direction counted with its own read of dt and initial states (a lower bound would share them)
+    E_dtd = ndir * E_dt
+    fwd_rd = s * (E_x + 2 * E_bc + E_dtd + E_st)
+    fwd = fwd_rd + s * E_x + 4 * E_st
+    bwd = fwd_rd + s * E_x + 4 * E_st + s * (E_x + 2 * E_bc + E_dtd + E_st)
+    w["step"] = (sum(f for f, _ in w.values()), fwd + bwd)
+    return w
 
 
-def stage_bound(flops, nbytes, us):
+def stage_bound(flops, nbytes, us, elt=4):
     """The roofline that bounds a stage is the one with the longer minimum time; returns (bound, achieved in the
-    bound's unit, fraction of its peak, {mfma fraction, hbm fraction})."""
+    bound's unit, fraction of its peak, {mfma fraction, hbm fraction}).  The matrix peak is the one of the inputs' type:
+    fp32 (157.3 TFLOP/s) for fp32 inputs, bf16 (2.5 PFLOP/s) for bf16 inputs -- with those every stage is HBM-bound."""
     t = us * 1e-6
-    f_mfma = flops / t / (PEAK_FP32_MFMA_TFLOPS * 1e12)
+    peak = PEAK_BF16_MFMA_TFLOPS if elt == 2 else PEAK_FP32_MFMA_TFLOPS
+    f_mfma = flops / t / (peak * 1e12)
     f_hbm = nbytes / t / (PEAK_HBM_GBS * 1e9)
     both = {"mfma_frac": round(f_mfma, 4), "hbm_frac": round(f_hbm, 4)}
     if f_mfma >= f_hbm:
         return "mfma", flops / t / 1e12, f_mfma, both
     return "hbm", nbytes / t / 1e9, f_hbm, both
+
+
+def workload_report(run, step_us, reps=20):
+    """Per-kernel durations of a workload with the roofline that bounds each (the one with the longer minimum time:
+    fp32 matrix peak for the FLOPs, HBM peak for the bytes), and the same for the whole step on its compulsory bytes."""
+    stages = run.stage_times(reps)
+    work = stage_work(run.ndir, run.shape, run.elt)
+    per_stage = {}
+    for k, (fl, nb) in work.items():
+        if k == "step":
+            continue
+        b, _, fr, both = stage_bound(fl, nb, stages[k], run.elt)
+        per_stage[k] = {"us": round(stages[k], 2), "bound": b, "frac": round(fr, 4), **both}
+    b, ach, fr, both = stage_bound(*work["step"], step_us, run.elt)
+    return {"stages_us": {k: round(v, 2) for k, v in stages.items()}, "stage_roofline": per_stage,
+            "step_roofline": {"us": round(step_us, 2), "gflop": round(work["step"][0] / 1e9, 2),
+                              "compulsory_mb": round(work["step"][1] / 1e6, 1), "bound": b, "frac": round(fr, 4), **both}}
 
 
 def cpu_baseline(torch):
@@ -251,8 +319,16 @@ def cpu_baseline(torch):
         y, fin = R.issm_scan_chunked(*ins, SHAPE["cs"])
         ((y * I["dy"]).sum() + (fin * I["dfinal"]).sum()).backward()
         best = min(best, time.perf_counter() - t0)
+    # configs[0] as BASELINE.json states it: forward only, B=2, the same formulation, no gradient bookkeeping
+    with torch.no_grad():
+        fwd = float("inf")
+        for _ in range(2):
+            t0 = time.perf_counter()
+            R.issm_scan_chunked(*[t.detach() for t in ins], SHAPE["cs"])
+            fwd = min(fwd, time.perf_counter() - t0)
     return {"value": best * 8 * 1e6, "unit": "us/call", "cores": cores, "kind": "port",
-            "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional"}
+            "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional",
+            "config0_forward_only_B2_us": round(fwd * 1e6, 1)}
 
 
 def time_box_dist_layer(torch, steps=10, warmup=3):
@@ -436,6 +512,8 @@ def main():
                     help="time only the backbone's point-set operators and print their JSON line (ms per call)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="run only this scan workload's forward + backward step loop and print its JSON line")
     ap.add_argument("--traffic", type=float, default=None,
                     help="measured HBM bytes per launch of the dominant kernel (from rocprofv3 --pmc), echoed into roofline.traffic")
     args = ap.parse_args()
@@ -467,44 +545,40 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if args.workload:
+        # one workload's step loop only (what the profiles under profiles/ are taken from)
+        spec = WORKLOADS[args.workload]
+        r = Runner(torch, spec["ndir"], getattr(torch, spec["dtype"]), spec["shape"], spec.get("h0_std", 0.0))
+        us = r.time_steps(args.steps, args.warmup)
+        print(json.dumps({"workload": args.workload, "us_per_step": round(us, 2), "steps": args.steps,
+                          "warmup": args.warmup, **({} if args.no_variants else workload_report(r, us))}))
+        return
     run = Runner(torch, 2, torch.float32)
     us = run.time_steps(args.steps, args.warmup)
     pct = run.step_percentiles(max(args.steps, 20))
-    stages = run.stage_times()
+    rep = workload_report(run, us)
+    stages, per_stage = rep["stages_us"], rep["stage_roofline"]
     work = stage_work(2)
     dom = max((k for k in stages if k in work), key=lambda k: stages[k])
     bound, achieved, frac, _ = stage_bound(*work[dom], stages[dom])
     roof = {"bound": bound, "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS if bound == "mfma" else PEAK_HBM_GBS,
             "unit": "TFLOP/s" if bound == "mfma" else "GB/s", "frac": frac, "traffic": None, "kernel": dom}
-    roof["traffic"] = args.traffic if args.traffic is not None else MEASURED_TRAFFIC_BYTES.get(dom)
-    per_stage = {}
-    for k, (fl, nb) in work.items():
-        b, _, fr, both = stage_bound(fl, nb, stages[k])
-        per_stage[k] = {"us": round(stages[k], 2), "bound": b, "frac": round(fr, 4), **both}
-    variants = {}
+    roof["traffic"] = args.traffic if args.traffic is not None else measured_traffic(dom)
+    variants, variant_rooflines = {}, {}
     if not args.no_variants:
         variants["headline_as_hip_graph_replay"] = round(run.time_graph_replays(args.steps, 5), 2)
-        for name, nd, dt, pdim in (("uni_fp32", 1, torch.float32, 32), ("uni_bf16", 1, torch.bfloat16, 32),
-                                   ("bidir_bf16", 2, torch.bfloat16, 32),
-                                   ("bidir_bf16_headdim36", 2, torch.bfloat16, 36)):  # the detector's head size
-            SHAPE["P"] = pdim
-            r = Runner(torch, nd, dt)
-            variants[name] = round(r.time_steps(max(args.steps // 2, 5), 5), 2)
-            del r
-        SHAPE["P"] = 32
-        # the other scan configurations of the baseline: long sequence (B 2, L 16384, bf16, one direction) and
-        # large state (B 16, L 2048, H 16, P 64, N 512, fp32, both directions)
-        keep = dict(SHAPE)
-        for name, shp, nd, dt in (("long_sequence_B2_L16384_uni_bf16", dict(B=2, L=16384), 1, torch.bfloat16),
-                                  ("large_state_B16_L2048_H16_P64_N512_bidir_fp32",
-                                   dict(B=16, L=2048, H=16, P=64, N=512), 2, torch.float32)):
-            SHAPE.update(shp)
-            r = Runner(torch, nd, dt)
-            variants[name] = round(r.time_steps(5, 2), 2)
+        del run
+        for name, spec in WORKLOADS.items():
+            if name == "headline":
+                continue
+            big = bool(spec["shape"].get("L", 0) > 4096 or spec["shape"].get("N", 0) > 256)
+            r = Runner(torch, spec["ndir"], getattr(torch, spec["dtype"]), spec["shape"], spec.get("h0_std", 0.0))
+            v = r.time_steps(5 if big else max(args.steps // 2, 5), 2 if big else 5)
+            variants[name] = round(v, 2)
+            if name in ("bidir_bf16", "long_sequence_B2_L16384_uni_bf16", "large_state_B16_L2048_H16_P64_N512_bidir_fp32"):
+                variant_rooflines[name] = workload_report(r, v, reps=5 if big else 20)
             del r
             torch.cuda.empty_cache()
-            SHAPE.clear()
-            SHAPE.update(keep)
         variants["detector_layer_bf16_fwd_bwd"] = round(time_module_layer(torch), 2)
         variants["detector_layer_bf16_fwd_bwd_as_hip_graph"] = round(time_module_layer(torch, as_graph=True), 2)
         variants["detector_layer_fp32_fwd_bwd"] = round(time_module_layer(torch, dtype=torch.float32), 2)
@@ -517,9 +591,11 @@ def main():
                                "(fused), fp32 I/O, fp32 MFMA accumulate"},
         "roofline": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in roof.items()},
         "step_us_percentiles": pct,
-        "stages_us": {k: round(v, 2) for k, v in stages.items()},
+        "stages_us": stages,
         "stage_roofline": per_stage,
+        "step_roofline": rep["step_roofline"],
         "variants_us": variants,
+        "variant_rooflines": variant_rooflines,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch)
