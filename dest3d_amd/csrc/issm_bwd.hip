@@ -302,13 +302,25 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd(KP p, const float* __res
 // for the head's last row: it issues the same loads (so that every load of the loop is unconditional) but stores
 // nothing and adds nothing to the column sums -- what a stand-in computes is never used, so it does not matter that
 // the row's owner overwrites dH with dS while the stand-in's prefetches of that row are in flight.
-template <int NQ, int KM, int R>
+template <int NQ, int KM, int R, bool BATCH>
 __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* __restrict__ states,
                                                              const float* __restrict__ cs_last,
                                                              float* __restrict__ dstates, float* __restrict__ g_last,
                                                              float* __restrict__ dh0_dir) {
   constexpr int NCOL = NQ * 4, PGN = NTHREADS / NQ;
-  __shared__ __align__(16) float red2[2][PGN * NCOL];  // two buffers, used in turn: one barrier per step
+  // The column sums g = sum_p H dS need the rows of all four waves.  Two ways to add them up:
+  //  - per step (BATCH = false): every thread leaves its partial sums in local memory and, behind the step's barrier,
+  //    the first wave adds each column's PGN of them.  That exchange (local-memory round trips one after the other)
+  //    lies on the path from one chunk to the next, which a chip full of workgroups hides: from 256 workgroups on
+  //    this form is as fast as the other or up to 10 % faster;
+  //  - K steps at once (BATCH = true): the steps only deposit partial sums -- 16 per column: a wave's lanes of one
+  //    16-lane row share a column quad, after one in-row rotation for NQ = 8 -- and one thread per (step, column)
+  //    adds them behind one barrier per K steps.  With few workgroups walking hundreds of chunks the pace of the
+  //    exchange is the run time: 1.3-1.6x faster up to 128 workgroups (batch 2, 256 chunks: 145 -> 110 us).
+  // Two buffers, used in turn, either way.
+  constexpr int K = !BATCH ? 1 : R * NCOL <= NTHREADS ? R : R / 2;
+  static_assert(R % K == 0 && K * NCOL <= NTHREADS && (NQ == 8 || NQ == 16), "batches of K steps tile the ring");
+  __shared__ __align__(16) float red2[2][BATCH ? K * NCOL * 16 : PGN * NCOL];
   int par = 0;
   const int nsl = p.N / NCOL;
   int bid = blockIdx.x;
@@ -319,6 +331,8 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   const int b = bt / p.ndir, dir = bt % p.ndir;
   const int tid = threadIdx.x, pg = tid / NQ, nq = tid % NQ;
   const int n = ns * NCOL + nq * 4;
+  const int part = (tid >> 6) * 4 + ((tid & 63) >> 4);  // (wave, 16-lane row): which of a column's 16 partial sums
+  const bool deposits = NQ == 16 || !(tid & 8);
   long rowk[KM];   // offsets of the thread's rows
   bool own[KM];    // a row of its own (stores, takes part in the column sums) or a stand-in (loads only)
 #pragma unroll
@@ -336,7 +350,7 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
   const float* hp = states + st_off(p, bt, p.nc, h);      // H_{c+1}, c = nc - 1
   float* dd = dstates + dst_off(p, bt, p.nc - 1, h);      // dH_c in, dS_c out
   const float* cl = cs_last + vec_off(p, bt, p.nc - 1, h) + n;
-  float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;
+  float* gl = g_last + vec_off(p, bt, p.nc - 1, h) + ns * NCOL;  // of the first step of the current batch
   // Operands of R chunks in R register slots: the one being used and the next R - 1, the last of which is requested
   // at the top of a step (the final steps request chunk 0 again: in range, unused).  Step j = nc-1-c uses slot
   // j % R; the loop is unrolled over the slots so that none is ever copied (a copy would wait for its load).
@@ -366,30 +380,70 @@ __global__ __launch_bounds__(NTHREADS) void k_state_bwd_full(KP p, const float* 
         carry[k][j] = e[j] * carry[k][j] + dh[cur][k][j];
       }
     }
-    float* red = red2[par];
-    par ^= 1;
-    *(f4*)(red + pg * NCOL + nq * 4) = gp;
-    __syncthreads();  // the buffer is written again two steps later, after the next step's barrier
-    if (tid < 64) {
-      constexpr int PARTS = 64 / NCOL;
-      const int col = tid % NCOL, part = tid / NCOL;
-      float sum = 0.0f;
+    if (!BATCH) {
+      *(f4*)(red2[par] + pg * NCOL + nq * 4) = gp;
+    } else {
+      if (NQ == 8) {
+        // lanes l and l ^ 8 of a 16-lane row hold the same column quad: rotate the row by 8 and add
 #pragma unroll
-      for (int k = 0; k < PGN / PARTS; ++k) sum += red[(k * PARTS + part) * NCOL + col];
+        for (int j = 0; j < 4; ++j) {
+          const float own_sum = gp[j];  // a scalar copy: the bit cast below must not be applied to a vector element
+          gp[j] = own_sum + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                                                          0, __builtin_bit_cast(int, own_sum), 0x128, 0xf, 0xf, false));
+        }
+      }
+      if (deposits) {
+        // the 16 partial sums of a column are added in the order of their places, whatever lane filled them: the
+        // place is rotated by the column so that a wave's stores spread over the banks
+        float* red = red2[par] + ((cur % K) * NCOL + nq * 4) * 16;
 #pragma unroll
-      for (int d = NCOL; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
-      if (part == 0) gl[col] = sum;
+        for (int j = 0; j < 4; ++j) red[j * 16 + ((part + nq * 4 + j) & 15)] = gp[j];
+      }
     }
-    hp -= cstep; dd -= cstep; cl -= vstep; gl -= vstep;
+    hp -= cstep; dd -= cstep; cl -= vstep;
+  };
+  // The column sums of the batch's first cnt steps: thread = (step, column).
+  auto add_up = [&](int cnt) {
+    __syncthreads();  // the other buffer is filled next; this one again after the next barrier
+    if (!BATCH) {
+      if (tid < 64) {
+        // 64 lanes over NCOL columns: a lane sums every (64 / NCOL)-th row group of its column, then the lanes of a
+        // column (NCOL apart) are added
+        constexpr int PARTS = 64 / NCOL;
+        const int col = tid % NCOL, prt = tid / NCOL;
+        const float* red = red2[par];
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < PGN / PARTS; ++k) sum += red[(k * PARTS + prt) * NCOL + col];
+#pragma unroll
+        for (int d = NCOL; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
+        if (prt == 0) gl[col] = sum;
+      }
+    } else if (tid < cnt * NCOL) {
+      const f4* r = (const f4*)(red2[par] + tid * 16);
+      const f4 a = r[0], b4 = r[1], c4 = r[2], d4 = r[3];
+      const f4 s4 = (a + b4) + (c4 + d4);
+      gl[-(long)(tid / NCOL) * vstep + tid % NCOL] = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    }
+    gl -= (long)cnt * vstep;
+    par ^= 1;
   };
   int c = p.nc - 1;
   for (; c >= R - 1; c -= R) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) step(i, (i + R - 1) % R, c - i);
+    for (int i = 0; i < R; ++i) {
+      step(i, (i + R - 1) % R, c - i);
+      if ((i + 1) % K == 0) add_up(K);
+    }
   }
 #pragma unroll
-  for (int i = 0; i < R - 1; ++i)
-    if (c - i >= 0) step(i, (i + R - 1) % R, c - i);  // uniform: the last nc % R chunks
+  for (int i = 0; i < R - 1; ++i) {  // uniform: the last nc % R chunks
+    if (c - i >= 0) {
+      step(i, (i + R - 1) % R, c - i);
+      if ((i + 1) % K == 0) add_up(K);
+      else if (c - i == 0) add_up(i % K + 1);
+    }
+  }
 #pragma unroll
   for (int k = 0; k < KM; ++k)
     if (own[k]) *(f4*)(dh0_dir + (((long)dir * p.B + b) * p.H + h) * p.P * p.N + rowk[k]) = carry[k];
@@ -1492,17 +1546,20 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
   // One workgroup walks the chunks of its columns one after the other.  Complete shapes take the variant without
   // conditional accesses; with few (batch, head) pairs narrower column slices put more workgroups on the chip.
   const int wide = p.B * p.ndir * p.H * ((p.N + 63) / 64);
-#define ISSM_STATE_BWD_FULL(NQ_, KM_, R_)                                                                                  \
-  hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_, R_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), 0, st, p, \
-                     states, cs_last, dstates, g_last, dh0_dir)
+#define ISSM_STATE_BWD_FULL(NQ_, KM_, R_, BATCH_)                                                                          \
+  hipLaunchKernelGGL((k_state_bwd_full<NQ_, KM_, R_, BATCH_>), dim3(p.B * p.ndir * p.H * (p.N / (4 * NQ_))), dim3(NTHREADS), \
+                     0, st, p, states, cs_last, dstates, g_last, dh0_dir)
   if (p.N % 32 == 0 && (wide < 256 || p.N % 64 != 0)) {
-    if (p.P <= 32) ISSM_STATE_BWD_FULL(8, 1, 6); else ISSM_STATE_BWD_FULL(8, 2, 4);
+    // few workgroups walking many chunks: the column sums of several steps behind one barrier
+    const bool batch = p.B * p.ndir * p.H * (p.N / 32) <= 128 && p.nc >= 32;
+    if (p.P <= 32) { if (batch) ISSM_STATE_BWD_FULL(8, 1, 6, true); else ISSM_STATE_BWD_FULL(8, 1, 6, false); }
+    else { if (batch) ISSM_STATE_BWD_FULL(8, 2, 4, true); else ISSM_STATE_BWD_FULL(8, 2, 4, false); }
   } else if (p.N % 64 == 0) {
     switch ((p.P + 15) / 16) {
-      case 1: ISSM_STATE_BWD_FULL(16, 1, 3); break;
-      case 2: ISSM_STATE_BWD_FULL(16, 2, 3); break;
-      case 3: ISSM_STATE_BWD_FULL(16, 3, 3); break;
-      default: ISSM_STATE_BWD_FULL(16, 4, 3); break;
+      case 1: ISSM_STATE_BWD_FULL(16, 1, 3, false); break;
+      case 2: ISSM_STATE_BWD_FULL(16, 2, 3, false); break;
+      case 3: ISSM_STATE_BWD_FULL(16, 3, 3, false); break;
+      default: ISSM_STATE_BWD_FULL(16, 4, 3, false); break;
     }
   } else if (wide < 256) {
     const int blocks = p.B * p.ndir * p.H * ((p.N + 15) / 16);

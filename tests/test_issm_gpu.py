@@ -106,11 +106,15 @@ CASES = [
     (1, 128, 2, 36, 64, 1, dict(D="hp", z=True)),        # complete chunks / slices, ragged head dimension
     (2, 64, 2, 20, 128, 2, dict(softplus=False)),
     (1, 192, 1, 64, 64, 1, dict()),                       # complete tiles, widest head dimension
-    # state passing: 32-column slices with stand-in rows, 37 chunks (not a multiple of the six register slots)
+    # state passing: 32-column slices with stand-in rows, 37 chunks (six register slots, a last batch of one step)
     (1, 64 * 37, 2, 20, 64, 1, dict()),
     (1, 64 * 7 - 5, 1, 40, 96, 1, dict(D="hp")),          # two rows per thread, four slots, ragged last chunk
     (4, 64 * 5, 8, 36, 256, 1, dict(softplus=False)),    # 64-column slices, three slots, 5 chunks, P = 36
     (16, 70, 8, 16, 96, 1, dict()),                      # many workgroups, N a multiple of 32 but not of 64
+    # state passing, few workgroups and many chunks (column sums of several steps added up together): 35 chunks
+    # leave a last batch of five steps with one row per thread, of three with two rows per thread
+    (1, 64 * 35, 1, 32, 32, 1, dict(softplus=False)),
+    (1, 64 * 35 - 9, 1, 40, 32, 1, dict(D="h")),
 ]
 
 
