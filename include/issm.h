@@ -28,12 +28,16 @@
  *  - ndir = 2 runs the module's bidirectional pair (models/dest_module.py:565-575) in
  *    one call: direction 1 walks the same dt / A / D / h0 backwards in time with its
  *    own x / Bm / Cm and writes its outputs back in natural (un-flipped) time order.
- *  - Numerics: cumulative sums, decays, states and all accumulation are fp32 for every
- *    I/O dtype.  The products x^T.(B dt' decay), dy^T.(C decay), x.dS and dy.H are
- *    evaluated as three bf16 matrix products with fp32 accumulation on operands split
- *    into bf16 high and low parts (16 significand bits per operand; relative error of a
- *    product <= 2^-16); every other product is fp32.  Results are bit-reproducible
- *    from run to run (fixed-order reductions, no atomics).
+ *  - Numerics: cumulative sums, decays, dt', states and all accumulation are fp32 for every
+ *    I/O dtype.  With io_dtype = ISSM_F32 the products x^T.(B dt' decay), dy^T.(C decay),
+ *    x.dS, dy.H and the within-chunk matrix M of the forward are evaluated as three bf16
+ *    matrix products with fp32 accumulation on operands split into bf16 high and low parts
+ *    (16 significand bits per operand; relative error of a product <= 2^-16); every other
+ *    product is fp32.  With io_dtype = ISSM_BF16 every matrix product takes its operands
+ *    rounded once to bf16 (as the reference's kernels cast their dot operands to the input
+ *    dtype, issm_triton/issm_cabt_bmm.py:42-43), except x.dS and dy.H, whose fp32 state
+ *    operands enter as high and low parts.  Results are bit-reproducible from run to run
+ *    (fixed-order reductions, no atomics).
  *  - Strides: stride[1] * seqlen must stay below 2^30 elements (row byte offsets are 32-bit).
  */
 #ifndef ISSM_H
