@@ -81,6 +81,8 @@ class NormArgs(C.Structure):
         ("dx_row_stride", C.c_int64), ("dz_row_stride", C.c_int64),
         ("dw_partial", C.c_void_p), ("dw", C.c_void_p),
         ("stream", C.c_void_p),
+        ("layer_norm", C.c_int32), ("bias", C.c_void_p), ("mean", C.c_void_p),
+        ("db_partial", C.c_void_p), ("db", C.c_void_p),
     ]
 
 

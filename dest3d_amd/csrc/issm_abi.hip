@@ -412,6 +412,10 @@ static int norm_params(const issm_norm_args* a, NormP* p, bool bwd) {
   if (!bwd && !a->y) return fail(ISSM_E_NULL, "rmsnorm: y is NULL");
   if (bwd && (!a->dy || !a->dx || !a->dw_partial || !a->dw)) return fail(ISSM_E_NULL, "rmsnorm bwd: NULL buffer");
   if (bwd && a->z && !a->dz) return fail(ISSM_E_NULL, "rmsnorm bwd: dz is NULL");
+  if (a->layer_norm && !a->mean) return fail(ISSM_E_NULL, "layernorm: mean is NULL");
+  if (bwd && a->bias && (!a->db_partial || !a->db)) return fail(ISSM_E_NULL, "norm bwd with bias: db_partial/db is NULL");
+  if (a->bias && a->ncols > 8192 && !(a->ncols / gs == 1 && (a->ncols & 3) == 0 && a->ncols <= 1024))
+    return fail(ISSM_E_UNSUPPORTED, "norm with bias: ncols %d > 8192", a->ncols);
   p->rows = a->rows; p->ncols = a->ncols; p->gs = gs; p->ngroups = a->ncols / gs;
   p->dt = a->dtype; p->wdt = a->weight_dtype; p->nbg = a->norm_before_gate; p->eps = a->eps;
   p->x = a->x; p->z = a->z; p->w = a->w; p->xs = a->x_row_stride; p->zs = a->z_row_stride;
@@ -419,6 +423,7 @@ static int norm_params(const issm_norm_args* a, NormP* p, bool bwd) {
   p->dy = a->dy; p->dys = a->dy_row_stride; p->dx = a->dx; p->dz = a->dz; p->dxs = a->dx_row_stride;
   p->dzs = a->dz_row_stride; p->dw_partial = a->dw_partial; p->dw = a->dw;
   p->nblocks = issm_rmsnorm_bwd_blocks(a->rows);
+  p->ln = a->layer_norm ? 1 : 0; p->b = a->bias; p->mean = a->mean; p->db_partial = a->db_partial; p->db = a->db;
   return ISSM_OK;
 }
 
@@ -475,19 +480,23 @@ int issm_gated_rmsnorm_bwd_noalloc(const issm_norm_args* a) {
   issm_norm_args b = *a;
   float* scratch = nullptr;
   // sizes are checked before anything touches the device
-  if (b.rows > 0 && b.ncols > 0 &&
-      (int64_t)issm_rmsnorm_bwd_blocks(b.rows) * b.ncols > (int64_t)ISSM_NORM_SCRATCH_FLOATS)
+  const int64_t part = b.rows > 0 && b.ncols > 0 ? (int64_t)issm_rmsnorm_bwd_blocks(b.rows) * b.ncols : 0;
+  const int64_t need = part * (b.bias ? 2 : 1);  // the partial sums of dw, then those of db
+  if (need > (int64_t)ISSM_NORM_SCRATCH_FLOATS)
     return fail(ISSM_E_WORKSPACE,
-                "rmsnorm bwd without allocation: %d row blocks x %d columns = %lld floats of partial sums exceed the "
+                "rmsnorm bwd without allocation: %d row blocks x %d columns%s = %lld floats of partial sums exceed the "
                 "library's %d-float scratch array; use issm_gated_rmsnorm_bwd with a dw_partial buffer",
-                issm_rmsnorm_bwd_blocks(b.rows), b.ncols, (long long)issm_rmsnorm_bwd_blocks(b.rows) * b.ncols,
+                issm_rmsnorm_bwd_blocks(b.rows), b.ncols, b.bias ? " x 2 (weight and bias)" : "", (long long)need,
                 (int)ISSM_NORM_SCRATCH_FLOATS);
-  b.dw_partial = (float*)(uintptr_t)256;  // placeholder so that the shared validation sees a buffer; replaced below
+  // placeholders so that the shared validation sees buffers; replaced below
+  b.dw_partial = (float*)(uintptr_t)256;
+  b.db_partial = (float*)(uintptr_t)256;
   NormP p;
   int rc = norm_params(&b, &p, true);
   if (rc) return rc;
   if ((rc = norm_scratch_ptr(&scratch))) return rc;
   p.dw_partial = scratch;  // every launched block writes its whole row of partials before the sum reads it
+  p.db_partial = scratch + part;
   return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd_noalloc");
 }
 

@@ -76,6 +76,11 @@ struct NormP {
   float* dw_partial;
   float* dw;
   int nblocks;
+  int ln;           // LayerNorm statistics (mean subtracted) instead of RMS
+  const void* b;    // bias in the weight's dtype, or null
+  float* mean;
+  float* db_partial;
+  float* db;
 };
 
 // parameters of the serialization-code kernel (hilbert.hip)

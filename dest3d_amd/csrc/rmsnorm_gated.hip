@@ -1,7 +1,10 @@
-// Gated RMSNorm forward / backward for gfx950: one 64-lane wavefront per row group,
+// Gated RMSNorm / LayerNorm forward and backward for gfx950: one 64-lane wavefront per row group,
 // HBM-bound streaming kernels with wave-level shuffles for the row reductions.
-//   norm_before_gate = 0:  y = (x*silu(z)) * rstd * w,   rstd = 1/sqrt(mean((x*silu z)^2) + eps)
-//   norm_before_gate = 1:  y = x * rstd * w * silu(z)
+//   norm_before_gate = 0:  y = xhat(x*silu(z)) * w + b
+//   norm_before_gate = 1:  y = (xhat(x) * w + b) * silu(z)
+//   xhat(v) = v * rstd,            rstd = 1/sqrt(mean(v^2) + eps)              (RMS statistics, p.ln = 0)
+//   xhat(v) = (v - mean) * rstd,   rstd = 1/sqrt(mean((v - mean)^2) + eps)     (LayerNorm, p.ln = 1)
+// b is optional (issm_triton/layernorm_gated.py:35-97 forward, :145-260 backward).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -23,13 +26,24 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd(NormP p) {
   const long row = item / p.ngroups;
   const int grp = item % p.ngroups;
   const int c0 = grp * p.gs;
-  float ss = 0.0f;
-  for (int c = lane; c < p.gs; c += 64) {
+  auto gated_x = [&](int c) {
     float v = ldv(p.x, row * p.xs + c0 + c, p.dt);
     if (p.z && !p.nbg) {
       const float z = ldv(p.z, row * p.zs + c0 + c, p.dt);
       v *= z * sigmoidf_(z);
     }
+    return v;
+  };
+  float mean = 0.0f;
+  if (p.ln) {
+    float sm = 0.0f;
+    for (int c = lane; c < p.gs; c += 64) sm += gated_x(c);
+    mean = wave_sum(sm) / (float)p.gs;
+    if (lane == 0) p.mean[(long)grp * p.rows + row] = mean;
+  }
+  float ss = 0.0f;
+  for (int c = lane; c < p.gs; c += 64) {
+    const float v = gated_x(c) - mean;
     ss += v * v;
   }
   ss = wave_sum(ss);
@@ -43,7 +57,8 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd(NormP p) {
       gate = z * sigmoidf_(z);
     }
     if (p.z && !p.nbg) v *= gate;
-    float y = v * rstd * ldv(p.w, c0 + c, p.wdt);
+    float y = (v - mean) * rstd * ldv(p.w, c0 + c, p.wdt);
+    if (p.b) y += ldv(p.b, c0 + c, p.wdt);
     if (p.z && p.nbg) y *= gate;
     stv(p.y, row * p.ys + c0 + c, p.dt, y);
   }
@@ -116,7 +131,8 @@ __device__ __forceinline__ f4 silu4(f4 z, f4& sg) {
   return g;
 }
 
-template <bool BF, int NV>
+// EXT: LayerNorm statistics and / or a bias (p.ln, p.b); the plain RMS form compiles without either.
+template <bool BF, int NV, bool EXT>
 __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -135,7 +151,8 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
     gate[v] = ld4<BF>(zp, row * zs + 4 * vi, ok, az);
   }
   ldw<NV>(p.w, lane, nvec, p.wdt, wv);
-  float ss = 0.0f;
+  f4 bv[EXT ? NV : 1];
+  if constexpr (EXT) ldw<NV>(p.b ? p.b : p.w, lane, nvec, p.wdt, bv);  // without a bias: loaded, not used
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     if (p.z) {
@@ -143,8 +160,20 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
       gate[v] = silu4(gate[v], sg);
       if (!p.nbg) x[v] *= gate[v];
     }
-    ss += (x[v].x * x[v].x + x[v].y * x[v].y) + (x[v].z * x[v].z + x[v].w * x[v].w);
   }
+  if (EXT && p.ln) {
+    float sm = 0.0f;  // absent vectors were loaded as zeros
+#pragma unroll
+    for (int v = 0; v < NV; ++v) sm += (x[v].x + x[v].y) + (x[v].z + x[v].w);
+    const float mean = wave_sum(sm) / (float)p.ncols;
+    if (lane == 0) p.mean[row] = mean;
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+      if (lane + 64 * v < nvec) x[v] -= mean;
+  }
+  float ss = 0.0f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) ss += (x[v].x * x[v].x + x[v].y * x[v].y) + (x[v].z * x[v].z + x[v].w * x[v].w);
   ss = wave_sum(ss);
   const float rstd = 1.0f / sqrtf(ss / (float)p.ncols + p.eps);
   if (lane == 0 && p.rstd) p.rstd[row] = rstd;
@@ -153,30 +182,37 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_fwd_fast(NormP p) {
     const int vi = lane + 64 * v;
     if (vi < nvec) {
       f4 y = x[v] * rstd * wv[v];
+      if constexpr (EXT) { if (p.b) y += bv[v]; }
       if (p.z && p.nbg) y *= gate[v];
       st4<BF>(p.y, row * p.ys + 4 * vi, y, ay);
     }
   }
 }
 
-template <bool BF, int NV>
+template <bool BF, int NV, bool EXT>
 __global__ __launch_bounds__(64) void k_rmsnorm_bwd_fast(NormP p) {
   const int lane = threadIdx.x;
   const int nvec = p.ncols >> 2;
   const int ax = al_of(p.x, p.xs, BF), az = al_of(p.z, p.zs, BF), ady = al_of(p.dy, p.dys, BF);
   const int adx = al_of(p.dx, p.dxs, BF), adz = al_of(p.dz, p.dzs, BF);
-  f4 w[NV], dwacc[NV];
+  f4 w[NV], dwacc[NV], bv[EXT ? NV : 1], dbacc[EXT ? NV : 1];
 #pragma unroll
   for (int v = 0; v < NV; ++v) dwacc[v] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
   ldw<NV>(p.w, lane, nvec, p.wdt, w);
+  if constexpr (EXT) {
+    ldw<NV>(p.b ? p.b : p.w, lane, nvec, p.wdt, bv);  // without a bias: loaded, not used
+#pragma unroll
+    for (int v = 0; v < NV; ++v) dbacc[v] = (f4){0.0f, 0.0f, 0.0f, 0.0f};
+  }
   // The loads of the next row are requested before the current row is worked on (x, dy, z and rstd back to back,
   // nothing between them), so that a row costs no memory round trip of its own.
   const void* zp = p.z ? p.z : p.x;  // without a gate the third load repeats the first and is not used
   const long zs = p.z ? p.zs : p.xs;
   f4 xn[NV], dyn[NV], zn[NV];
-  float rstd_n = 0.0f;
+  float rstd_n = 0.0f, mean_n = 0.0f;
   auto fetch = [&](long row) {
     rstd_n = p.rstd[row];
+    if (EXT && p.ln) mean_n = p.mean[row];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
       const int vi = lane + 64 * v;
@@ -188,37 +224,46 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd_fast(NormP p) {
   };
   if ((long)blockIdx.x < p.rows) fetch(blockIdx.x);
   for (long row = blockIdx.x; row < p.rows; row += p.nblocks) {
-    const float rstd = rstd_n;
+    const float rstd = rstd_n, mean = mean_n;  // mean stays 0 for RMS statistics
     f4 xo[NV], dyo[NV], z[NV], sg[NV], gate[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) { xo[v] = xn[v]; dyo[v] = dyn[v]; z[v] = zn[v]; }
     if (row + p.nblocks < p.rows) fetch(row + p.nblocks);
-    float c1 = 0.0f;
+    // absent vectors carry dy = 0, so they add nothing to either sum although their x - mean is not zero
+    float c1 = 0.0f, c2 = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
       gate[v] = (f4){1.0f, 1.0f, 1.0f, 1.0f};
       if (p.z) gate[v] = silu4(z[v], sg[v]);
-      const f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+      f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+      if (EXT) vv -= mean;
       const f4 d = (p.z && p.nbg) ? dyo[v] * gate[v] : dyo[v];
-      const f4 t = vv * rstd * d * w[v];
+      const f4 wd = d * w[v];
+      const f4 t = vv * rstd * wd;
       c1 += (t.x + t.y) + (t.z + t.w);
+      if (EXT) c2 += (wd.x + wd.y) + (wd.z + wd.w);
     }
     c1 = wave_sum(c1) / (float)p.ncols;
+    c2 = (EXT && p.ln) ? wave_sum(c2) / (float)p.ncols : 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
       const int vi = lane + 64 * v;
       if (vi < nvec) {
-        const f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+        f4 vv = (p.z && !p.nbg) ? xo[v] * gate[v] : xo[v];
+        if (EXT) vv -= mean;
         const f4 d = (p.z && p.nbg) ? dyo[v] * gate[v] : dyo[v];
         const f4 xhat = vv * rstd;
-        f4 dxv = (w[v] * d - xhat * c1) * rstd;
+        f4 dxv = (w[v] * d - (xhat * c1 + c2)) * rstd;
         dwacc[v] += d * xhat;
+        if constexpr (EXT) dbacc[v] += d;
         if (p.z) {
           f4 dzv;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float ds = sg[v][i] * (1.0f + z[v][i] * (1.0f - sg[v][i]));  // d silu / dz
-            dzv[i] = p.nbg ? dyo[v][i] * (xhat[i] * w[v][i]) * ds : dxv[i] * xo[v][i] * ds;
+            float pre = xhat[i] * w[v][i];
+            if constexpr (EXT) { if (p.b) pre += bv[v][i]; }
+            dzv[i] = p.nbg ? dyo[v][i] * pre * ds : dxv[i] * xo[v][i] * ds;
           }
           if (!p.nbg) dxv *= gate[v];
           if (p.dz) st4<BF>(p.dz, row * p.dzs + 4 * vi, dzv, adz);
@@ -230,7 +275,10 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd_fast(NormP p) {
 #pragma unroll
   for (int v = 0; v < NV; ++v) {
     const int vi = lane + 64 * v;
-    if (vi < nvec) *(f4*)(p.dw_partial + (long)blockIdx.x * p.ncols + 4 * vi) = dwacc[v];
+    if (vi < nvec) {
+      *(f4*)(p.dw_partial + (long)blockIdx.x * p.ncols + 4 * vi) = dwacc[v];
+      if constexpr (EXT) { if (p.b) *(f4*)(p.db_partial + (long)blockIdx.x * p.ncols + 4 * vi) = dbacc[v]; }
+    }
   }
 }
 
@@ -238,14 +286,16 @@ static bool norm_fast_ok(const NormP& p) { return p.ngroups == 1 && (p.ncols & 3
 
 // One wavefront per block; block b walks rows b, b+nblocks, ... and keeps its dw partial in LDS.
 __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
-  extern __shared__ float dws[];
+  extern __shared__ float dws[];  // dw partial (ncols), then the db partial (ncols) when there is a bias
+  float* dbs = dws + p.ncols;
   const int lane = threadIdx.x;
-  for (int c = lane; c < p.ncols; c += 64) dws[c] = 0.0f;
+  for (int c = lane; c < (p.b ? 2 : 1) * p.ncols; c += 64) dws[c] = 0.0f;
   for (long row = blockIdx.x; row < p.rows; row += p.nblocks) {
     for (int grp = 0; grp < p.ngroups; ++grp) {
       const int c0 = grp * p.gs;
       const float rstd = p.rstd[(long)grp * p.rows + row];
-      float c1 = 0.0f;
+      const float mean = p.ln ? p.mean[(long)grp * p.rows + row] : 0.0f;
+      float c1 = 0.0f, c2 = 0.0f;
       for (int c = lane; c < p.gs; c += 64) {
         float v = ldv(p.x, row * p.xs + c0 + c, p.dt);
         float d = ldv(p.dy, row * p.dys + c0 + c, p.dt);
@@ -254,9 +304,12 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
           const float gate = z * sigmoidf_(z);
           if (p.nbg) d *= gate; else v *= gate;
         }
-        c1 += v * rstd * d * ldv(p.w, c0 + c, p.wdt);
+        const float wd = d * ldv(p.w, c0 + c, p.wdt);
+        c1 += (v - mean) * rstd * wd;
+        c2 += wd;
       }
       c1 = wave_sum(c1) / (float)p.gs;
+      c2 = p.ln ? wave_sum(c2) / (float)p.gs : 0.0f;
       for (int c = lane; c < p.gs; c += 64) {
         const float xo = ldv(p.x, row * p.xs + c0 + c, p.dt);
         const float dyo = ldv(p.dy, row * p.dys + c0 + c, p.dt);
@@ -267,14 +320,16 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
           sg = sigmoidf_(z);
           gate = z * sg;
         }
-        const float v = (p.z && !p.nbg) ? xo * gate : xo;
+        const float v = ((p.z && !p.nbg) ? xo * gate : xo) - mean;
         const float d = (p.z && p.nbg) ? dyo * gate : dyo;
         const float xhat = v * rstd;
-        float dxv = (w * d - xhat * c1) * rstd;
+        float dxv = (w * d - (xhat * c1 + c2)) * rstd;
         dws[c0 + c] += d * xhat;
+        if (p.b) dbs[c0 + c] += d;
         if (p.z) {
           float dzv;
-          if (p.nbg) dzv = dyo * (xhat * w) * sg * (1.0f + z * (1.0f - sg));
+          const float pre = p.b ? xhat * w + ldv(p.b, c0 + c, p.wdt) : xhat * w;
+          if (p.nbg) dzv = dyo * pre * sg * (1.0f + z * (1.0f - sg));
           else {
             dzv = dxv * xo * sg * (1.0f + z * (1.0f - sg));
             dxv *= gate;
@@ -285,22 +340,26 @@ __global__ __launch_bounds__(64) void k_rmsnorm_bwd(NormP p) {
       }
     }
   }
-  for (int c = lane; c < p.ncols; c += 64) p.dw_partial[(long)blockIdx.x * p.ncols + c] = dws[c];
+  for (int c = lane; c < p.ncols; c += 64) {
+    p.dw_partial[(long)blockIdx.x * p.ncols + c] = dws[c];
+    if (p.b) p.db_partial[(long)blockIdx.x * p.ncols + c] = dbs[c];
+  }
 }
 
 // dw[c] = sum over the per-block partials, in a fixed order: block = 8 columns x 32 row groups, row group g adds
 // partials g, g+32, ... with two independent accumulators, then the 32 group sums are combined in order.
-__global__ __launch_bounds__(NTHREADS) void k_rmsnorm_dw(NormP p) {
+__global__ __launch_bounds__(NTHREADS) void k_rmsnorm_dw(NormP p, const float* __restrict__ partial,
+                                                         float* __restrict__ out) {
   __shared__ float red[NTHREADS];
   const int c = blockIdx.x * 8 + (threadIdx.x & 7), g = threadIdx.x >> 3;
   float a0 = 0.0f, a1 = 0.0f;
   if (c < p.ncols) {
     int b = g;
     for (; b + 32 < p.nblocks; b += 64) {
-      a0 += p.dw_partial[(long)b * p.ncols + c];
-      a1 += p.dw_partial[(long)(b + 32) * p.ncols + c];
+      a0 += partial[(long)b * p.ncols + c];
+      a1 += partial[(long)(b + 32) * p.ncols + c];
     }
-    if (b < p.nblocks) a0 += p.dw_partial[(long)b * p.ncols + c];
+    if (b < p.nblocks) a0 += partial[(long)b * p.ncols + c];
   }
   red[threadIdx.x] = a0 + a1;
   __syncthreads();
@@ -308,21 +367,26 @@ __global__ __launch_bounds__(NTHREADS) void k_rmsnorm_dw(NormP p) {
     float t = 0.0f;
 #pragma unroll
     for (int k = 0; k < 32; ++k) t += red[k * 8 + (threadIdx.x & 7)];
-    p.dw[c] = t;
+    out[c] = t;
   }
 }
 
-#define NORM_FAST(KERNEL, GRID, BLOCK)                                                            \
+#define NORM_FAST_NV(KERNEL, GRID, BLOCK, BF_, EXT_)                                              \
   do {                                                                                           \
     const int nv = (p.ncols / 4 + 63) / 64;                                                      \
+    if (nv <= 1) hipLaunchKernelGGL((KERNEL<BF_, 1, EXT_>), GRID, BLOCK, 0, st, p);              \
+    else if (nv == 2) hipLaunchKernelGGL((KERNEL<BF_, 2, EXT_>), GRID, BLOCK, 0, st, p);         \
+    else hipLaunchKernelGGL((KERNEL<BF_, 4, EXT_>), GRID, BLOCK, 0, st, p);                      \
+  } while (0)
+#define NORM_FAST(KERNEL, GRID, BLOCK)                                                            \
+  do {                                                                                           \
+    const bool ext = p.ln || p.b;                                                                \
     if (p.dt) {                                                                                  \
-      if (nv <= 1) hipLaunchKernelGGL((KERNEL<true, 1>), GRID, BLOCK, 0, st, p);                 \
-      else if (nv == 2) hipLaunchKernelGGL((KERNEL<true, 2>), GRID, BLOCK, 0, st, p);            \
-      else hipLaunchKernelGGL((KERNEL<true, 4>), GRID, BLOCK, 0, st, p);                         \
+      if (ext) NORM_FAST_NV(KERNEL, GRID, BLOCK, true, true);                                    \
+      else NORM_FAST_NV(KERNEL, GRID, BLOCK, true, false);                                       \
     } else {                                                                                     \
-      if (nv <= 1) hipLaunchKernelGGL((KERNEL<false, 1>), GRID, BLOCK, 0, st, p);                \
-      else if (nv == 2) hipLaunchKernelGGL((KERNEL<false, 2>), GRID, BLOCK, 0, st, p);           \
-      else hipLaunchKernelGGL((KERNEL<false, 4>), GRID, BLOCK, 0, st, p);                        \
+      if (ext) NORM_FAST_NV(KERNEL, GRID, BLOCK, false, true);                                   \
+      else NORM_FAST_NV(KERNEL, GRID, BLOCK, false, false);                                      \
     }                                                                                            \
   } while (0)
 
@@ -338,10 +402,11 @@ int launch_rmsnorm_fwd(const NormP& p, hipStream_t st) {
 
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st) {
   if (norm_fast_ok(p)) NORM_FAST(k_rmsnorm_bwd_fast, dim3(p.nblocks), dim3(64));
-  else hipLaunchKernelGGL(k_rmsnorm_bwd, dim3(p.nblocks), dim3(64), (size_t)p.ncols * sizeof(float), st, p);
+  else hipLaunchKernelGGL(k_rmsnorm_bwd, dim3(p.nblocks), dim3(64), (size_t)(p.b ? 2 : 1) * p.ncols * sizeof(float), st, p);
   int e = (int)hipGetLastError();
   if (e) return e;
-  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 7) / 8), dim3(NTHREADS), 0, st, p);
+  hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 7) / 8), dim3(NTHREADS), 0, st, p, p.dw_partial, p.dw);
+  if (p.b) hipLaunchKernelGGL(k_rmsnorm_dw, dim3((p.ncols + 7) / 8), dim3(NTHREADS), 0, st, p, p.db_partial, p.db);
   return (int)hipGetLastError();
 }
 

@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define ISSM_ABI_VERSION 2
+#define ISSM_ABI_VERSION 3
 #define ISSM_CHUNK 64 /* tokens per internal chunk */
 
 typedef enum issm_status {
@@ -232,6 +232,17 @@ typedef struct issm_norm_args {
   float* dw_partial;
   float* dw;
   void* stream;
+  /* LayerNorm statistics and bias (HAS_BIAS / IS_RMS_NORM = False of issm_triton/layernorm_gated.py:35-97, 145-260):
+   * layer_norm = 0 normalises with x * rstd, rstd = 1/sqrt(mean(x^2) + eps); layer_norm = 1 with (x - mean) * rstd,
+   * rstd = 1/sqrt(mean((x - mean)^2) + eps), and `mean` (ngroups*rows, fp32) is then required: written by the forward,
+   * read by the backward.  bias (ncols, weight_dtype), optional, is added after the weight and before the gate; the
+   * backward then needs db_partial (nblocks, ncols) fp32 scratch and writes db (ncols) fp32.  With a bias and more than
+   * one group per row or more than 1024 columns, ncols <= 8192. */
+  int32_t layer_norm;
+  const void* bias;
+  float* mean;
+  float* db_partial;
+  float* db;
 } issm_norm_args;
 
 int issm_rmsnorm_bwd_blocks(int64_t rows);
@@ -243,7 +254,9 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
  * results, bit for bit, as issm_gated_rmsnorm_bwd, except that args->dw_partial is ignored: the per-block partial
  * sums of dw go into a scratch array inside the library (ISSM_NORM_SCRATCH_FLOATS floats = 8 MiB per GPU the library
  * runs on, held until the process ends).  Problems with issm_rmsnorm_bwd_blocks(rows) * ncols >
- * ISSM_NORM_SCRATCH_FLOATS return ISSM_E_WORKSPACE (rows of up to 1024 columns always fit).  The function calls no
+ * ISSM_NORM_SCRATCH_FLOATS return ISSM_E_WORKSPACE (rows of up to 1024 columns always fit; with a bias db_partial is
+ * ignored as well, its partial sums follow those of dw in the array, and the bound holds for twice the product:
+ * up to 512 columns always fit).  The function calls no
  * hipMalloc / hipFree or other allocating routine.  All calls on one GPU share that GPU's array: two calls that
  * overlap in time on one GPU (different streams or host threads) race; calls on one stream are ordered and safe.
  * Nothing in the array has to be cleared between calls (every partial that is read was written by the same call). */

@@ -1,1 +1,1 @@
-from dest3d_amd.layernorm_gated import RMSNorm, rmsnorm_fn  # noqa: F401
+from dest3d_amd.layernorm_gated import LayerNorm, LayerNormFn, RMSNorm, layernorm_fn, rmsnorm_fn  # noqa: F401

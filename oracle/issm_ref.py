@@ -28,7 +28,7 @@ What each function restates (paths relative to the reference checkout):
                               calls), used to cross-check autograd and to debug kernels;
                               its per-chunk intermediates (S, states, M, dM, dH, dS,
                               g_next, y) are what the GPU stage tests compare with
-* ``gated_rmsnorm_ref``       issm_triton/layernorm_gated.py:8-29
+* ``gated_rmsnorm_ref``       issm_triton/layernorm_gated.py:8-29 (+ the LayerNorm form, :73-89)
 
 Pinning status: every function here is pinned by tests/test_oracle.py against an
 independent brute-force numpy loop on tiny shapes, against closed forms (A=0, dt=0,
@@ -298,11 +298,12 @@ def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias
 
 # ------------------------------------------------------------- gated RMSNorm
 def gated_rmsnorm_ref(x, weight, z=None, eps=1e-5, norm_before_gate=False, group_size=None,
-                      dtype=torch.float64):
-    """RMSNorm with optional SiLU gate (issm_triton/layernorm_gated.py:8-29).
+                      dtype=torch.float64, bias=None, layer_norm=False):
+    """RMSNorm with optional SiLU gate (issm_triton/layernorm_gated.py:8-29) and, with ``layer_norm``, the LayerNorm
+    form of the same kernels (IS_RMS_NORM = False, layernorm_gated.py:73-89: mean subtracted, variance about the mean).
 
-    norm_before_gate=False (what DEST uses, dest_module.py:512): y = rmsnorm(x*silu(z))*w.
-    norm_before_gate=True: y = rmsnorm(x)*w*silu(z).
+    norm_before_gate=False (what DEST uses, dest_module.py:512): y = norm(x*silu(z))*w + b.
+    norm_before_gate=True: y = (norm(x)*w + b)*silu(z).
     """
     x_ = x.to(dtype)
     w_ = weight.to(dtype)
@@ -312,8 +313,12 @@ def gated_rmsnorm_ref(x, weight, z=None, eps=1e-5, norm_before_gate=False, group
     d = x_.shape[-1]
     gs = d if group_size is None else group_size
     xg = x_.reshape(*x_.shape[:-1], d // gs, gs)
+    if layer_norm:
+        xg = xg - xg.mean(dim=-1, keepdim=True)
     rstd = torch.rsqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
     out = (xg * rstd).reshape(x_.shape) * w_
+    if bias is not None:
+        out = out + bias.to(dtype)
     if z_ is not None and norm_before_gate:
         out = out * torch.nn.functional.silu(z_)
     return out

@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported(lib):
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/issm.h but not exported"
     assert sorted(L.EXPORTS) == names
-    assert lib.issm_abi_version() == 2
+    assert lib.issm_abi_version() == 3
 
 
 def test_struct_layout_matches_header(lib):
@@ -92,6 +92,14 @@ def test_status_codes(lib):
     assert lib.issm_scan_fwd(C.byref(a)) == -6          # now only the workspace is missing
     na = L.NormArgs()
     assert lib.issm_gated_rmsnorm_fwd(C.byref(na)) == -2
+    # the fields appended for LayerNorm statistics and the bias are read where the header puts them
+    na.rows, na.ncols = 4, 8
+    na.x = na.w = na.rstd = na.y = fake
+    na.layer_norm = 1
+    assert lib.issm_gated_rmsnorm_fwd(C.byref(na)) == -1 and b"mean is NULL" in lib.issm_last_error()
+    na.layer_norm, na.bias = 0, fake
+    na.dy = na.dx = na.dw_partial = na.dw = fake
+    assert lib.issm_gated_rmsnorm_bwd(C.byref(na)) == -1 and b"db_partial" in lib.issm_last_error()
     assert lib.issm_rmsnorm_bwd_blocks(10) == 10 and lib.issm_rmsnorm_bwd_blocks(10 ** 6) == 2048
 
 

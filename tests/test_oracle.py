@@ -262,6 +262,31 @@ def test_gated_rmsnorm_closed_form_and_grad():
     assert torch.autograd.gradcheck(lambda a, b, c: R.gated_rmsnorm_ref(a, b, z=c), ins, eps=1e-6, atol=1e-7)
 
 
+def test_layernorm_form_against_the_library_routines():
+    """layer_norm=True / bias: torch's own layer_norm (one group) and group_norm (several groups per row) are the
+    library routines; the gate is the plain product on either side; shift invariance and the bias as closed forms."""
+    F = torch.nn.functional
+    x = torch.randn(6, 24, dtype=torch.float64)
+    z = torch.randn(6, 24, dtype=torch.float64)
+    w = torch.randn(24, dtype=torch.float64)
+    b = torch.randn(24, dtype=torch.float64)
+    y = R.gated_rmsnorm_ref(x, w, eps=1e-5, bias=b, layer_norm=True)
+    torch.testing.assert_close(y, F.layer_norm(x, (24,), w, b, eps=1e-5), rtol=1e-12, atol=1e-12)
+    yg = R.gated_rmsnorm_ref(x, w, eps=1e-5, bias=b, layer_norm=True, group_size=8)
+    torch.testing.assert_close(yg, F.group_norm(x, 3, w, b, eps=1e-5), rtol=1e-12, atol=1e-12)
+    # gate after the norm multiplies the biased output; gate before the norm replaces the input
+    y1 = R.gated_rmsnorm_ref(x, w, z=z, eps=1e-5, bias=b, layer_norm=True, norm_before_gate=True)
+    torch.testing.assert_close(y1, F.layer_norm(x, (24,), w, b, eps=1e-5) * F.silu(z), rtol=1e-12, atol=1e-12)
+    y0 = R.gated_rmsnorm_ref(x, w, z=z, eps=1e-5, bias=b, layer_norm=True, norm_before_gate=False)
+    torch.testing.assert_close(y0, F.layer_norm(x * F.silu(z), (24,), w, b, eps=1e-5), rtol=1e-12, atol=1e-12)
+    # a constant added to a row changes nothing with the mean subtracted, and does change the RMS form
+    torch.testing.assert_close(R.gated_rmsnorm_ref(x + 3.0, w, layer_norm=True), R.gated_rmsnorm_ref(x, w, layer_norm=True),
+                               rtol=1e-10, atol=1e-10)
+    assert (R.gated_rmsnorm_ref(x + 3.0, w) - R.gated_rmsnorm_ref(x, w)).abs().max() > 0.1
+    # the bias of the RMS form is a plain addition
+    torch.testing.assert_close(R.gated_rmsnorm_ref(x, w, bias=b), R.gated_rmsnorm_ref(x, w) + b, rtol=1e-13, atol=1e-13)
+
+
 def test_make_inputs_is_deterministic_and_in_range():
     a = R.make_inputs(1, 8, 2, 4, 8, seed=7)
     b = R.make_inputs(1, 8, 2, 4, 8, seed=7)

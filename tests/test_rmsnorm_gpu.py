@@ -44,6 +44,70 @@ def test_gated_rmsnorm_fwd_bwd(shape, gs, nbg, use_z, dtype):
         _check("dz", zg.grad, ins[2].grad, bt)
 
 
+@pytest.mark.parametrize("shape,gs,nbg,use_z,rms,use_b,dtype", [
+    ((8, 128, 288), None, False, True, False, True, torch.float32),    # LayerNorm module, gate before the norm
+    ((3, 77, 288), None, True, True, False, True, torch.float32),      # gate after the norm: dz sees the bias
+    ((5, 33, 288), 96, True, True, False, True, torch.float32),        # several groups per row (generic kernels)
+    ((5, 33, 288), 96, False, True, True, True, torch.float32),        # RMS statistics with a bias, groups
+    ((4, 50, 100), None, True, False, False, False, torch.float32),    # no gate, no bias, mean subtracted
+    ((2, 9, 1500), None, False, True, False, True, torch.float32),     # rows wider than the register-resident form
+    ((4, 64, 256), None, True, True, True, True, torch.float32),       # RMS statistics with a bias, one group
+    ((8, 256, 256), None, False, True, False, True, torch.bfloat16),
+    ((8, 64, 512), 128, True, True, False, True, torch.bfloat16),
+])
+def test_gated_layernorm_and_bias_fwd_bwd(shape, gs, nbg, use_z, rms, use_b, dtype):
+    """LayerNorm statistics and the bias of layernorm_gated.py:35-97 / 145-260 (layernorm_fn, rmsnorm_fn with a bias),
+    forward and all four gradients against the fp64 oracle."""
+    from dest3d_amd import layernorm_fn
+    _say(f"layernorm {shape} gs={gs} nbg={nbg} z={use_z} rms={rms} bias={use_b} {dtype}")
+    g = torch.Generator().manual_seed(shape[1] + 1)
+    x = (torch.randn(*shape, generator=g) + 0.7).to(dtype)      # a mean that is not zero
+    z = torch.randn(*shape, generator=g).to(dtype) if use_z else None
+    w = torch.randn(shape[-1], generator=g) * 0.5 + 1.0
+    b = torch.randn(shape[-1], generator=g) * 0.5 if use_b else None
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    leaf = lambda t: None if t is None else t.double().clone().requires_grad_()
+    xr, wr, br, zr = leaf(x), leaf(w), leaf(b), leaf(z)
+    yr = R.gated_rmsnorm_ref(xr, wr, z=zr, eps=1e-5, norm_before_gate=nbg, group_size=gs, bias=br, layer_norm=not rms)
+    (yr * dy.double()).sum().backward()
+    dev = lambda t: None if t is None else t.cuda().requires_grad_()
+    xg, wg, bg, zg = dev(x), dev(w), dev(b), dev(z)
+    y = layernorm_fn(xg, wg, bg, z=zg, eps=1e-5, group_size=gs, norm_before_gate=nbg, is_rms_norm=rms)
+    assert y.dtype == dtype and y.shape == x.shape
+    (y.float() * dy.cuda().float()).sum().backward()
+    torch.cuda.synchronize()
+    ft, bt = (FWD32, BWD32) if dtype == torch.float32 else (FWD16, BWD16)
+    _check("y", y, yr, ft)
+    _check("dx", xg.grad, xr.grad, bt)
+    _check("dw", wg.grad, wr.grad, bt)
+    if use_b:
+        _check("db", bg.grad, br.grad, bt)
+    if use_z:
+        _check("dz", zg.grad, zr.grad, bt)
+
+
+def test_layernorm_module_matches_torch_layer_norm():
+    """The LayerNorm module without a gate is torch's own layer_norm (the library routine), forward and backward."""
+    from issm_triton.layernorm_gated import LayerNorm
+    _say("LayerNorm module against torch.nn.functional.layer_norm")
+    torch.manual_seed(5)
+    m = LayerNorm(288, eps=1e-5, device="cuda")
+    with torch.no_grad():
+        m.weight.normal_(1.0, 0.3)
+        m.bias.normal_(0.0, 0.3)
+    x = (torch.randn(40, 17, 288, device="cuda") * 2 + 1).requires_grad_()
+    dy = torch.randn(40, 17, 288, device="cuda")
+    y = m(x)
+    (y * dy).sum().backward()
+    got = (y.detach(), x.grad.clone(), m.weight.grad.clone(), m.bias.grad.clone())
+    x.grad = None
+    m.zero_grad()
+    yr = torch.nn.functional.layer_norm(x.double(), (288,), m.weight.double(), m.bias.double(), eps=1e-5)
+    gx, gw, gb = torch.autograd.grad((yr * dy.double()).sum(), (x, m.weight, m.bias))
+    for name, a, b_, tol in zip(("y", "dx", "dw", "db"), got, (yr, gx, gw, gb), (FWD32, BWD32, BWD32, BWD32)):
+        _check(name, a, b_, tol)
+
+
 def test_rmsnorm_strided_rows_and_import_shim():
     from issm_triton.layernorm_gated import RMSNorm as Shim
     from issm_triton.issm_combined import ISSM_chunk_scan_combined  # noqa: F401
