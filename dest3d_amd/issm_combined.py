@@ -245,8 +245,47 @@ def ISSM_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias
     Return:
         out: (batch, seqlen, nheads, headdim)  [, final_states (batch, nheads, headdim, dstate) fp32]
     """
-    return ISSMChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
-                                         dt_softplus, dt_limit, return_final_states)
+    s = _head_split(x.shape[-1]) if x.dim() == 4 else 1
+    if s > 1:
+        x, dt, A, D, z, dt_bias, initial_states = _split_heads(s, x, dt, A, D, z, dt_bias, initial_states)
+    res = ISSMChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
+                                        dt_softplus, dt_limit, return_final_states)
+    if s == 1:
+        return res
+    if return_final_states:
+        return _merge_heads(s, res[0]), _merge_heads(s, res[1], state=True)
+    return _merge_heads(s, res)
+
+
+MAX_HEADDIM = 64   # what one workgroup's tiles are built for (ISSM_E_UNSUPPORTED above it)
+
+
+def _head_split(headdim: int) -> int:
+    """The scan is independent across the head dimension, so a head wider than the kernels' 64 runs as `s` heads of
+    headdim / s that share the head's dt, A and dt_bias (the reference has no such limit, issm_combined.py:58-83):
+    the smallest s that divides headdim with headdim / s <= 64."""
+    if headdim <= MAX_HEADDIM:
+        return 1
+    return next(s for s in range(2, headdim + 1) if headdim % s == 0 and headdim // s <= MAX_HEADDIM)
+
+
+def _split_heads(s, x, dt, A, D, z, dt_bias, h0):
+    """Views / repeats that turn (H, P) into (H s, P / s), head h -> heads h s .. h s + s - 1 (same group as h).
+    Plain differentiable tensor operations: autograd sums the gradients of the repeated dt, A, dt_bias, D."""
+    b, l, h, p = x.shape
+    q = p // s
+    rep = lambda t, dim: None if t is None else t.repeat_interleave(s, dim=dim)
+    heads = lambda t: None if t is None else t.reshape(b, l, h * s, q)
+    if D is not None:
+        D = D.reshape(h * s, q) if D.dim() == 2 else D.repeat_interleave(s, dim=0)
+    h0 = None if h0 is None else h0.reshape(b, h * s, q, h0.shape[-1])
+    return heads(x), rep(dt, 2), rep(A, 0), D, heads(z), rep(dt_bias, 0), h0
+
+
+def _merge_heads(s, t, state=False):
+    if state:   # (B, H s, P / s, N) -> (B, H, P, N)
+        return t.reshape(t.shape[0], t.shape[1] // s, t.shape[2] * s, t.shape[3])
+    return t.reshape(t.shape[0], t.shape[1], t.shape[2] // s, t.shape[3] * s)
 
 
 class ISSMBiScanFn(torch.autograd.Function):
@@ -282,5 +321,13 @@ class ISSMBiScanFn(torch.autograd.Function):
 def ISSM_biscan_combined(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, chunk_size, D=None, dt_bias=None,
                          initial_states=None, dt_softplus=False, dt_limit=(0.0, INF)):
     """Returns (y_f, y_b, last_f, last_b), all in natural time order; see ISSMBiScanFn."""
-    return ISSMBiScanFn.apply(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, chunk_size, D, dt_bias, initial_states,
-                              dt_softplus, dt_limit)
+    s = _head_split(x_f.shape[-1]) if x_f.dim() == 4 else 1
+    if s > 1:
+        x_b = x_b.reshape(x_b.shape[0], x_b.shape[1], x_b.shape[2] * s, x_b.shape[3] // s)
+        x_f, dt, A, D, _, dt_bias, initial_states = _split_heads(s, x_f, dt, A, D, None, dt_bias, initial_states)
+    res = ISSMBiScanFn.apply(x_f, x_b, dt, A, B_f, B_b, C_f, C_b, chunk_size, D, dt_bias, initial_states,
+                             dt_softplus, dt_limit)
+    if s == 1:
+        return res
+    return (_merge_heads(s, res[0]), _merge_heads(s, res[1]), _merge_heads(s, res[2], state=True),
+            _merge_heads(s, res[3], state=True))

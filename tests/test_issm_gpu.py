@@ -135,6 +135,33 @@ def test_operator_fp32_matches_oracle(case):
         _check("d" + k, g[k], g_ref[k], BWD32)
 
 
+@pytest.mark.parametrize("P", [128, 96, 67])
+def test_head_dimension_above_the_tile_limit(P):
+    """Heads wider than the kernels' 64 run as several narrower heads that share dt, A, dt_bias and the group's B, C
+    (128 -> 2 x 64, 96 -> 2 x 48, the prime 67 -> 67 x 1); every gradient, the repeated parameters' included."""
+    _say(f"operator fp32 headdim {P}")
+    d = _problem(1, 100, 2, P, 48, 1, seed=P, D="hp", z=True)
+    y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+    y, fin, g, _ = _run_operator(d, torch.float32)
+    _check("out", y, y_ref, FWD32)
+    _check("final_states", fin, fin_ref, FWD32)
+    for k in GRAD_NAMES:
+        _check("d" + k, g[k], g_ref[k], BWD32)
+    if P == 128:
+        from dest3d_amd import ISSM_biscan_combined, ISSM_chunk_scan_combined
+        cu = lambda t: t.cuda()
+        x2 = torch.randn(1, 100, 2, P, generator=torch.Generator().manual_seed(1))
+        args = (cu(d["dt"]), cu(d["A"]), cu(d["B"]), cu(d["B"]), cu(d["C"]), cu(d["C"]))
+        yf, yb, lf, lb = ISSM_biscan_combined(cu(d["x"]), cu(x2), *args, 64, D=cu(d["D"]), dt_bias=cu(d["dt_bias"]),
+                                              dt_softplus=True, dt_limit=d["dt_limit"])
+        flip = lambda t: t.flip(1)
+        yb1, lb1 = ISSM_chunk_scan_combined(flip(cu(x2)), flip(args[0]), args[1], flip(args[2]), flip(args[4]), 64,
+                                            D=cu(d["D"]), dt_bias=cu(d["dt_bias"]), dt_softplus=True,
+                                            dt_limit=d["dt_limit"], return_final_states=True)
+        assert yb.shape == (1, 100, 2, P) and lb.shape == (1, 2, P, 48)
+        assert torch.equal(yb, flip(yb1)) and torch.equal(lb, lb1)
+
+
 def test_operator_bf16_matches_oracle():
     _say("operator bf16")
     d = _problem(2, 192, 4, 32, 128, 1, seed=5)
