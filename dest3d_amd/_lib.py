@@ -64,6 +64,7 @@ class ScanArgs(C.Structure):
         ("dA", C.c_void_p), ("dD", C.c_void_p), ("ddt_bias", C.c_void_p), ("dh0", C.c_void_p),
         ("bwd_workspace", C.c_void_p), ("bwd_workspace_bytes", C.c_size_t),
         ("stream", C.c_void_p),
+        ("seq_idx", C.c_void_p), ("seq_idx_stride", C.c_int64 * 2),
     ]
 
 

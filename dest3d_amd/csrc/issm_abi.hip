@@ -143,7 +143,13 @@ static int check_common(const issm_scan_args* a) {
   if (rc) return rc;
   if ((unsigned)a->io_dtype > 1u || (unsigned)a->dt_dtype > 1u || (unsigned)a->h0_dtype > 1u)
     return fail(ISSM_E_DTYPE, "unknown dtype code (io=%d dt=%d h0=%d)", a->io_dtype, a->dt_dtype, a->h0_dtype);
-  if (a->flags & ISSM_FLAG_SEQ_IDX) return fail(ISSM_E_UNSUPPORTED, "seq_idx is not supported");
+  if (a->flags & ISSM_FLAG_SEQ_IDX) {
+    if (!a->seq_idx) return fail(ISSM_E_NULL, "ISSM_FLAG_SEQ_IDX is set and seq_idx is NULL");
+    if (a->dims.ndir != 1) return fail(ISSM_E_UNSUPPORTED, "seq_idx with ndir = %d (one direction only)", a->dims.ndir);
+    if (a->seq_idx_stride[0] < 0 || a->seq_idx_stride[1] < 0 ||
+        a->seq_idx_stride[1] * (int64_t)a->dims.seqlen >= ((int64_t)1 << 31))
+      return fail(ISSM_E_STRIDE, "seq_idx strides (%lld, %lld)", (long long)a->seq_idx_stride[0], (long long)a->seq_idx_stride[1]);
+  }
   if (!(a->dt_min >= 0.0f)) return fail(ISSM_E_UNSUPPORTED, "dt_limit[0] = %g < 0 is not supported", a->dt_min);
   if (!(a->dt_max >= a->dt_min)) return fail(ISSM_E_SHAPE, "dt_limit is empty (%g, %g)", a->dt_min, a->dt_max);
   if (!a->A) return fail(ISSM_E_NULL, "A is NULL");
@@ -211,6 +217,9 @@ static KP make_kp(const issm_scan_args* a) {
   }
   p.dt = td(a->dt); p.ddt = td(a->ddt); p.h0 = td(a->h0);
   p.A = a->A; p.D = a->D; p.dt_bias = a->dt_bias;
+  if (a->flags & ISSM_FLAG_SEQ_IDX) {
+    p.seq_idx = a->seq_idx; p.seq_s0 = a->seq_idx_stride[0]; p.seq_s1 = a->seq_idx_stride[1];
+  }
   return p;
 }
 

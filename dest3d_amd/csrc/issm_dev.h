@@ -54,9 +54,13 @@ struct KP {
   const float* dt_bias;
   float* final_states[2];
   const float* dfinal[2];
+  const int* seq_idx;   // (B, L) sequence ids of packed rows, or null
+  long seq_s0, seq_s1;
 };
 
 enum : unsigned { F_SOFTPLUS = 1u, F_D_HDIM = 2u, F_NOCLAMP = 4u };
+// What the running sum of dt' A log2(e) takes where the sequence id changes: decays across the change become 2^-128.
+constexpr float SEQ_CUT = 128.0f;
 
 // Parameter block of the gated RMSNorm kernels.
 struct NormP {
@@ -471,6 +475,7 @@ __device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
 struct RowMap {
   int base, step, nvalid;
   bool full;
+  unsigned long long cut;  // bit r: the sequence id changes between rows r - 1 and r of the chunk (scan order); uniform
 };
 template <bool FULL>
 __device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4, int n0) {
@@ -481,6 +486,18 @@ __device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4
   r.nvalid = min(CS, p.L - u.c * CS);
   // FULL kernels are only launched when every chunk and every column slice is complete
   r.full = FULL;
+  r.cut = 0;
+  if (!FULL && p.seq_idx) {  // packed sequences take the kernels' general variants
+    // lane = row of the chunk in scan order; its predecessor in scan order may be the previous chunk's last row
+    const int row = u.c * CS + (int)(threadIdx.x & 63);
+    bool changes = false;
+    if (row > 0 && row < p.L) {
+      const long t = u.dir ? p.L - 1 - row : row, tp = u.dir ? t + 1 : t - 1;
+      const int* q = p.seq_idx + (long)u.b * p.seq_s0;
+      changes = q[t * p.seq_s1] != q[tp * p.seq_s1];
+    }
+    r.cut = __ballot(changes);
+  }
   return r;
 }
 // Lane's 16 values of column n of a (B,L,G|H,N)-shaped tensor.
@@ -631,15 +648,29 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
   // step is issued for all four before any result is used (a cross-lane fetch goes through the LDS pipe: taken tile
   // by tile, twelve latencies would line up instead of three).  Same operations in the same order as tile by tile.
   float c[4], v[4], t[4];
+  if (rm.full || rm.cut == 0) {  // uniform (and the only form the complete-tile variants contain)
 #pragma unroll
-  for (int J = 0; J < 4; ++J) {
-    float a = 0.0f;
+    for (int J = 0; J < 4; ++J) {
+      float a = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      a += dtp[4 * J + j] * A2;
-      cs[4 * J + j] = a;
+      for (int j = 0; j < 4; ++j) {
+        a += dtp[4 * J + j] * A2;
+        cs[4 * J + j] = a;
+      }
+      c[J] = a;
     }
-    c[J] = a;
+  } else {  // packed sequences: the sum drops by SEQ_CUT at every row where the sequence id changes
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      const unsigned bits = (unsigned)(rm.cut >> (16 * J + 4 * g4)) & 15u;
+      float a = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a += dtp[4 * J + j] * A2 - (((bits >> j) & 1u) ? SEQ_CUT : 0.0f);
+        cs[4 * J + j] = a;
+      }
+      c[J] = a;
+    }
   }
 #pragma unroll
   for (int J = 0; J < 4; ++J) t[J] = __shfl_up(c[J], 16, 64);
@@ -847,7 +878,7 @@ __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   do {                                                                                               \
     const int pt_ = ((p).P + 15) / 16;                                                               \
     const bool iob_ = (p).io_dt != 0, dtb_ = (p).dt_dt != 0;                                         \
-    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0);                                       \
+    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0) && !(p).seq_idx;                      \
     if (pt_ <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }        \
     else if (pt_ == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }   \
     else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }                 \

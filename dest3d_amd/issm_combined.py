@@ -46,8 +46,6 @@ class _Problem:
     """Validated, kernel-ready view of one call (1 or 2 directions)."""
 
     def __init__(self, xs, dt, A, Bs, Cs, chunk_size, D, zs, dt_bias, h0, seq_idx, dt_softplus, dt_limit):
-        if seq_idx is not None:
-            raise NotImplementedError("seq_idx (packed variable-length batches) is not supported; DEST never passes it")
         x0 = xs[0]
         L.require_gpu(x0, "x")
         if x0.dim() != 4:
@@ -74,6 +72,12 @@ class _Problem:
             assert dt_bias.shape == (h, n)
         if h0 is not None:
             assert h0.shape == (b, h, p, n)
+        self.seq_idx = None
+        if seq_idx is not None:
+            assert seq_idx.shape == (b, l)                      # issm_combined.py:70-71
+            if len(xs) != 1:
+                raise NotImplementedError("seq_idx with the fused bidirectional scan")
+            self.seq_idx = seq_idx.detach().to(torch.int32).contiguous()
         if not (isinstance(chunk_size, int) and chunk_size > 0):
             raise ValueError(f"chunk_size must be a positive int, got {chunk_size!r}")
         self.ndir = len(xs)
@@ -107,6 +111,10 @@ class _Problem:
         a.h0_dtype = L.dtype_code(self.h0.dtype) if self.h0 is not None else L.ISSM_F32
         a.flags = (L.FLAG_DT_SOFTPLUS if self.dt_softplus else 0) | \
                   (L.FLAG_D_HAS_HDIM if (self.D is not None and self.D.dim() == 2) else 0)
+        if self.seq_idx is not None:
+            a.flags |= L.FLAG_SEQ_IDX
+            a.seq_idx = self.seq_idx.data_ptr()
+            a.seq_idx_stride[0], a.seq_idx_stride[1] = self.seq_idx.stride(0), self.seq_idx.stride(1)
         a.dt_min = self.dt_limit[0]
         a.dt_max = min(self.dt_limit[1], 3.0e38)
         for i in range(self.ndir):
@@ -240,7 +248,7 @@ def ISSM_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias
         z: (batch, seqlen, nheads, headdim)
         dt_bias: (nheads, dstate)
         initial_states: (batch, nheads, headdim, dstate)
-        seq_idx: must be None
+        seq_idx: (batch, seqlen) integer ids of the sequences packed into a row, or None
         dt_softplus: whether to apply softplus to dt (+ dt_bias)
     Return:
         out: (batch, seqlen, nheads, headdim)  [, final_states (batch, nheads, headdim, dstate) fp32]

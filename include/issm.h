@@ -59,7 +59,7 @@ typedef enum issm_status {
   ISSM_E_SHAPE = -2,       /* a dimension is non-positive / inconsistent (issm_combined.py:58-83) */
   ISSM_E_STRIDE = -3,      /* a stride is unusable */
   ISSM_E_DTYPE = -4,       /* unknown dtype code */
-  ISSM_E_UNSUPPORTED = -5, /* legal in the reference but not built (seq_idx, dt_min < 0) */
+  ISSM_E_UNSUPPORTED = -5, /* legal in the reference but not built (dt_min < 0, headdim > 64) */
   ISSM_E_WORKSPACE = -6,   /* workspace missing or too small */
   ISSM_E_LAUNCH = -7       /* hipGetLastError() != hipSuccess after a launch */
 } issm_status;
@@ -69,7 +69,7 @@ typedef enum issm_dtype { ISSM_F32 = 0, ISSM_BF16 = 1 } issm_dtype;
 enum {
   ISSM_FLAG_DT_SOFTPLUS = 1u << 0, /* apply softplus to dt + dt_bias (softplus.py:7-16) */
   ISSM_FLAG_D_HAS_HDIM = 1u << 1,  /* D is (H,P) instead of (H) */
-  ISSM_FLAG_SEQ_IDX = 1u << 2      /* caller had a seq_idx: rejected with ISSM_E_UNSUPPORTED */
+  ISSM_FLAG_SEQ_IDX = 1u << 2      /* args->seq_idx is given (packed sequences, issm_combined.py:29) */
 };
 
 typedef struct issm_dims {
@@ -125,6 +125,13 @@ typedef struct issm_scan_args {
   void* bwd_workspace;
   size_t bwd_workspace_bytes;
   void* stream; /* hipStream_t */
+  /* seq_idx (issm_triton/issm_combined.py:29, ndir = 1 only): (batch, seqlen) int32, read when ISSM_FLAG_SEQ_IDX is
+   * set.  Tokens of a batch row whose values differ belong to different sequences packed into that row, and no
+   * state passes from one to the next: wherever seq_idx changes from a token to its successor the running sum of
+   * dt'.A takes an extra -128 ln 2, i.e. every decay across the change is multiplied by 2^-128 (3e-39: zero at fp32
+   * resolution, where the reference's kernels multiply by an exact 0).  The backward must be given the same array. */
+  const int32_t* seq_idx;
+  int64_t seq_idx_stride[2]; /* element strides of (batch, seqlen) */
 } issm_scan_args;
 
 /* Version of this header the library was built against. */

@@ -77,12 +77,17 @@ def _expand_groups(t: torch.Tensor, nheads: int) -> torch.Tensor:
 # ------------------------------------------------------------ ground truth scan
 def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
                          initial_states=None, dt_softplus=False, dt_limit=(0.0, INF),
-                         dtype=torch.float64) -> Tuple[torch.Tensor, torch.Tensor]:
+                         dtype=torch.float64, seq_idx=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Token-by-token recurrence, differentiable, evaluated in ``dtype``.
 
         a_t   = dt'_t * A                         (B,H,N)
         h_t   = exp(a_t) * h_{t-1} + dt'_t * B_t * x_t     (B,H,P,N)
         y_t   = sum_n C_t * h_t + D * x_t ;  out_t = y_t * silu(z_t) if z given
+
+    seq_idx (B,L), optional: ids of the sequences packed into a row (issm_combined.py:29).  Where the id changes
+    from one token to the next no state is carried over -- what the reference's kernels obtain by zeroing every
+    decay between tokens of different ids (issm_chunk_state.py, issm_state_passing.py, issm_chunk_scan.py and
+    issm_cabt_bmm.py:14 under HAS_SEQ_IDX).
 
     Returns (out (B,L,H,P), final_states (B,H,P,N)).
     """
@@ -102,6 +107,8 @@ def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
     dts, Bs, Cs, xs = dtp.unbind(1), Bh.unbind(1), Ch.unbind(1), x_.unbind(1)
     for t in range(L):
         decay = torch.exp(dts[t] * A_[None])                          # (B,H,N)
+        if seq_idx is not None and t > 0:
+            decay = decay * (seq_idx[:, t] == seq_idx[:, t - 1]).to(dtype)[:, None, None]
         inject = (dts[t] * Bs[t])[:, :, None, :] * xs[t][..., None]
         h = decay[:, :, None, :] * h + inject
         ys.append(torch.einsum("bhpn,bhn->bhp", h, Cs[t]))

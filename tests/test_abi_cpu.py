@@ -90,6 +90,16 @@ def test_status_codes(lib):
     assert lib.issm_scan_fwd(C.byref(a)) == -3 and b"32-bit" in lib.issm_last_error()
     a.dt.stride[1] = 3 * 64
     assert lib.issm_scan_fwd(C.byref(a)) == -6          # now only the workspace is missing
+    # seq_idx: the flag without the array, and the array (the struct's last fields) with two directions
+    a.flags |= L.FLAG_SEQ_IDX
+    assert lib.issm_scan_fwd(C.byref(a)) == -1 and b"seq_idx is NULL" in lib.issm_last_error()
+    a.seq_idx = fake
+    a.seq_idx_stride[0], a.seq_idx_stride[1] = 64, 1
+    assert lib.issm_scan_fwd(C.byref(a)) == -6
+    a.dims.ndir = 2
+    assert lib.issm_scan_fwd(C.byref(a)) == -5 and b"one direction" in lib.issm_last_error()
+    a.dims.ndir = 1
+    a.flags &= ~L.FLAG_SEQ_IDX
     na = L.NormArgs()
     assert lib.issm_gated_rmsnorm_fwd(C.byref(na)) == -2
     # the fields appended for LayerNorm statistics and the bias are read where the header puts them

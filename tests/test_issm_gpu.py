@@ -162,6 +162,73 @@ def test_head_dimension_above_the_tile_limit(P):
         assert torch.equal(yb, flip(yb1)) and torch.equal(lb, lb1)
 
 
+def _seq_ids(Bsz, L, cuts):
+    """(Bsz, L) ids that go up by one at the given token positions (row b uses cuts[b])."""
+    s = torch.zeros(Bsz, L, dtype=torch.int32)
+    for b in range(Bsz):
+        for c in cuts[b]:
+            s[b, c:] += 1
+    return s
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_packed_sequences_match_oracle(dtype):
+    """seq_idx (issm_combined.py:29): several sequences packed into a batch row; no state crosses a change of id.
+    Changes inside a chunk, at a chunk's first row, at its last row, in adjacent rows and in the ragged last chunk;
+    row 1 of the batch has no change at all.  Every gradient against the oracle's recurrence with resets."""
+    _say(f"operator with seq_idx {dtype}")
+    L_ = 64 * 3 + 21
+    d = _problem(2, L_, 2, 32, 96, 1, seed=77, D="h", z=True)
+    if dtype == torch.bfloat16:
+        for k in ("x", "dt", "B", "C", "z"):
+            d[k] = d[k].bfloat16().float()
+    seq = _seq_ids(2, L_, [[5, 40, 41, 64, 127, 130, 200], []])
+    ins = {k: d[k].double().clone().requires_grad_() for k in GRAD_NAMES if d[k] is not None}
+    y_ref, fin_ref = R.issm_scan_sequential(ins["x"], ins["dt"], ins["A"], ins["B"], ins["C"], D=ins["D"], z=ins["z"],
+                                            dt_bias=ins["dt_bias"], initial_states=ins["h0"],
+                                            dt_softplus=d["softplus"], dt_limit=d["dt_limit"], seq_idx=seq)
+    ((y_ref * d["dy"].double()).sum() + (fin_ref * d["dfinal"].double()).sum()).backward()
+    from dest3d_amd import ISSM_chunk_scan_combined
+    cast = lambda t, dt_=dtype: None if t is None else t.to("cuda", dt_).requires_grad_()
+    g = dict(x=cast(d["x"]), dt=cast(d["dt"]), A=cast(d["A"], torch.float32), B=cast(d["B"]), C=cast(d["C"]),
+             D=cast(d["D"], torch.float32), z=cast(d["z"]), dt_bias=cast(d["dt_bias"], torch.float32),
+             h0=cast(d["h0"], torch.float32))
+    y, fin = ISSM_chunk_scan_combined(g["x"], g["dt"], g["A"], g["B"], g["C"], 64, D=g["D"], z=g["z"],
+                                      dt_bias=g["dt_bias"], initial_states=g["h0"], seq_idx=seq.cuda().long(),
+                                      dt_softplus=d["softplus"], dt_limit=d["dt_limit"], return_final_states=True)
+    ((y.float() * d["dy"].cuda()).sum() + (fin * d["dfinal"].cuda()).sum()).backward()
+    torch.cuda.synchronize()
+    ft, bt = (FWD32, BWD32) if dtype == torch.float32 else (FWD16, BWD16)
+    _check("out", y, y_ref.detach(), ft)
+    _check("final_states", fin, fin_ref.detach(), ft)
+    for k in GRAD_NAMES:
+        if d[k] is not None:
+            _check("d" + k, g[k].grad, ins[k].grad, bt)
+
+
+def test_packed_sequences_equal_separate_calls():
+    """Two sequences packed into one row give what two calls give, the second without an initial state; a constant
+    seq_idx changes nothing, bit for bit."""
+    from dest3d_amd import ISSM_chunk_scan_combined
+    _say("seq_idx: packed = separate")
+    d = _problem(1, 150, 2, 32, 64, 1, seed=9, softplus=False)
+    t = {k: d[k].cuda() for k in ("x", "dt", "A", "B", "C")}
+    cut = 70
+    seq = _seq_ids(1, 150, [[cut]]).cuda()
+    y, fin = ISSM_chunk_scan_combined(t["x"], t["dt"], t["A"], t["B"], t["C"], 64, seq_idx=seq, return_final_states=True)
+    part = lambda sl: ISSM_chunk_scan_combined(t["x"][:, sl], t["dt"][:, sl], t["A"], t["B"][:, sl], t["C"][:, sl], 64,
+                                               return_final_states=True)
+    y0, _ = part(slice(0, cut))
+    y1, fin1 = part(slice(cut, 150))
+    _check("first sequence", y[:, :cut], y0, FWD32)
+    _check("second sequence", y[:, cut:], y1, FWD32)
+    _check("final state", fin, fin1, FWD32)
+    ya, fa = ISSM_chunk_scan_combined(t["x"], t["dt"], t["A"], t["B"], t["C"], 64, seq_idx=torch.zeros_like(seq),
+                                      return_final_states=True)
+    yb, fb = ISSM_chunk_scan_combined(t["x"], t["dt"], t["A"], t["B"], t["C"], 64, return_final_states=True)
+    assert torch.equal(ya, yb) and torch.equal(fa, fb)
+
+
 def test_operator_bf16_matches_oracle():
     _say("operator bf16")
     d = _problem(2, 192, 4, 32, 128, 1, seed=5)
@@ -325,7 +392,7 @@ def test_error_codes_do_not_abort():
     assert lib.issm_fwd_workspace_bytes(C.byref(a), C.byref(n)) == -5 and b"headdim" in lib.issm_last_error()
     a.dims.headdim = 32
     a.flags |= L.FLAG_SEQ_IDX
-    assert lib.issm_scan_fwd(C.byref(a)) == -5
+    assert lib.issm_scan_fwd(C.byref(a)) == -1 and b"seq_idx is NULL" in lib.issm_last_error()
     a.flags &= ~L.FLAG_SEQ_IDX
     a.dt_min = -1.0
     assert lib.issm_scan_fwd(C.byref(a)) == -5
@@ -335,8 +402,6 @@ def test_error_codes_do_not_abort():
     assert lib.issm_scan_fwd(C.byref(a)) == -4
     from dest3d_amd import ISSM_chunk_scan_combined
     t = {k: d[k].cuda() for k in ("x", "dt", "A", "B", "C")}
-    with pytest.raises(NotImplementedError):
-        ISSM_chunk_scan_combined(t["x"], t["dt"], t["A"], t["B"], t["C"], 64, seq_idx=torch.zeros(1, 64).cuda())
     with pytest.raises(RuntimeError, match="dt_limit"):
         ISSM_chunk_scan_combined(t["x"], t["dt"], t["A"], t["B"], t["C"], 64, dt_limit=(-1.0, 1.0))
     with pytest.raises(RuntimeError, match="no CPU path"):

@@ -287,6 +287,35 @@ def test_layernorm_form_against_the_library_routines():
     torch.testing.assert_close(R.gated_rmsnorm_ref(x, w, bias=b), R.gated_rmsnorm_ref(x, w) + b, rtol=1e-13, atol=1e-13)
 
 
+def test_packed_sequences_are_independent_runs():
+    """seq_idx: a row that packs three sequences gives, segment by segment, what three separate runs give (the later
+    ones without an initial state) -- outputs, final state and gradients; ids need not start at zero."""
+    torch.manual_seed(3)
+    Bsz, L, H, P, N = 1, 11, 2, 3, 4
+    x = torch.randn(Bsz, L, H, P, dtype=torch.float64, requires_grad=True)
+    dt = (torch.rand(Bsz, L, H, N, dtype=torch.float64) * 0.5).requires_grad_()
+    A = -torch.rand(H, N, dtype=torch.float64) * 3
+    Bm = torch.randn(Bsz, L, 1, N, dtype=torch.float64)
+    Cm = torch.randn(Bsz, L, 1, N, dtype=torch.float64)
+    h0 = torch.randn(Bsz, H, P, N, dtype=torch.float64)
+    seq = torch.tensor([[4, 4, 4, 7, 7, 7, 7, 7, 9, 9, 9]])
+    y, fin = R.issm_scan_sequential(x, dt, A, Bm, Cm, initial_states=h0, seq_idx=seq)
+    w = torch.randn_like(y)
+    gx, gdt = torch.autograd.grad((y * w).sum() + fin.sum(), (x, dt))
+    ys, gxs, gdts = [], [], []
+    for lo, hi in ((0, 3), (3, 8), (8, 11)):
+        xs = x.detach()[:, lo:hi].clone().requires_grad_()
+        dts = dt.detach()[:, lo:hi].clone().requires_grad_()
+        yi, fi = R.issm_scan_sequential(xs, dts, A, Bm[:, lo:hi], Cm[:, lo:hi], initial_states=h0 if lo == 0 else None)
+        loss = (yi * w[:, lo:hi]).sum() + (fi.sum() if hi == L else 0.0)
+        a, b = torch.autograd.grad(loss, (xs, dts))
+        ys.append(yi.detach()); gxs.append(a); gdts.append(b)
+    torch.testing.assert_close(y.detach(), torch.cat(ys, 1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(fin.detach(), fi.detach(), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(gx, torch.cat(gxs, 1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(gdt, torch.cat(gdts, 1), rtol=1e-12, atol=1e-12)
+
+
 def test_make_inputs_is_deterministic_and_in_range():
     a = R.make_inputs(1, 8, 2, 4, 8, seed=7)
     b = R.make_inputs(1, 8, 2, 4, 8, seed=7)
