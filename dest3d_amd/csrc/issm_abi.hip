@@ -220,6 +220,8 @@ static KP make_kp(const issm_scan_args* a) {
   if (a->flags & ISSM_FLAG_SEQ_IDX) {
     p.seq_idx = a->seq_idx; p.seq_s0 = a->seq_idx_stride[0]; p.seq_s1 = a->seq_idx_stride[1];
   }
+  p.c_lo = 0; p.ncl = p.nc;
+  if (p.N % 64 == 0 && !p.seq_idx) p.full_tiles = p.L % ISSM_CHUNK == 0 ? 1 : (p.nc > 1 ? 2 : 0);
   return p;
 }
 

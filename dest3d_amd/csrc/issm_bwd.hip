@@ -63,8 +63,7 @@ struct BwdStSmem {
 // comes straight from the registers of the column-lane layout; each wave walks its own 16
 // columns of every 64-column slice without any barrier after the dy / x tiles are staged.
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __restrict__ dy_ws,
-                                                          float* __restrict__ dstates, float* __restrict__ dm) {
+__device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __restrict__ dy_ws, float* __restrict__ dstates, float* __restrict__ dm) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdStSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -174,6 +173,18 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __r
       }
   }
 }
+template <int PT, bool IOB, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS) void k_bwd_dstates(KP p, const float* __restrict__ dy_ws, float* __restrict__ dstates, float* __restrict__ dm) {
+  k_bwd_dstates_body<PT, IOB, DTB, FULL>(p, dy_ws, dstates, dm);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool IOB, bool DTB>
+__global__ __launch_bounds__(NTHREADS) void k_bwd_dstates_mixed(KP p, const float* __restrict__ dy_ws, float* __restrict__ dstates, float* __restrict__ dm) {
+  if (decode_unit(p, xcd_remap(blockIdx.x, gridDim.x)).c == p.nc - 1) k_bwd_dstates_body<PT, IOB, DTB, false>(p, dy_ws, dstates, dm);
+  else k_bwd_dstates_body<PT, IOB, DTB, true>(p, dy_ws, dstates, dm);
+}
+
 
 // ------------------------------------------------------- reverse state passing
 // Block = (bt, h, 64 state columns); thread (pg = tid >> 4, nq = tid & 15) carries rows
@@ -626,12 +637,7 @@ __device__ __forceinline__ void bwd_small_levels(const float (&cs)[16], const fl
 
 // partA, partBias: (Bt*nc, H, N) per-unit partial sums of dA and ddt_bias
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws,
-                                                           const float* __restrict__ states,
-                                                           const float* __restrict__ dstates,
-                                                           const float* __restrict__ dm,
-                                                           const float* __restrict__ g_last,
-                                                           float* __restrict__ partA, float* __restrict__ partBias) {
+__device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -646,8 +652,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
   id /= nsl;
   u.g = id % p.G;
   id /= p.G;
-  u.c = id % p.nc;
-  u.b = id / p.nc;
+  u.c = p.c_lo + id % p.ncl;
+  u.b = id / p.ncl;
   u.dir = p.dir0;
   u.bt = u.b * p.ndir + u.dir;
   u.h = u.g * p.hpg;
@@ -884,6 +890,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __
     if (p.dC[u.dir].ptr) lane_store_ln<IOB>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
   }
 }
+template <int PT, bool IOB, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+  k_bwd_chunk_body<PT, IOB, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool IOB, bool DTB>
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_mixed(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_body<PT, IOB, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+  else k_bwd_chunk_body<PT, IOB, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+}
+
 
 // ------------------------------------------------- chunk backward, bf16 inputs
 // The same computation for bf16 x / B / C / dy: every matrix product runs on v_mfma_f32_16x16x32_bf16 with operands
@@ -1051,12 +1069,7 @@ __device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const
 }
 
 template <int PT, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws,
-                                                              const float* __restrict__ states,
-                                                              const float* __restrict__ dstates,
-                                                              const float* __restrict__ dm,
-                                                              const float* __restrict__ g_last,
-                                                              float* __restrict__ partA, float* __restrict__ partBias) {
+__device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkBfSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -1071,8 +1084,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float*
   id /= nsl;
   u.g = id % p.G;
   id /= p.G;
-  u.c = id % p.nc;
-  u.b = id / p.nc;
+  u.c = p.c_lo + id % p.ncl;
+  u.b = id / p.ncl;
   u.dir = p.dir0;
   u.bt = u.b * p.ndir + u.dir;
   u.h = u.g * p.hpg;
@@ -1270,6 +1283,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float*
     if (p.dC[u.dir].ptr) lane_store_ln<true>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
   }
 }
+template <int PT, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+  k_bwd_chunk_bf_body<PT, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool DTB>
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf_mixed(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_bf_body<PT, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+  else k_bwd_chunk_bf_body<PT, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+}
+
 
 // ------------------------------------------------------------------------- dx
 // BF (bf16 inputs): the operands of the product over the state index are bf16 tiles read as matrix fragments of 8
@@ -1301,9 +1326,7 @@ __device__ __forceinline__ bf8 frag8(const uint16_t* tile, int row, int g4, int 
 
 // partD: (Bt*nc*H, P) per-unit sums over rows of dy*x
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(KP p, const float* __restrict__ dy_ws,
-                                                     const float* __restrict__ dstates,
-                                                     const float* __restrict__ cabt, float* __restrict__ partD) {
+__device__ __forceinline__ void k_bwd_dx_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ dstates, const float* __restrict__ cabt, float* __restrict__ partD) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdDxSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -1444,6 +1467,18 @@ __global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(
     }
   }
 }
+template <int PT, bool IOB, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL) ? 4 : 1) void k_bwd_dx(KP p, const float* __restrict__ dy_ws, const float* __restrict__ dstates, const float* __restrict__ cabt, float* __restrict__ partD) {
+  k_bwd_dx_body<PT, IOB, DTB, FULL>(p, dy_ws, dstates, cabt, partD);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool IOB, bool DTB>
+__global__ __launch_bounds__(NTHREADS, (PT <= 2 && false) ? 4 : 1) void k_bwd_dx_mixed(KP p, const float* __restrict__ dy_ws, const float* __restrict__ dstates, const float* __restrict__ cabt, float* __restrict__ partD) {
+  if (decode_unit(p, xcd_remap(blockIdx.x, gridDim.x)).c == p.nc - 1) k_bwd_dx_body<PT, IOB, DTB, false>(p, dy_ws, dstates, cabt, partD);
+  else k_bwd_dx_body<PT, IOB, DTB, true>(p, dy_ws, dstates, cabt, partD);
+}
+
 
 // ------------------------------------------------------------------- reductions
 // All final reductions run as ONE launch (they are independent of each other and tiny, so separate
@@ -1535,8 +1570,9 @@ int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* d
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
     const size_t sm = sizeof(BwdStSmem<PT_, IOB_>);
-    if (int e = set_lds(k_bwd_dstates<PT_, IOB_, DTB_, FULL_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_dstates<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
+    constexpr auto kern = MIXED_ ? &k_bwd_dstates_mixed<PT_, IOB_, DTB_> : &k_bwd_dstates<PT_, IOB_, DTB_, FULL_>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, dm);
   });
   return (int)hipGetLastError();
 }
@@ -1571,19 +1607,19 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
   return (int)hipGetLastError();
 }
 
-template <int PT, bool IOB, bool DTB, bool FULL>
+template <int PT, bool IOB, bool DTB, bool FULL, bool MIXED>
 static int launch_bwd_chunk_t(const KP& p, int blocks, const float* dy_ws, const float* states, const float* dstates,
                               const float* dm, const float* g_last, float* partA, float* partBias, hipStream_t st) {
   if constexpr (IOB) {  // bf16 inputs: every product on the bf16 matrix instructions
     const size_t sm = sizeof(BwdChunkBfSmem<PT>);
-    if (int e = set_lds(k_bwd_chunk_bf<PT, DTB, FULL>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_chunk_bf<PT, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm,
-                       g_last, partA, partBias);
+    constexpr auto kern = MIXED ? &k_bwd_chunk_bf_mixed<PT, DTB> : &k_bwd_chunk_bf<PT, DTB, FULL>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
   } else {
     const size_t sm = sizeof(BwdChunkSmem<PT>);
-    if (int e = set_lds(k_bwd_chunk<PT, false, DTB, FULL>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_chunk<PT, false, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates,
-                       dm, g_last, partA, partBias);
+    constexpr auto kern = MIXED ? &k_bwd_chunk_mixed<PT, false, DTB> : &k_bwd_chunk<PT, false, DTB, FULL>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
   }
   return 0;
 }
@@ -1592,7 +1628,8 @@ int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const
                      const float* g_last, float* partA, float* partBias, hipStream_t st) {
   const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
   ISSM_DISPATCH(p, {
-    if (int e = launch_bwd_chunk_t<PT_, IOB_, DTB_, FULL_>(p, blocks, dy_ws, states, dstates, dm, g_last, partA, partBias, st))
+    if (int e = launch_bwd_chunk_t<PT_, IOB_, DTB_, FULL_, MIXED_>(p, blocks, dy_ws, states, dstates, dm, g_last, partA,
+                                                                  partBias, st))
       return e;
   });
   return (int)hipGetLastError();
@@ -1603,8 +1640,9 @@ int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const f
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
     const size_t sm = sizeof(BwdDxSmem<PT_, IOB_>);
-    if (int e = set_lds(k_bwd_dx<PT_, IOB_, DTB_, FULL_>, sm)) return e;
-    hipLaunchKernelGGL((k_bwd_dx<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
+    constexpr auto kern = MIXED_ ? &k_bwd_dx_mixed<PT_, IOB_, DTB_> : &k_bwd_dx<PT_, IOB_, DTB_, FULL_>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, dy_ws, dstates, cabt, partD);
   });
   return (int)hipGetLastError();
 }

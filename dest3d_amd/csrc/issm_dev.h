@@ -56,6 +56,13 @@ struct KP {
   const float* dfinal[2];
   const int* seq_idx;   // (B, L) sequence ids of packed rows, or null
   long seq_s0, seq_s1;
+  // Chunks [c_lo, c_lo + ncl) are the ones a launch of a per-chunk kernel covers (all nc of them).  full_tiles picks
+  // the kernel variants: 1 = every chunk has 64 rows and every column slice 64 columns (complete-tile code, no
+  // masks); 2 = that holds for all chunks but the last in scan order (the sequence length is not a multiple of 64):
+  // one launch whose workgroups take the complete-tile code except those of the last chunk, which take the general
+  // code -- the general code alone runs 1.5 - 2x longer; 0 = general code everywhere (ragged column slices, packed
+  // sequences, a single chunk).
+  int c_lo, ncl, full_tiles;
 };
 
 enum : unsigned { F_SOFTPLUS = 1u, F_D_HDIM = 2u, F_NOCLAMP = 4u };
@@ -431,13 +438,13 @@ __device__ __forceinline__ Unit decode_unit(const KP& p, int u) {
   if (p.ndir == 2) {
     r.dir = u & 1;
     u >>= 1;
-    const int j = u % p.nc;
-    r.b = u / p.nc;
-    r.c = r.dir ? p.nc - 1 - j : j;
+    const int j = u % p.ncl;
+    r.b = u / p.ncl;
+    r.c = p.c_lo + (r.dir ? p.ncl - 1 - j : j);
     r.bt = r.b * 2 + r.dir;
   } else {
-    r.c = u % p.nc;
-    r.bt = u / p.nc;
+    r.c = p.c_lo + u % p.ncl;
+    r.bt = u / p.ncl;
     r.dir = r.bt % p.ndir;
     r.b = r.bt / p.ndir;
   }
@@ -859,11 +866,12 @@ __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   return (((long)bt * p.nc + c) * p.H + h) * CS * CS;
 }
 
-// Kernel dispatch on (P tiles, io dtype, dt dtype, complete tiles): the statement sees PT_, IOB_, DTB_, FULL_
+// Kernel dispatch on (P tiles, io dtype, dt dtype, complete / mixed tiles): the statement sees PT_, IOB_, DTB_, FULL_, MIXED_
 // as constants.
-#define ISSM_DISPATCH_FULL(full, ...)                                  \
-  if (full) { constexpr bool FULL_ = true; __VA_ARGS__ }               \
-  else { constexpr bool FULL_ = false; __VA_ARGS__ }
+#define ISSM_DISPATCH_FULL(full, ...)                                                                       \
+  if ((full) == 1) { constexpr bool FULL_ = true; constexpr bool MIXED_ = false; (void)MIXED_; __VA_ARGS__ }        \
+  else if ((full) == 2) { constexpr bool FULL_ = false; constexpr bool MIXED_ = true; (void)FULL_; __VA_ARGS__ }    \
+  else { constexpr bool FULL_ = false; constexpr bool MIXED_ = false; (void)MIXED_; __VA_ARGS__ }
 #define ISSM_DISPATCH_DT(iob, dtb, full, ...)                          \
   if (iob) {                                                           \
     constexpr bool IOB_ = true;                                        \
@@ -878,7 +886,7 @@ __device__ __forceinline__ long sq_off(const KP& p, int bt, int c, int h) {
   do {                                                                                               \
     const int pt_ = ((p).P + 15) / 16;                                                               \
     const bool iob_ = (p).io_dt != 0, dtb_ = (p).dt_dt != 0;                                         \
-    const bool full_ = ((p).L % CS == 0) && ((p).N % NS == 0) && !(p).seq_idx;                      \
+    const int full_ = (p).full_tiles;                                                                \
     if (pt_ <= 2) { constexpr int PT_ = 2; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }        \
     else if (pt_ == 3) { constexpr int PT_ = 3; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }   \
     else { constexpr int PT_ = 4; ISSM_DISPATCH_DT(iob_, dtb_, full_, __VA_ARGS__) }                 \

@@ -72,8 +72,7 @@ __device__ __forceinline__ bf8 op_frag(const uint16_t* tile, int row, int g4, in
 }
 
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __restrict__ states,
-                                                          float* __restrict__ cs_last, float* __restrict__ cabt) {
+__device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restrict__ states, float* __restrict__ cs_last, float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr bool SPLIT = !IOB;
   typedef FwdLocalSmem<PT, SPLIT> SM;
@@ -277,6 +276,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __rest
     }
   }
 }
+template <int PT, bool IOB, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local(KP p, float* __restrict__ states, float* __restrict__ cs_last, float* __restrict__ cabt) {
+  k_chunk_local_body<PT, IOB, DTB, FULL>(p, states, cs_last, cabt);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool IOB, bool DTB>
+__global__ __launch_bounds__(NTHREADS, 2) void k_chunk_local_mixed(KP p, float* __restrict__ states, float* __restrict__ cs_last, float* __restrict__ cabt) {
+  if (decode_unit(p, xcd_remap(blockIdx.x, gridDim.x)).c == p.nc - 1) k_chunk_local_body<PT, IOB, DTB, false>(p, states, cs_last, cabt);
+  else k_chunk_local_body<PT, IOB, DTB, true>(p, states, cs_last, cabt);
+}
+
 
 // ---------------------------------------------------------------- state passing
 // One thread carries 4 adjacent state columns of one (bt, h, p) through all chunks.
@@ -427,8 +438,7 @@ __device__ __forceinline__ void col_store_bf(const float (&v)[16], uint16_t* dst
 }
 
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states,
-                                                         const float* __restrict__ cabt, float* __restrict__ out_x) {
+__device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __restrict__ states, const float* __restrict__ cabt, float* __restrict__ out_x) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef FwdScanSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -558,6 +568,18 @@ __global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __re
     gstore<IOB, 4>(const_cast<void*>(to.ptr), (long)u.b * to.s0 + (long)u.h * to.s2, off, v);
   }
 }
+template <int PT, bool IOB, bool DTB, bool FULL>
+__global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states, const float* __restrict__ cabt, float* __restrict__ out_x) {
+  k_chunk_scan_body<PT, IOB, DTB, FULL>(p, states, cabt, out_x);
+}
+// One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
+// for the last one (uniform per workgroup).
+template <int PT, bool IOB, bool DTB>
+__global__ __launch_bounds__(NTHREADS) void k_chunk_scan_mixed(KP p, const float* __restrict__ states, const float* __restrict__ cabt, float* __restrict__ out_x) {
+  if (decode_unit(p, xcd_remap(blockIdx.x, gridDim.x)).c == p.nc - 1) k_chunk_scan_body<PT, IOB, DTB, false>(p, states, cabt, out_x);
+  else k_chunk_scan_body<PT, IOB, DTB, true>(p, states, cabt, out_x);
+}
+
 
 // ------------------------------------------------------------------- launchers
 template <typename K>
@@ -569,8 +591,9 @@ int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, 
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
     const size_t sm = sizeof(FwdLocalSmem<PT_, !IOB_>);
-    if (int e = set_lds(k_chunk_local<PT_, IOB_, DTB_, FULL_>, sm)) return e;
-    hipLaunchKernelGGL((k_chunk_local<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
+    constexpr auto kern = MIXED_ ? &k_chunk_local_mixed<PT_, IOB_, DTB_> : &k_chunk_local<PT_, IOB_, DTB_, FULL_>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);
   });
   return (int)hipGetLastError();
 }
@@ -593,8 +616,9 @@ int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float
   const int units = p.B * p.ndir * p.nc * p.H;
   ISSM_DISPATCH(p, {
     const size_t sm = sizeof(FwdScanSmem<PT_, IOB_>);
-    if (int e = set_lds(k_chunk_scan<PT_, IOB_, DTB_, FULL_>, sm)) return e;
-    hipLaunchKernelGGL((k_chunk_scan<PT_, IOB_, DTB_, FULL_>), dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
+    constexpr auto kern = MIXED_ ? &k_chunk_scan_mixed<PT_, IOB_, DTB_> : &k_chunk_scan<PT_, IOB_, DTB_, FULL_>;
+    if (int e = set_lds(kern, sm)) return e;
+    hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, states, cabt, out_x);
   });
   return (int)hipGetLastError();
 }
