@@ -296,12 +296,20 @@ def _stage_args(d, ndir=1):
     return L, prob, prob.args()
 
 
-def test_stage_entry_points_match_oracle_intermediates():
+@pytest.mark.parametrize("shape", [
+    (2, 150, 4, 32, 96, 2),
+    # head dimensions that leave threads of the state-passing kernels without a row of their own (stand-ins that only
+    # load): 20 of 32 rows and 40 of 64 with 32-column slices, 36 of 48 with 64-column slices and many workgroups
+    (1, 150, 2, 20, 64, 1), (1, 150, 2, 40, 96, 1), (4, 130, 8, 36, 512, 1),
+], ids=lambda s: "B%dL%dH%dP%dN%dG%d" % s)
+def test_stage_entry_points_match_oracle_intermediates(shape):
     """chunk_local -> state_passing -> chunk_scan and the backward stages, each against the
     explicit sums of the oracle (oracle.issm_bwd_closed_form(intermediates=True))."""
-    _say("stage entry points")
-    Bsz, L_, H, P, N, G = 2, 150, 4, 32, 96, 2
-    d = _problem(Bsz, L_, H, P, N, G, seed=21, D="h")
+    _say(f"stage entry points {shape}")
+    Bsz, L_, H, P, N, G = shape
+    # (the seed is one for which no dt lands within fp32 rounding of a clamp limit: there the mask of the fp32 kernels
+    # and of the fp64 oracle differ for that one element, and with it the element's whole ddt)
+    d = _problem(Bsz, L_, H, P, N, G, seed=23, D="h")
     ref = R.issm_bwd_closed_form(d["x"], d["dt"], d["A"], d["B"], d["C"], 64, d["dy"], dfinal=d["dfinal"], D=d["D"],
                                  dt_bias=d["dt_bias"], initial_states=d["h0"], dt_softplus=True,
                                  dt_limit=d["dt_limit"], intermediates=True)
