@@ -530,15 +530,24 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
 #pragma unroll
     for (int k = 0; k < 16; ++k) out[k] = BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k];
   } else {
-    bool ok[16];
+    // The same 32-bit addressing with the row clamped to the chunk's last existing row and the column to 0: every
+    // lane reads an address inside the tensor, and what it read is replaced by zero where the row or column is absent
+    // (64-bit per-element offsets and a mask array held across the loads cost the general variants some forty
+    // registers per call site).
+    (void)ss;
+    const int rmax = rm.nvalid - 1 - 4 * g4;  // last existing row, relative to the lane's row 0 (may be negative)
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + (vn ? n : 0)) * (unsigned)sizeof(T);
+    unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
+    asm volatile("" : "+s"(ks));
+    const char* qb = (const char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      ok[k] = vn && lane_row(k, g4) < rm.nvalid;
-      const long o = ok[k] ? (long)rm.base * t.s1 + n + (16 * (k >> 2) + (k & 3)) * ss : 0;
-      r[k] = q[o];
+      const int rk = 16 * (k >> 2) + (k & 3);
+      r[k] = *(const T*)(qb + (lo + (unsigned)min(rk, rmax) * ks));  // a negative row wraps like the base does
     }
 #pragma unroll
-    for (int k = 0; k < 16; ++k) out[k] = ok[k] ? (BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k]) : 0.0f;
+    for (int k = 0; k < 16; ++k)
+      out[k] = (vn && 16 * (k >> 2) + (k & 3) <= rmax) ? (BF ? bf16_to_f((uint16_t)r[k]) : (float)r[k]) : 0.0f;
   }
 }
 // Store of the lane's 16 values to column n of a (B,L,G|H,N)-shaped tensor (absent rows / columns skipped).
@@ -559,10 +568,17 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
       if (BF) *d = (T)f_to_bf16(v[k]); else *d = (T)v[k];
     }
   } else {
+    (void)ss;
+    const int rmax = rm.nvalid - 1 - 4 * g4;
+    const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
+    unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
+    asm volatile("" : "+s"(ks));
+    char* qb = (char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      if (vn && lane_row(k, g4) < rm.nvalid) {
-        T* d = q + ((long)rm.base * t.s1 + n + (16 * (k >> 2) + (k & 3)) * ss);
+      const int rk = 16 * (k >> 2) + (k & 3);
+      if (vn && rk <= rmax) {
+        T* d = (T*)(qb + (lo + (unsigned)rk * ks));
         if (BF) *d = (T)f_to_bf16(v[k]); else *d = (T)v[k];
       }
     }
@@ -580,16 +596,18 @@ __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int 
 #pragma unroll
     for (int q = 0; q < CNT; ++q) out[q] = *(const float*)(sb + (lo + (unsigned)(16 * (q >> 2) + (q & 3)) * nb));
   } else {
+    // rows clamped to the last one of the head, the column to 0; absent values replaced by zero afterwards
     float r[CNT];
-    bool ok[CNT];
+    const int pmax = P - 1 - 4 * g4;
+    const unsigned lo = (unsigned)(4 * g4 * N + (vn ? n : 0)) * 4u;
+    unsigned nb = (unsigned)N * 4u;
+    asm volatile("" : "+s"(nb));
+    const char* sb = (const char*)src;
 #pragma unroll
-    for (int q = 0; q < CNT; ++q) {
-      const int pp = 16 * (q >> 2) + 4 * g4 + (q & 3);
-      ok[q] = vn && pp < P;
-      r[q] = src[ok[q] ? (long)pp * N + n : 0];
-    }
+    for (int q = 0; q < CNT; ++q)
+      r[q] = *(const float*)(sb + (lo + (unsigned)min(16 * (q >> 2) + (q & 3), pmax) * nb));
 #pragma unroll
-    for (int q = 0; q < CNT; ++q) out[q] = ok[q] ? r[q] : 0.0f;
+    for (int q = 0; q < CNT; ++q) out[q] = (vn && 16 * (q >> 2) + (q & 3) <= pmax) ? r[q] : 0.0f;
   }
 }
 // dt transform (bias -> softplus -> clamp) of the lane's rows and the inclusive running sum of
