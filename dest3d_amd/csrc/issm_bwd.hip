@@ -116,20 +116,24 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
         for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
       }
       if (IOB) {
-        // bf16 inputs: the block goes out as two bf16 copies in the same 16 KB, dM[l][s] at [l][s] of the first half
-        // and at [s][l] of the second, which is what k_bwd_chunk_bf's matrix operands read (blocks above the diagonal
-        // are not written and never read)
+        // bf16 inputs: the block goes out as one symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] (8 KB at the
+        // start of the unit's 16 KB): the F sums of k_bwd_chunk_bf contract over the columns of dM and the G sums over
+        // its rows, and with T both are rows of one tile, contiguous for a lane's 8 k-slots.
         uint16_t* mb = reinterpret_cast<uint16_t*>(m);
         const int sc = j * 16 + cm, l0 = wave * 16 + 4 * g4;
-        float v[4];
+        const unsigned w0 = pack_bf16(acc[0], acc[1]), w1 = pack_bf16(acc[2], acc[3]);
+        const uint16_t h[4] = {(uint16_t)w0, (uint16_t)(w0 >> 16), (uint16_t)w1, (uint16_t)(w1 >> 16)};
+        if (j < wave) {  // a block below the diagonal blocks: whole, and whole again mirrored
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = sc <= l0 + r ? acc[r] : 0.0f;
-        const unsigned w0 = pack_bf16(v[0], v[1]), w1 = pack_bf16(v[2], v[3]);
-        mb[(l0 + 0) * CS + sc] = (uint16_t)w0;
-        mb[(l0 + 1) * CS + sc] = (uint16_t)(w0 >> 16);
-        mb[(l0 + 2) * CS + sc] = (uint16_t)w1;
-        mb[(l0 + 3) * CS + sc] = (uint16_t)(w1 >> 16);
-        *(uint2*)(mb + CS * CS + sc * CS + l0) = make_uint2(w0, w1);
+          for (int r = 0; r < 4; ++r) mb[(l0 + r) * CS + sc] = h[r];
+          *(uint2*)(mb + sc * CS + l0) = make_uint2(w0, w1);
+        } else {  // a diagonal block: the lane's entries on or below the diagonal, each mirrored
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (sc <= l0 + r) mb[(l0 + r) * CS + sc] = h[r];
+            if (sc < l0 + r) mb[sc * CS + l0 + r] = h[r];
+          }
+        }
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -906,16 +910,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_mixed(KP p, const flo
 // ------------------------------------------------- chunk backward, bf16 inputs
 // The same computation for bf16 x / B / C / dy: every matrix product runs on v_mfma_f32_16x16x32_bf16 with operands
 // rounded once to bf16 (the reference casts its dot operands to the input dtype as well, issm_cabt_bmm.py:42-43;
-// running sums, decays, states and all accumulation stay fp32).  x and dy are bf16 already, so their tiles are exact;
-// dM arrives from k_bwd_dstates as two bf16 copies, row-major and transposed, because the F sums contract over the
-// columns of dM and the G sums over its rows, and a lane's operand must be contiguous in LDS.
+// running sums, decays, states and all accumulation stay fp32).  x and dy are bf16 already, so their tiles are exact
+// copies; dM arrives from k_bwd_dstates as the symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)]: the F sums
+// contract over the columns of dM and the G sums over its rows, and in T both are rows, contiguous for a lane's k-slots.
+// Up to three head tiles the workgroup holds two sets of tiles and uses them in turn: the next head's are requested
+// once the products over the head dimension are done (their registers are free then), land in the other set while
+// the levels run, and one barrier per head is all the exchange needs.  With four head tiles two sets would not leave
+// room for two workgroups per CU: one set, requested and waited for at the top of each head.
 template <int PT>
 struct BwdChunkBfSmem {
   static constexpr int KW = 16 * PT, LDP = KW + 8;  // x / dy tiles [l][p]
-  static constexpr int LDM = CS + 8;                // dM tiles [row][col]
-  uint16_t xs[CS * LDP], dys[CS * LDP];
-  uint16_t dmr[CS * LDM];  // dM[l][s]
-  uint16_t dmt[CS * LDM];  // dM[s][l] stored at [l][s]: the transpose
+  static constexpr int LDM = CS + 8;                // dM tile [row][col]
+  static constexpr int SETS = PT <= 3 ? 2 : 1;
+  uint16_t xs[SETS][CS * LDP], dys[SETS][CS * LDP];
+  uint16_t dm[SETS][CS * LDM];  // T[i][j] = dM[max(i,j)][min(i,j)]
   float dbc[32 * NTHREADS];
 };
 
@@ -1102,10 +1110,45 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
 #pragma unroll
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
+  // The reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
+  // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first.
+  auto head_of = [&](int hh) { return u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh); };
+  constexpr bool TWO_SETS = SM::SETS == 2;
+  // a head's tiles on their way from global memory to LDS: raw bf16 pairs (x, dy) and the thread's two 16-byte pieces
+  // of T (rows tq >> 3 and 32 + (tq >> 3), columns 8 (tq & 7) .. + 7)
+  uint2 nx[PT], ny[PT];
+  uint4 nm0, nm1;
+  // (the thread index is made opaque at each use: the per-lane addresses derived from it are then formed next to the
+  // accesses instead of being kept, as 64-bit values, across the whole head loop)
+  auto request = [&](int h) {
+    int tq = tid;
+    asm volatile("" : "+v"(tq));
+    const int mrow = tq >> 3, mcol = (tq & 7) * 8;
+    Unit v = u;
+    v.h = h;
+    dy_load_bf<PT, FULL>(p, v, dy_ws, ny, tq);
+    lp_load_bf<PT, FULL>(p, v, p.x[u.dir], nx, tq);
+    const uint16_t* dmb = reinterpret_cast<const uint16_t*>(dm + sq_off(p, u.bt, u.c, h));
+    nm0 = *(const uint4*)(dmb + mrow * CS + mcol);
+    nm1 = *(const uint4*)(dmb + (32 + mrow) * CS + mcol);
+  };
+  auto deposit = [&](int set) {
+    int tq = tid;
+    asm volatile("" : "+v"(tq));
+    const int mrow = tq >> 3, mcol = (tq & 7) * 8;
+    lp_store_raw<PT, LDP>(ny, s.dys[set], tq);
+    lp_store_raw<PT, LDP>(nx, s.xs[set], tq);
+    *(uint4*)(s.dm[set] + mrow * LDM + mcol) = nm0;
+    *(uint4*)(s.dm[set] + (32 + mrow) * LDM + mcol) = nm1;
+  };
+  request(head_of(0));
+  deposit(0);
+  __syncthreads();
+
   for (int hh = 0; hh < p.hpg; ++hh) {
-    // the reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
-    // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first
-    u.h = u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh);
+    const int set = TWO_SETS ? (hh & 1) : 0;
+    const bool more = hh + 1 < p.hpg;  // uniform
+    u.h = head_of(hh);
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
@@ -1113,28 +1156,15 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     const float gl = (g4 == 3 && vn) ? g_last[vec_off(p, u.bt, u.c, u.h) + n] : 0.0f;
     lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
     lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
-    {
-      float xv[CS * PT * 16 / NTHREADS], dv[CS * PT * 16 / NTHREADS];
-      int tq = tid;
-      asm volatile("" : "+v"(tq));
-      dy_load<true, PT, FULL>(p, u, dy_ws, dv, tq);
-      lp_load<true, PT, FULL>(p, u, p.x[u.dir], xv, tq);
-      // both bf16 copies of dM: 2 x (64 x 64) halves, 16 bytes per access
-      const uint16_t* dmb = reinterpret_cast<const uint16_t*>(dm + sq_off(p, u.bt, u.c, u.h));
-      // (thread tq: row tq >> 3 and row 32 + (tq >> 3), columns 8 (tq & 7) .. + 7 of either copy)
-      const int mrow = tq >> 3, mcol = (tq & 7) * 8;
-      const uint4 mr0 = *(const uint4*)(dmb + mrow * CS + mcol), mr1 = *(const uint4*)(dmb + (32 + mrow) * CS + mcol);
-      const uint4 mt0 = *(const uint4*)(dmb + CS * CS + mrow * CS + mcol);
-      const uint4 mt1 = *(const uint4*)(dmb + CS * CS + (32 + mrow) * CS + mcol);
-      __syncthreads();  // the previous head no longer reads the LDS tiles
-      lp_store_bf<PT, LDP>(dv, s.dys, tq);
-      lp_store_bf<PT, LDP>(xv, s.xs, tq);
-      *(uint4*)(s.dmr + mrow * LDM + mcol) = mr0;
-      *(uint4*)(s.dmr + (32 + mrow) * LDM + mcol) = mr1;
-      *(uint4*)(s.dmt + mrow * LDM + mcol) = mt0;
-      *(uint4*)(s.dmt + (32 + mrow) * LDM + mcol) = mt1;
+    if (!TWO_SETS && hh > 0) {  // one set of tiles: this head's replace the previous head's
+      request(u.h);
+      __syncthreads();  // the previous head no longer reads the tiles
+      deposit(0);
+      __syncthreads();
     }
-    __syncthreads();
+    const uint16_t* xs_ = s.xs[set];
+    const uint16_t* dys_ = s.dys[set];
+    const uint16_t* dm_ = s.dm[set];
 
     const float An = cf.A;
     float dtp[16], cs[16], dfac[16];
@@ -1167,8 +1197,8 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
           const bool half = (PT & 1) && t == KT - 1;
-          const bf8 xf = half ? split_frag<LDP, true>(s.xs, I * 16 + cq, gq, t) : split_frag<LDP>(s.xs, I * 16 + cq, gq, t);
-          const bf8 yf = half ? split_frag<LDP, true>(s.dys, I * 16 + cq, gq, t) : split_frag<LDP>(s.dys, I * 16 + cq, gq, t);
+          const bf8 xf = half ? split_frag<LDP, true>(xs_, I * 16 + cq, gq, t) : split_frag<LDP>(xs_, I * 16 + cq, gq, t);
+          const bf8 yf = half ? split_frag<LDP, true>(dys_, I * 16 + cq, gq, t) : split_frag<LDP>(dys_, I * 16 + cq, gq, t);
           q = mfma_bf(xf, dsl[t], q);
           r = mfma_bf(yf, hl_[t], r);
           q = mfma_bf(xf, dsh[t], q);
@@ -1183,21 +1213,24 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     }
 
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 5>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    // the state operands are done with: their registers take the next head's tiles, which travel while the levels run
+    if (TWO_SETS && more) request(head_of(hh + 1));
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 4>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    bwd_big_level_bf<LDM, 5>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 3>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    bwd_big_level_bf<LDM, 4>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, s.dmr, s.dmt, e1, x2, cq, gq);
+    bwd_mid_level_bf<LDM, 3>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
     pin16(cs); pin16(e1); pin16(x2);
@@ -1205,7 +1238,9 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     float old[16];
     if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_small_levels_bf<LDM>(cs, Bv, dtp, Cv, s.dmr, e1, x2, gq);
+    bwd_small_levels_bf<LDM>(cs, Bv, dtp, Cv, dm_, e1, x2, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    if (TWO_SETS && more) deposit(set ^ 1);  // nobody reads that set before the barrier at the end of this head
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase (as in k_bwd_chunk)
@@ -1270,6 +1305,7 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
       partA[vec_off(p, u.bt, u.c, u.h) + n] = sumA;
       partBias[vec_off(p, u.bt, u.c, u.h) + n] = sumB;
     }
+    if (TWO_SETS) __syncthreads();  // the next head's tiles are in place, this head's are no longer read
   }
 
   {

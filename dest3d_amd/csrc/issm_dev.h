@@ -802,6 +802,53 @@ __device__ __forceinline__ void dy_load(const KP& p, const Unit& u, const float*
   }
 }
 
+// The same tiles for bf16 tensors as raw pairs of bf16 (no trip through fp32): group i of thread `tid` (lp_load's
+// layout) in r[i], zeros where the row or the columns do not exist.  dy from the gated fp32 workspace is rounded here.
+template <int PT, bool FULL>
+__device__ __forceinline__ void lp_load_bf(const KP& p, const Unit& u, const TensorD& t, uint2 (&r)[PT], int tid) {
+  if (lp_vec_ok(p, t, 2)) {
+    constexpr int G4 = 4 * PT;
+    const uint16_t* q = (const uint16_t*)t.ptr + ((long)u.b * t.s0 + (long)u.h * t.s2);
+    const int nvalid = min(CS, p.L - u.c * CS);
+    const long ss = (long)(u.dir ? -1 : 1) * t.s1;
+    const long r0 = (long)(u.dir ? p.L - 1 - u.c * CS : u.c * CS) * t.s1;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const int e4 = tid + i * NTHREADS, l = e4 / G4, p4 = (e4 % G4) * 4;
+      const bool ok = p4 < p.P && (FULL || l < nvalid);
+      const uint2 w = *(const uint2*)(q + (ok ? r0 + l * ss + p4 : 0));
+      r[i] = ok ? w : make_uint2(0u, 0u);
+    }
+  } else {
+    float v[CS * PT * 16 / NTHREADS];
+    lp_load<true, PT, FULL>(p, u, t, v, tid);
+#pragma unroll
+    for (int i = 0; i < PT; ++i)  // exact: the values are bf16
+      r[i] = make_uint2(pack_bf16(v[4 * i], v[4 * i + 1]), pack_bf16(v[4 * i + 2], v[4 * i + 3]));
+  }
+}
+template <int PT, bool FULL>
+__device__ __forceinline__ void dy_load_bf(const KP& p, const Unit& u, const float* dy_ws, uint2 (&r)[PT], int tid) {
+  if (dy_ws) {
+    float v[CS * PT * 16 / NTHREADS];
+    dy_load<true, PT, FULL>(p, u, dy_ws, v, tid);
+#pragma unroll
+    for (int i = 0; i < PT; ++i)
+      r[i] = make_uint2(pack_bf16(v[4 * i], v[4 * i + 1]), pack_bf16(v[4 * i + 2], v[4 * i + 3]));
+  } else {
+    lp_load_bf<PT, FULL>(p, u, p.dout[u.dir], r, tid);
+  }
+}
+template <int PT, int LD>
+__device__ __forceinline__ void lp_store_raw(const uint2 (&r)[PT], uint16_t* dst, int tid) {
+  constexpr int G4 = 4 * PT;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int e4 = tid + i * NTHREADS;
+    *(uint2*)(dst + (e4 / G4) * LD + (e4 % G4) * 4) = r[i];
+  }
+}
+
 // Lower triangle (s <= l, rest zero) of a 64x64 fp32 block: registers, then LDS dst[l][s] (ld = LDC).
 __device__ __forceinline__ void tril_load(const float* __restrict__ src, f4 (&v)[4], int tid = threadIdx.x) {
 #pragma unroll

@@ -179,9 +179,9 @@ int issm_stage_chunk_scan(const issm_scan_args* args, const float* states, const
 int issm_stage_bwd_gate(const issm_scan_args* args, const float* out_x, float* dy_gated);
 /* issm_stage_bwd_dstates: dH_c = dy^T . (C*exp(cs)) into dstates (Bt,nc,H,P,N) and
  *   dM = tril(dy . x^T) into dm (Bt,nc,H,64,64); either output may be NULL.  `dy` is args->dout
- *   unless dy_gated is given.  With io_dtype = ISSM_BF16 a block of dm holds, in the same 16 KB, two bf16 copies
- *   instead of one fp32 matrix: dM[l][s] (64 x 64 bf16, entries above the diagonal of the off-diagonal 16 x 16
- *   blocks unwritten) followed by its transpose -- the form issm_stage_bwd_chunk reads for bf16 inputs.  Replaces _chunk_scan_bwd_dstates (issm_chunk_scan.py:380-512) and
+ *   unless dy_gated is given.  With io_dtype = ISSM_BF16 a block of dm holds, in the first 8 of its 16 KB, the
+ *   symmetric 64 x 64 bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] instead of the fp32 lower triangle -- the form
+ *   issm_stage_bwd_chunk reads for bf16 inputs.  Replaces _chunk_scan_bwd_dstates (issm_chunk_scan.py:380-512) and
  *   _chunk_scan_bwd_dcb (issm_chunk_scan.py:790-900). */
 int issm_stage_bwd_dstates(const issm_scan_args* args, const float* dy_gated, float* dstates, float* dm);
 /* issm_stage_state_passing_bwd: reverse recurrence in place (dstates[c] becomes dS_c, the gradient
