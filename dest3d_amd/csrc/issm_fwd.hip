@@ -128,12 +128,30 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       cf = lane_coef(p, u.h, n, vn);
     }
 
+    // Decays inside the lane's groups of four rows (rows 4J .. 4J+3 of tile J), from three exponentials per group:
+    //   up[k] = 2^(cs[k] - cs[4J])  and  lo[k] = 2^(cs[4J+3] - cs[k]),  all <= 1.
+    // Every other decay the slice needs is one of these times a factor that is the same for the four rows of a group
+    // (2^(cs[4J] - ref) for rows after the reference row of a level, 2^(ref - cs[4J+3]) for rows up to it, again
+    // <= 1): one exponential per group and level instead of one per element.
+    float up[16], lo[16], d21[4];  // d21[J] = 2^(cs[4J+2] - cs[4J+1]), the one in-group decay that is neither
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      const float d1 = ex2(cs[4 * J + 1] - cs[4 * J]), d2 = ex2(cs[4 * J + 2] - cs[4 * J + 1]);
+      const float d3 = ex2(cs[4 * J + 3] - cs[4 * J + 2]);
+      d21[J] = d2;
+      up[4 * J] = 1.0f; up[4 * J + 1] = d1; up[4 * J + 2] = d1 * d2; up[4 * J + 3] = up[4 * J + 2] * d3;
+      lo[4 * J + 3] = 1.0f; lo[4 * J + 2] = d3; lo[4 * J + 1] = d2 * d3; lo[4 * J] = up[4 * J + 3];
+    }
+
     if (want_s) {
       // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
       f4 acc[PT];
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-      rows_product_split<PT, LDT, SPLIT ? 1 : 2>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * ex2(last - cs[k]); }, cm, g4);
+      float tail[4];  // 2^(last - cs[4J+3])
+#pragma unroll
+      for (int J = 0; J < 4; ++J) tail[J] = ex2(last - cs[4 * J + 3]);
+      rows_product_split<PT, LDT, SPLIT ? 1 : 2>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * (lo[k] * tail[k >> 2]); }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
       const int nn = n0 + wave * 16 + cm;
       if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
@@ -163,7 +181,9 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
           for (int js = 0; js <= jl; ++js) {
             const int kl = 4 * J + jl, ks = 4 * J + js;
             const float cb = cv[kl] * bd[ks];
-            sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * ex2(cs[kl] - cs[ks]);
+            // 2^(cs[kl] - cs[ks]): pairs with the group's first row are entries of up, with its last row of lo
+            const float dec = js == 0 ? up[kl] : jl == 3 ? lo[ks] : d21[J];
+            sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * dec;
           }
       // reference rows of the four levels: cross-lane fetches, all issued before the first is used
       const float r15 = __shfl(cs[3], cm + 48, 64), r31 = __shfl(cs[7], cm + 48, 64), r47 = __shfl(cs[11], cm + 48, 64);
@@ -175,21 +195,40 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       const int col = wave * 16 + cm;
       float v[16];
       // levels 16 and 32 pair rows of different tiles: the role of a row is fixed by its tile
+      // rows after a level's reference row: C * up * 2^(cs[4J] - ref); rows up to it: Bd * lo * 2^(ref - cs[4J+3])
       auto big16 = [&]() {
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-          const int J = k >> 2;
+        for (int J = 0; J < 4; ++J) {
           const float ref = (J & 2) ? r47 : r15;
-          v[k] = (J & 1) ? cv[k] * ex2(cs[k] - ref) : bd[k] * ex2(ref - cs[k]);
+          const float e = (J & 1) ? ex2(cs[4 * J] - ref) : ex2(ref - cs[4 * J + 3]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int k = 4 * J + j;
+            v[k] = (J & 1) ? cv[k] * (up[k] * e) : bd[k] * (lo[k] * e);
+          }
         }
       };
       auto big32 = [&]() {
 #pragma unroll
-        for (int k = 0; k < 16; ++k) v[k] = (k >> 3) ? cv[k] * ex2(cs[k] - r31) : bd[k] * ex2(r31 - cs[k]);
-      };
-      auto mid = [&](const float (&ref)[4], bool up, float sg) {
+        for (int J = 0; J < 4; ++J) {
+          const float e = (J & 2) ? ex2(cs[4 * J] - r31) : ex2(r31 - cs[4 * J + 3]);
 #pragma unroll
-        for (int k = 0; k < 16; ++k) v[k] = (up ? cv[k] : bd[k]) * ex2(sg * (cs[k] - ref[k >> 2]));
+          for (int j = 0; j < 4; ++j) {
+            const int k = 4 * J + j;
+            v[k] = (J & 2) ? cv[k] * (up[k] * e) : bd[k] * (lo[k] * e);
+          }
+        }
+      };
+      auto mid = [&](const float (&ref)[4], bool upper, float /*sg*/) {
+#pragma unroll
+        for (int J = 0; J < 4; ++J) {
+          const float e = ex2(upper ? cs[4 * J] - ref[J] : ref[J] - cs[4 * J + 3]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int k = 4 * J + j;
+            v[k] = (upper ? cv[k] : bd[k]) * ((upper ? up[k] : lo[k]) * e);
+          }
+        }
       };
       // products of one pass: T16 / T32 / T8 / T4 name the (hi, lo) tiles holding that level (nullptr = not in this pass)
       auto products = [&](const uint16_t* h16, const uint16_t* l16, const uint16_t* h32, const uint16_t* l32,
