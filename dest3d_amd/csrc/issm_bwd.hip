@@ -947,8 +947,25 @@ __device__ __forceinline__ bf8 frag4_lo(const uint16_t* q, bool keep = true) {
   return __builtin_shufflevector(a, z, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// In-group decays of the lane's rows (rows 4J .. 4J+3 of tile J): up[k] = 2^(cs[k] - cs[4J]), lo[k] = 2^(cs[4J+3] - cs[k]),
+// d21[J] = 2^(cs[4J+2] - cs[4J+1]), from three exponentials per group.  A level's factor of a row is up (rows after the
+// level's reference row) or lo (rows up to it) times one exponential per group, all <= 1.
+struct GroupDecays {
+  float up[16], lo[16], d21[4];
+};
+__device__ __forceinline__ void group_decays(const float (&cs)[16], GroupDecays& g) {
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    const float d1 = ex2(cs[4 * J + 1] - cs[4 * J]), d2 = ex2(cs[4 * J + 2] - cs[4 * J + 1]);
+    const float d3 = ex2(cs[4 * J + 3] - cs[4 * J + 2]);
+    g.d21[J] = d2;
+    g.up[4 * J] = 1.0f; g.up[4 * J + 1] = d1; g.up[4 * J + 2] = d1 * d2; g.up[4 * J + 3] = g.up[4 * J + 2] * d3;
+    g.lo[4 * J + 3] = 1.0f; g.lo[4 * J + 2] = d3; g.lo[4 * J + 1] = d2 * d3; g.lo[4 * J] = g.up[4 * J + 3];
+  }
+}
+
 template <int LDM, int LV>
-__device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+__device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
                                                  float (&e1)[16], float (&x2)[16], int cm, int g4) {
   float op[16], ee[16];
@@ -958,10 +975,11 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const fl
   for (int J = 0; J < 4; ++J) {
     const float ref = (J & 2) ? ref_b : ref_a;
     const bool upper = LV == 4 ? (J & 1) : (J & 2);
+    const float edge = ex2(upper ? cs[4 * J] - ref : ref - cs[4 * J + 3]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const float e = ex2(upper ? cs[k] - ref : ref - cs[k]);
+      const float e = (upper ? gd.up[k] : gd.lo[k]) * edge;
       ee[k] = e;
       op[k] = (upper ? Cv[k] : Bv[k] * dtp[k]) * e;
     }
@@ -1006,11 +1024,11 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const fl
 }
 
 template <int LDM, int LV>
-__device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+__device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
                                                  float (&e1)[16], float (&x2)[16], int cm, int g4) {
   const bool up = LV == 2 ? (g4 & 1) : (g4 & 2);  // role of the lane's rows 4 g4 + j
-  const float upf = up ? 1.0f : 0.0f, lof = up ? 0.0f : 1.0f, sg = up ? 1.0f : -1.0f;
+  const float upf = up ? 1.0f : 0.0f, lof = up ? 0.0f : 1.0f;
   // A operand: row i = cm of T_w (see bwd_mid_level), columns 4 g4 + jj; non-zero only where (i, kk) is a level-w pair
   const int cg = cm >> 2;
   const bool iup = LV == 2 ? (cg & 1) : (cg & 2);
@@ -1024,10 +1042,15 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const fl
 #pragma unroll
   for (int I = 0; I < 4; ++I) a[I] = frag4_lo(abase + I * (16 * LDM + 16), nz);
 #pragma unroll
-  for (int k = 0; k < 16; ++k) {
-    const float e = ex2(sg * (cs[k] - refs[k >> 2]));
-    ee[k] = e;
-    op[k] = (up ? Cv[k] : Bv[k] * dtp[k]) * e;
+  for (int J = 0; J < 4; ++J) {
+    const float edge = ex2(up ? cs[4 * J] - refs[J] : refs[J] - cs[4 * J + 3]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * J + j;
+      const float e = (up ? gd.up[k] : gd.lo[k]) * edge;
+      ee[k] = e;
+      op[k] = (up ? Cv[k] : Bv[k] * dtp[k]) * e;
+    }
   }
   const f4 z = {0, 0, 0, 0};
 #pragma unroll
@@ -1043,7 +1066,7 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const fl
 }
 
 template <int LDM>
-__device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+__device__ __forceinline__ void bwd_small_levels_bf(const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                     const uint16_t* __restrict__ dmr, float (&e1)[16], float (&x2)[16],
                                                     int g4) {
 #pragma unroll
@@ -1068,7 +1091,7 @@ __device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const
 #pragma unroll
       for (int js = 0; js < jl; ++js) {
         const int ks = 4 * J + js;
-        const float wgt = at(jl, js) * ex2(cs[kl] - cs[ks]);
+        const float wgt = at(jl, js) * (js == 0 ? gd.up[kl] : jl == 3 ? gd.lo[ks] : gd.d21[J]);
         e1[ks] = fmaf(wgt, Cv[kl], e1[ks]);
         x2[kl] = fmaf(wgt, Bd[js], x2[kl]);
       }
@@ -1170,6 +1193,8 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     float dtp[16], cs[16], dfac[16];
     const float last = lane_prep<true>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dfac);
     pin16(cs);
+    GroupDecays gd;
+    group_decays(cs, gd);
 
     int cq = cm, gq = g4;
     asm volatile("" : "+v"(cq), "+v"(gq));
@@ -1204,10 +1229,11 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
           q = mfma_bf(xf, dsh[t], q);
           r = mfma_bf(yf, hh_[t], r);
         }
+        const float tail = ex2(last - cs[4 * I + 3]), head = ex2(cs[4 * I]);
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          e1[4 * I + rr] = ex2(last - cs[4 * I + rr]) * q[rr];
-          x2[4 * I + rr] = ex2(cs[4 * I + rr]) * r[rr];
+          e1[4 * I + rr] = (gd.lo[4 * I + rr] * tail) * q[rr];
+          x2[4 * I + rr] = (gd.up[4 * I + rr] * head) * r[rr];
         }
       }
     }
@@ -1217,28 +1243,28 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     if (TWO_SETS && more) request(head_of(hh + 1));
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 5>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin_group_ends(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 5>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 4>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin_group_ends(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 4>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 3>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin_group_ends(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 3>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin_group_ends(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 2>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin16(cs); pin16(e1); pin16(x2);
+    pin_group_ends(cs); pin16(e1); pin16(x2);
     // the second direction adds to the first one's ddt: fetch it while the last levels run
     float old[16];
     if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_small_levels_bf<LDM>(cs, Bv, dtp, Cv, dm_, e1, x2, gq);
+    bwd_small_levels_bf<LDM>(gd, Bv, dtp, Cv, dm_, e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
     if (TWO_SETS && more) deposit(set ^ 1);  // nobody reads that set before the barrier at the end of this head
     __builtin_amdgcn_sched_barrier(0);
