@@ -166,7 +166,7 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
     f4 acc[PT];
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt) acc[pt] = (f4){0, 0, 0, 0};
-    rows_product_split<PT, LDT, IOB ? 2 : 1>(acc, s.dyt_hi, s.dyt_lo, [&](int k) { return ct[k]; }, cm, g4);
+    rows_product_split<PT, LDT, IOB ? 0 : 1>(acc, s.dyt_hi, s.dyt_lo, [&](int k) { return ct[k]; }, cm, g4);
     float* dst = dstates + dst_off(p, u.bt, u.c, u.h);
 #pragma unroll
     for (int pt = 0; pt < PT; ++pt)
