@@ -143,6 +143,30 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       lo[4 * J + 3] = 1.0f; lo[4 * J + 2] = d3; lo[4 * J + 1] = d2 * d3; lo[4 * J] = up[4 * J + 3];
     }
 
+    if (want_m) {
+      // pairs inside the lane's groups of four rows (levels 2, 1 and the diagonal)
+#pragma unroll
+      for (int J = 0; J < 4; ++J)
+#pragma unroll
+        for (int jl = 0; jl < 4; ++jl)
+#pragma unroll
+          for (int js = 0; js <= jl; ++js) {
+            const int kl = 4 * J + jl, ks = 4 * J + js;
+            const float cb = cv[kl] * bd[ks];
+            // 2^(cs[kl] - cs[ks]): pairs with the group's first row are entries of up, with its last row of lo
+            const float dec = js == 0 ? up[kl] : jl == 3 ? lo[ks] : d21[J];
+            sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * dec;
+          }
+    }
+    // What the levels (and the chunk state) multiply by their per-group factor: C * up for a row after a level's
+    // reference row, Bd * lo for a row up to it.  C, Bd, up and lo themselves are not needed beyond this point.
+    float pu[16], pl[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      pu[k] = cv[k] * up[k];
+      pl[k] = bd[k] * lo[k];
+    }
+
     if (want_s) {
       // S[p][n] = sum_l x[l][p] * Bd[l][n] exp2(last - cs[l][n]); B operand straight from registers
       f4 acc[PT];
@@ -151,7 +175,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       float tail[4];  // 2^(last - cs[4J+3])
 #pragma unroll
       for (int J = 0; J < 4; ++J) tail[J] = ex2(last - cs[4 * J + 3]);
-      rows_product_split<PT, LDT, SPLIT ? 1 : 0>(acc, s.xt_hi, s.xt_lo, [&](int k) { return bd[k] * (lo[k] * tail[k >> 2]); }, cm, g4);
+      rows_product_split<PT, LDT, SPLIT ? 1 : 0>(acc, s.xt_hi, s.xt_lo, [&](int k) { return pl[k] * tail[k >> 2]; }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
       const int nn = n0 + wave * 16 + cm;
       if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
@@ -172,19 +196,6 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
     }
 
     if (want_m) {
-      // pairs inside the lane's groups of four rows (levels 2, 1 and the diagonal)
-#pragma unroll
-      for (int J = 0; J < 4; ++J)
-#pragma unroll
-        for (int jl = 0; jl < 4; ++jl)
-#pragma unroll
-          for (int js = 0; js <= jl; ++js) {
-            const int kl = 4 * J + jl, ks = 4 * J + js;
-            const float cb = cv[kl] * bd[ks];
-            // 2^(cs[kl] - cs[ks]): pairs with the group's first row are entries of up, with its last row of lo
-            const float dec = js == 0 ? up[kl] : jl == 3 ? lo[ks] : d21[J];
-            sp[10 * J + jl * (jl + 1) / 2 + js] += jl == js ? cb : cb * dec;
-          }
       // reference rows of the four levels: cross-lane fetches, all issued before the first is used
       const float r15 = __shfl(cs[3], cm + 48, 64), r31 = __shfl(cs[7], cm + 48, 64), r47 = __shfl(cs[11], cm + 48, 64);
       float ref8[4], ref4[4];
@@ -195,7 +206,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       const int col = wave * 16 + cm;
       float v[16];
       // levels 16 and 32 pair rows of different tiles: the role of a row is fixed by its tile
-      // rows after a level's reference row: C * up * 2^(cs[4J] - ref); rows up to it: Bd * lo * 2^(ref - cs[4J+3])
+      // rows after a level's reference row: (C * up) * 2^(cs[4J] - ref); rows up to it: (Bd * lo) * 2^(ref - cs[4J+3])
       auto big16 = [&]() {
 #pragma unroll
         for (int J = 0; J < 4; ++J) {
@@ -204,7 +215,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int k = 4 * J + j;
-            v[k] = (J & 1) ? cv[k] * (up[k] * e) : bd[k] * (lo[k] * e);
+            v[k] = ((J & 1) ? pu[k] : pl[k]) * e;
           }
         }
       };
@@ -215,7 +226,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int k = 4 * J + j;
-            v[k] = (J & 2) ? cv[k] * (up[k] * e) : bd[k] * (lo[k] * e);
+            v[k] = ((J & 2) ? pu[k] : pl[k]) * e;
           }
         }
       };
@@ -226,7 +237,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int k = 4 * J + j;
-            v[k] = (upper ? cv[k] : bd[k]) * ((upper ? up[k] : lo[k]) * e);
+            v[k] = (upper ? pu[k] : pl[k]) * e;
           }
         }
       };
