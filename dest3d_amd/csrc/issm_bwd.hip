@@ -964,7 +964,7 @@ __device__ __forceinline__ void group_decays(const float (&cs)[16], GroupDecays&
   }
 }
 
-template <int LDM, int LV>
+template <int LDM, int LV, bool GD>
 __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
                                                  float (&e1)[16], float (&x2)[16], int cm, int g4) {
@@ -975,11 +975,11 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const Gr
   for (int J = 0; J < 4; ++J) {
     const float ref = (J & 2) ? ref_b : ref_a;
     const bool upper = LV == 4 ? (J & 1) : (J & 2);
-    const float edge = ex2(upper ? cs[4 * J] - ref : ref - cs[4 * J + 3]);
+    const float edge = GD ? ex2(upper ? cs[4 * J] - ref : ref - cs[4 * J + 3]) : 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const float e = (upper ? gd.up[k] : gd.lo[k]) * edge;
+      const float e = GD ? (upper ? gd.up[k] : gd.lo[k]) * edge : ex2(upper ? cs[k] - ref : ref - cs[k]);
       ee[k] = e;
       op[k] = (upper ? Cv[k] : Bv[k] * dtp[k]) * e;
     }
@@ -1023,7 +1023,7 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const Gr
   }
 }
 
-template <int LDM, int LV>
+template <int LDM, int LV, bool GD>
 __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
                                                  float (&e1)[16], float (&x2)[16], int cm, int g4) {
@@ -1043,11 +1043,11 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const Gr
   for (int I = 0; I < 4; ++I) a[I] = frag4_lo(abase + I * (16 * LDM + 16), nz);
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    const float edge = ex2(up ? cs[4 * J] - refs[J] : refs[J] - cs[4 * J + 3]);
+    const float edge = GD ? ex2(up ? cs[4 * J] - refs[J] : refs[J] - cs[4 * J + 3]) : 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const float e = (up ? gd.up[k] : gd.lo[k]) * edge;
+      const float e = GD ? (up ? gd.up[k] : gd.lo[k]) * edge : ex2(up ? cs[k] - refs[J] : refs[J] - cs[k]);
       ee[k] = e;
       op[k] = (up ? Cv[k] : Bv[k] * dtp[k]) * e;
     }
@@ -1065,8 +1065,8 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const Gr
   }
 }
 
-template <int LDM>
-__device__ __forceinline__ void bwd_small_levels_bf(const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+template <int LDM, bool GD>
+__device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                     const uint16_t* __restrict__ dmr, float (&e1)[16], float (&x2)[16],
                                                     int g4) {
 #pragma unroll
@@ -1091,7 +1091,7 @@ __device__ __forceinline__ void bwd_small_levels_bf(const GroupDecays& gd, const
 #pragma unroll
       for (int js = 0; js < jl; ++js) {
         const int ks = 4 * J + js;
-        const float wgt = at(jl, js) * (js == 0 ? gd.up[kl] : jl == 3 ? gd.lo[ks] : gd.d21[J]);
+        const float wgt = at(jl, js) * (GD ? (js == 0 ? gd.up[kl] : jl == 3 ? gd.lo[ks] : gd.d21[J]) : ex2(cs[kl] - cs[ks]));
         e1[ks] = fmaf(wgt, Cv[kl], e1[ks]);
         x2[kl] = fmaf(wgt, Bd[js], x2[kl]);
       }
@@ -1193,8 +1193,11 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     float dtp[16], cs[16], dfac[16];
     const float last = lane_prep<true>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dfac);
     pin16(cs);
+    // The in-group decays pay with up to two head tiles; with three the kernel has no registers for them (it spills,
+    // +34 % time measured at head dimension 36) and takes one exponential per element and level instead.
+    constexpr bool GD = PT <= 2;
     GroupDecays gd;
-    group_decays(cs, gd);
+    if (GD) group_decays(cs, gd);
 
     int cq = cm, gq = g4;
     asm volatile("" : "+v"(cq), "+v"(gq));
@@ -1229,11 +1232,11 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
           q = mfma_bf(xf, dsh[t], q);
           r = mfma_bf(yf, hh_[t], r);
         }
-        const float tail = ex2(last - cs[4 * I + 3]), head = ex2(cs[4 * I]);
+        const float tail = GD ? ex2(last - cs[4 * I + 3]) : 0.0f, head = GD ? ex2(cs[4 * I]) : 0.0f;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          e1[4 * I + rr] = (gd.lo[4 * I + rr] * tail) * q[rr];
-          x2[4 * I + rr] = (gd.up[4 * I + rr] * head) * r[rr];
+          e1[4 * I + rr] = (GD ? gd.lo[4 * I + rr] * tail : ex2(last - cs[4 * I + rr])) * q[rr];
+          x2[4 * I + rr] = (GD ? gd.up[4 * I + rr] * head : ex2(cs[4 * I + rr])) * r[rr];
         }
       }
     }
@@ -1243,28 +1246,28 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     if (TWO_SETS && more) request(head_of(hh + 1));
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin_group_ends(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 5>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 5, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin_group_ends(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 4>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
+    bwd_big_level_bf<LDM, 4, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin_group_ends(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 3>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 3, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin_group_ends(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 2>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
+    bwd_mid_level_bf<LDM, 2, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    pin_group_ends(cs); pin16(e1); pin16(x2);
+    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
     // the second direction adds to the first one's ddt: fetch it while the last levels run
     float old[16];
     if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_small_levels_bf<LDM>(gd, Bv, dtp, Cv, dm_, e1, x2, gq);
+    bwd_small_levels_bf<LDM, GD>(cs, gd, Bv, dtp, Cv, dm_, e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
     if (TWO_SETS && more) deposit(set ^ 1);  // nobody reads that set before the barrier at the end of this head
     __builtin_amdgcn_sched_barrier(0);
