@@ -51,10 +51,30 @@ WORKLOADS = {
 }
 
 
+def synthetic_inputs(torch, Bsz, L, H, P, N, G=1, seed=1234, h0_std=0.0):
+    """The benchmark configurations' synthetic inputs: generated on the CPU in fp32 in a fixed order (x, dt_raw, A, B,
+    C, D, h0, dy, dfinal).  x ~ N(0,1); dt_raw ~ U(-4,-1) (to be softplus'ed); A = -exp(U(ln 1, ln 16)) per head,
+    broadcast over N; B, C ~ N(0, 1/sqrt(N)); D ~ N(0,1); h0 = 0 or N(0, h0_std).  The same sequence of draws as the
+    tests' generator, so a seed names the same problem in both (tests/test_oracle.py checks that)."""
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    u = lambda *s: torch.rand(*s, generator=g)
+    x = r(Bsz, L, H, P)
+    dt_raw = u(Bsz, L, H, N) * 3.0 - 4.0
+    A = -torch.exp(u(H) * math.log(16.0))[:, None].expand(H, N).contiguous()
+    Bm = r(Bsz, L, G, N) / math.sqrt(N)
+    Cm = r(Bsz, L, G, N) / math.sqrt(N)
+    D = r(H)
+    h0 = r(Bsz, H, P, N) * h0_std
+    dy = r(Bsz, L, H, P)
+    dfinal = r(Bsz, H, P, N)
+    return dict(x=x, dt_raw=dt_raw, A=A, B=Bm, C=Cm, D=D, h0=h0, dy=dy, dfinal=dfinal)
+
+
 def make_problem(torch, shape, ndir, dtype, seed=1235, h0_std=0.0):
-    from oracle.issm_ref import make_inputs   # data generator only (shared with the tests)
     SHAPE = shape
-    I = make_inputs(SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed, h0_std=h0_std)
+    I = synthetic_inputs(torch, SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed,
+                         h0_std=h0_std)
     g = torch.Generator().manual_seed(seed + 1)
     dev = "cuda"
     t = dict(x=[I["x"]], B=[I["B"]], C=[I["C"]], dy=[I["dy"]], dfinal=[I["dfinal"]])

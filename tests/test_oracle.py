@@ -324,3 +324,13 @@ def test_make_inputs_is_deterministic_and_in_range():
     assert a["dt_raw"].min() >= -4 and a["dt_raw"].max() <= -1
     assert (a["A"] <= -1).all() and (a["A"] >= -16).all()
     assert (a["A"][:, :1] == a["A"]).all()
+
+
+def test_bench_generator_draws_the_same_problem_as_the_tests_generator():
+    """bench.py carries its own copy of the generator (it may not import this package's checker outside its CPU
+    baseline): a seed must name the same tensors in both."""
+    import bench
+    a = R.make_inputs(2, 24, 3, 4, 8, G=1, seed=1235, h0_std=0.1)
+    b = bench.synthetic_inputs(torch, 2, 24, 3, 4, 8, G=1, seed=1235, h0_std=0.1)
+    for k in b:
+        assert torch.equal(a[k], b[k]), k
