@@ -175,7 +175,7 @@ __device__ __forceinline__ void k_chunk_local_body(const KP& p, float* __restric
       float tail[4];  // 2^(last - cs[4J+3])
 #pragma unroll
       for (int J = 0; J < 4; ++J) tail[J] = ex2(last - cs[4 * J + 3]);
-      rows_product_split<PT, LDT, SPLIT ? 1 : 0>(acc, s.xt_hi, s.xt_lo, [&](int k) { return pl[k] * tail[k >> 2]; }, cm, g4);
+      rows_product_split<PT, LDT, SPLIT ? 1 : 2>(acc, s.xt_hi, s.xt_lo, [&](int k) { return pl[k] * tail[k >> 2]; }, cm, g4);
       float* dst = states + st_off(p, u.bt, u.c, u.h);
       const int nn = n0 + wave * 16 + cm;
       if (FULL && p.P == PT * 16) {  // uniform: nothing to mask
