@@ -913,17 +913,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_mixed(KP p, const flo
 // running sums, decays, states and all accumulation stay fp32).  x and dy are bf16 already, so their tiles are exact
 // copies; dM arrives from k_bwd_dstates as the symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)]: the F sums
 // contract over the columns of dM and the G sums over its rows, and in T both are rows, contiguous for a lane's k-slots.
-// Up to three head tiles the workgroup holds two sets of tiles and uses them in turn: the next head's are requested
-// once the products over the head dimension are done (their registers are free then), land in the other set while
-// the levels run, and one barrier per head is all the exchange needs.  With four head tiles two sets would not leave
-// room for two workgroups per CU: one set, requested and waited for at the top of each head.
+// The tiles of a head are requested at the top of its turn, behind its column operands, and copied to LDS as raw
+// bf16.  (Holding the next head's tiles in registers while the levels run -- two sets of tiles in LDS, one barrier per
+// head -- was 1 - 2 % faster as long as there were registers for it; the d/d(cs) accumulator below has taken them.)
 template <int PT>
 struct BwdChunkBfSmem {
   static constexpr int KW = 16 * PT, LDP = KW + 8;  // x / dy tiles [l][p]
   static constexpr int LDM = CS + 8;                // dM tile [row][col]
-  static constexpr int SETS = PT <= 3 ? 2 : 1;
-  uint16_t xs[SETS][CS * LDP], dys[SETS][CS * LDP];
-  uint16_t dm[SETS][CS * LDM];  // T[i][j] = dM[max(i,j)][min(i,j)]
+  uint16_t xs[CS * LDP], dys[CS * LDP];
+  uint16_t dm[CS * LDM];  // T[i][j] = dM[max(i,j)][min(i,j)]
   float dbc[32 * NTHREADS];
 };
 
@@ -947,27 +945,10 @@ __device__ __forceinline__ bf8 frag4_lo(const uint16_t* q, bool keep = true) {
   return __builtin_shufflevector(a, z, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// In-group decays of the lane's rows (rows 4J .. 4J+3 of tile J): up[k] = 2^(cs[k] - cs[4J]), lo[k] = 2^(cs[4J+3] - cs[k]),
-// d21[J] = 2^(cs[4J+2] - cs[4J+1]), from three exponentials per group.  A level's factor of a row is up (rows after the
-// level's reference row) or lo (rows up to it) times one exponential per group, all <= 1.
-struct GroupDecays {
-  float up[16], lo[16], d21[4];
-};
-__device__ __forceinline__ void group_decays(const float (&cs)[16], GroupDecays& g) {
-#pragma unroll
-  for (int J = 0; J < 4; ++J) {
-    const float d1 = ex2(cs[4 * J + 1] - cs[4 * J]), d2 = ex2(cs[4 * J + 2] - cs[4 * J + 1]);
-    const float d3 = ex2(cs[4 * J + 3] - cs[4 * J + 2]);
-    g.d21[J] = d2;
-    g.up[4 * J] = 1.0f; g.up[4 * J + 1] = d1; g.up[4 * J + 2] = d1 * d2; g.up[4 * J + 3] = g.up[4 * J + 2] * d3;
-    g.lo[4 * J + 3] = 1.0f; g.lo[4 * J + 2] = d3; g.lo[4 * J + 1] = d2 * d3; g.lo[4 * J] = g.up[4 * J + 3];
-  }
-}
-
-template <int LDM, int LV, bool GD>
-__device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+template <int LDM, int LV>
+__device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
-                                                 float (&e1)[16], float (&x2)[16], int cm, int g4) {
+                                                 float (&e1)[16], float (&x2)[16], float (&dcs)[16], int cm, int g4) {
   float op[16], ee[16];
   const float ref_a = __shfl(LV == 4 ? cs[3] : cs[7], cm + 48, 64);
   const float ref_b = LV == 4 ? __shfl(cs[11], cm + 48, 64) : ref_a;
@@ -975,11 +956,10 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const Gr
   for (int J = 0; J < 4; ++J) {
     const float ref = (J & 2) ? ref_b : ref_a;
     const bool upper = LV == 4 ? (J & 1) : (J & 2);
-    const float edge = GD ? ex2(upper ? cs[4 * J] - ref : ref - cs[4 * J + 3]) : 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const float e = GD ? (upper ? gd.up[k] : gd.lo[k]) * edge : ex2(upper ? cs[k] - ref : ref - cs[k]);
+      const float e = ex2(upper ? cs[k] - ref : ref - cs[k]);
       ee[k] = e;
       op[k] = (upper ? Cv[k] : Bv[k] * dtp[k]) * e;
     }
@@ -989,44 +969,64 @@ __device__ __forceinline__ void bwd_big_level_bf(const float (&cs)[16], const Gr
 #pragma unroll
     for (int j = 0; j < 8; ++j) { lo8[j] = op[j]; hi8[j] = op[8 + j]; }
     const bf8 blo = pack_bf8(lo8), bhi = pack_bf8(hi8);
-    // all four operand fragments first, then the products
-    const bf8 a2 = split_frag<LDM>(dmr, 32 + cm, g4, 0), a3 = split_frag<LDM>(dmr, 48 + cm, g4, 0);
-    const bf8 a0 = split_frag<LDM>(dmt, cm, g4, 1), a1 = split_frag<LDM>(dmt, 16 + cm, g4, 1);
+    // two products at a time (F: rows of tiles 2, 3 gather from tiles 0, 1; then G: rows of tiles 0, 1 gather from
+    // tiles 2, 3), so that only two operand fragments and two results are live at once
     const f4 z = {0, 0, 0, 0};
-    const f4 f2 = mfma_bf(a2, blo, z), f3 = mfma_bf(a3, blo, z);   // F: rows of tiles 2, 3 gather from tiles 0, 1
-    const f4 g0 = mfma_bf(a0, bhi, z), g1 = mfma_bf(a1, bhi, z);   // G: rows of tiles 0, 1 gather from tiles 2, 3
+    {
+      const bf8 a2 = split_frag<LDM>(dmr, 32 + cm, g4, 0), a3 = split_frag<LDM>(dmr, 48 + cm, g4, 0);
+      const f4 f2 = mfma_bf(a2, blo, z), f3 = mfma_bf(a3, blo, z);
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      e1[rr] += ee[rr] * g0[rr];
-      e1[4 + rr] += ee[4 + rr] * g1[rr];
-      x2[8 + rr] += ee[8 + rr] * f2[rr];
-      x2[12 + rr] += ee[12 + rr] * f3[rr];
+      for (int rr = 0; rr < 4; ++rr) {
+        x2[8 + rr] += ee[8 + rr] * f2[rr];
+        x2[12 + rr] += ee[12 + rr] * f3[rr];
+        dcs[8 + rr] += (float)bhi[rr] * f2[rr];
+        dcs[12 + rr] += (float)bhi[4 + rr] * f3[rr];
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const bf8 a0 = split_frag<LDM>(dmt, cm, g4, 1), a1 = split_frag<LDM>(dmt, 16 + cm, g4, 1);
+      const f4 g0 = mfma_bf(a0, bhi, z), g1 = mfma_bf(a1, bhi, z);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        e1[rr] += ee[rr] * g0[rr];
+        e1[4 + rr] += ee[4 + rr] * g1[rr];
+        dcs[rr] -= (float)blo[rr] * g0[rr];
+        dcs[4 + rr] -= (float)blo[4 + rr] * g1[rr];
+      }
     }
   } else {
-    bf8 a[4], b[4];
+    bf8 b[4];
 #pragma unroll
     for (int I = 0; I < 4; ++I) {
       const int K = (I & 1) ? I - 1 : I + 1;  // the tile contracted over
-      a[I] = frag4_lo(((I & 1) ? dmr : dmt) + (I * 16 + cm) * LDM + K * 16 + 4 * g4);
       b[I] = pack_bf4_lo(op[4 * K], op[4 * K + 1], op[4 * K + 2], op[4 * K + 3]);
     }
     const f4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int I = 0; I < 4; ++I) {
-      const f4 acc = mfma_bf(a[I], b[I], z);
+      const int K = (I & 1) ? I - 1 : I + 1;
+      if (I == 2) __builtin_amdgcn_sched_barrier(0);  // two products at a time
+      const f4 acc = mfma_bf(frag4_lo(((I & 1) ? dmr : dmt) + (I * 16 + cm) * LDM + K * 16 + 4 * g4), b[I], z);
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        if (I & 1) x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
-        else e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+        const float fr = (float)b[(I & 1) ? I - 1 : I + 1][rr];  // this row's operand as the partner tile's product took it
+        if (I & 1) {
+          x2[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+          dcs[4 * I + rr] += fr * acc[rr];
+        } else {
+          e1[4 * I + rr] += ee[4 * I + rr] * acc[rr];
+          dcs[4 * I + rr] -= fr * acc[rr];
+        }
       }
     }
   }
 }
 
-template <int LDM, int LV, bool GD>
-__device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+template <int LDM, int LV>
+__device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                  const uint16_t* __restrict__ dmr, const uint16_t* __restrict__ dmt,
-                                                 float (&e1)[16], float (&x2)[16], int cm, int g4) {
+                                                 float (&e1)[16], float (&x2)[16], float (&dcs)[16], int cm, int g4) {
   const bool up = LV == 2 ? (g4 & 1) : (g4 & 2);  // role of the lane's rows 4 g4 + j
   const float upf = up ? 1.0f : 0.0f, lof = up ? 0.0f : 1.0f;
   // A operand: row i = cm of T_w (see bwd_mid_level), columns 4 g4 + jj; non-zero only where (i, kk) is a level-w pair
@@ -1043,11 +1043,10 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const Gr
   for (int I = 0; I < 4; ++I) a[I] = frag4_lo(abase + I * (16 * LDM + 16), nz);
 #pragma unroll
   for (int J = 0; J < 4; ++J) {
-    const float edge = GD ? ex2(up ? cs[4 * J] - refs[J] : refs[J] - cs[4 * J + 3]) : 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = 4 * J + j;
-      const float e = GD ? (up ? gd.up[k] : gd.lo[k]) * edge : ex2(up ? cs[k] - refs[J] : refs[J] - cs[k]);
+      const float e = ex2(up ? cs[k] - refs[J] : refs[J] - cs[k]);
       ee[k] = e;
       op[k] = (up ? Cv[k] : Bv[k] * dtp[k]) * e;
     }
@@ -1055,18 +1054,20 @@ __device__ __forceinline__ void bwd_mid_level_bf(const float (&cs)[16], const Gr
   const f4 z = {0, 0, 0, 0};
 #pragma unroll
   for (int I = 0; I < 4; ++I) {
-    const f4 acc = mfma_bf(a[I], pack_bf4_lo(op[4 * I], op[4 * I + 1], op[4 * I + 2], op[4 * I + 3]), z);
+    const bf8 bo = pack_bf4_lo(op[4 * I], op[4 * I + 1], op[4 * I + 2], op[4 * I + 3]);
+    const f4 acc = mfma_bf(a[I], bo, z);
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const float v = ee[4 * I + rr] * acc[rr];
       x2[4 * I + rr] = fmaf(v, upf, x2[4 * I + rr]);
       e1[4 * I + rr] = fmaf(v, lof, e1[4 * I + rr]);
+      dcs[4 * I + rr] = fmaf((float)bo[rr] * acc[rr], upf - lof, dcs[4 * I + rr]);
     }
   }
 }
 
-template <int LDM, bool GD>
-__device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const GroupDecays& gd, const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
+template <int LDM>
+__device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const float (&Bv)[16], const float (&dtp)[16], const float (&Cv)[16],
                                                     const uint16_t* __restrict__ dmr, float (&e1)[16], float (&x2)[16],
                                                     int g4) {
 #pragma unroll
@@ -1091,7 +1092,7 @@ __device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const
 #pragma unroll
       for (int js = 0; js < jl; ++js) {
         const int ks = 4 * J + js;
-        const float wgt = at(jl, js) * (GD ? (js == 0 ? gd.up[kl] : jl == 3 ? gd.lo[ks] : gd.d21[J]) : ex2(cs[kl] - cs[ks]));
+        const float wgt = at(jl, js) * ex2(cs[kl] - cs[ks]);
         e1[ks] = fmaf(wgt, Cv[kl], e1[ks]);
         x2[kl] = fmaf(wgt, Bd[js], x2[kl]);
       }
@@ -1136,7 +1137,6 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
   // The reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
   // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first.
   auto head_of = [&](int hh) { return u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh); };
-  constexpr bool TWO_SETS = SM::SETS == 2;
   // a head's tiles on their way from global memory to LDS: raw bf16 pairs (x, dy) and the thread's two 16-byte pieces
   // of T (rows tq >> 3 and 32 + (tq >> 3), columns 8 (tq & 7) .. + 7)
   uint2 nx[PT], ny[PT];
@@ -1155,22 +1155,17 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     nm0 = *(const uint4*)(dmb + mrow * CS + mcol);
     nm1 = *(const uint4*)(dmb + (32 + mrow) * CS + mcol);
   };
-  auto deposit = [&](int set) {
+  auto deposit = [&]() {
     int tq = tid;
     asm volatile("" : "+v"(tq));
     const int mrow = tq >> 3, mcol = (tq & 7) * 8;
-    lp_store_raw<PT, LDP>(ny, s.dys[set], tq);
-    lp_store_raw<PT, LDP>(nx, s.xs[set], tq);
-    *(uint4*)(s.dm[set] + mrow * LDM + mcol) = nm0;
-    *(uint4*)(s.dm[set] + (32 + mrow) * LDM + mcol) = nm1;
+    lp_store_raw<PT, LDP>(ny, s.dys, tq);
+    lp_store_raw<PT, LDP>(nx, s.xs, tq);
+    *(uint4*)(s.dm + mrow * LDM + mcol) = nm0;
+    *(uint4*)(s.dm + (32 + mrow) * LDM + mcol) = nm1;
   };
-  request(head_of(0));
-  deposit(0);
-  __syncthreads();
 
   for (int hh = 0; hh < p.hpg; ++hh) {
-    const int set = TWO_SETS ? (hh & 1) : 0;
-    const bool more = hh + 1 < p.hpg;  // uniform
     u.h = head_of(hh);
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
@@ -1179,25 +1174,18 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     const float gl = (g4 == 3 && vn) ? g_last[vec_off(p, u.bt, u.c, u.h) + n] : 0.0f;
     lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, dsv);
     lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, u.h), p.P, p.N, n, vn, g4, pn_full, hv);
-    if (!TWO_SETS && hh > 0) {  // one set of tiles: this head's replace the previous head's
-      request(u.h);
-      __syncthreads();  // the previous head no longer reads the tiles
-      deposit(0);
-      __syncthreads();
-    }
-    const uint16_t* xs_ = s.xs[set];
-    const uint16_t* dys_ = s.dys[set];
-    const uint16_t* dm_ = s.dm[set];
+    request(u.h);
+    __syncthreads();  // the previous head no longer reads the tiles
+    deposit();
+    __syncthreads();
+    const uint16_t* xs_ = s.xs;
+    const uint16_t* dys_ = s.dys;
+    const uint16_t* dm_ = s.dm;
 
     const float An = cf.A;
     float dtp[16], cs[16], dfac[16];
     const float last = lane_prep<true>(p, cf, vn, cm, g4, rm, raw, dtp, cs, dfac);
     pin16(cs);
-    // The in-group decays pay with up to two head tiles; with three the kernel has no registers for them (it spills,
-    // +34 % time measured at head dimension 36) and takes one exponential per element and level instead.
-    constexpr bool GD = PT <= 2;
-    GroupDecays gd;
-    if (GD) group_decays(cs, gd);
 
     int cq = cm, gq = g4;
     asm volatile("" : "+v"(cq), "+v"(gq));
@@ -1232,56 +1220,57 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
           q = mfma_bf(xf, dsh[t], q);
           r = mfma_bf(yf, hh_[t], r);
         }
-        const float tail = GD ? ex2(last - cs[4 * I + 3]) : 0.0f, head = GD ? ex2(cs[4 * I]) : 0.0f;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-          e1[4 * I + rr] = (GD ? gd.lo[4 * I + rr] * tail : ex2(last - cs[4 * I + rr])) * q[rr];
-          x2[4 * I + rr] = (GD ? gd.up[4 * I + rr] * head : ex2(cs[4 * I + rr])) * r[rr];
+          e1[4 * I + rr] = ex2(last - cs[4 * I + rr]) * q[rr];
+          x2[4 * I + rr] = ex2(cs[4 * I + rr]) * r[rr];
         }
       }
     }
 
     __builtin_amdgcn_sched_barrier(0);
-    // the state operands are done with: their registers take the next head's tiles, which travel while the levels run
-    if (TWO_SETS && more) request(head_of(hh + 1));
+    asm volatile("" : "+v"(cq), "+v"(gq));
+    pin16(cs); pin16(e1); pin16(x2);
+    bwd_small_levels_bf<LDM>(cs, Bv, dtp, Cv, dm_, e1, x2, gq);
+    __builtin_amdgcn_sched_barrier(0);
+    // d/d(cs) so far (state terms and in-lane pairs, all fp32): C . X2 - Bd . E1.  The matrix levels add their share to
+    // it directly, as (the operand as the matrix instruction took it, rounded to bf16) x (the product): a pair (i, j)
+    // then enters row i and, negated, row j as the same product of the same three numbers, and the suffix sums below,
+    // in which the two cancel for every row before j, are left with fp32 rounding instead of bf16 rounding.
+    float dcs[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) dcs[k] = Cv[k] * x2[k] - Bv[k] * dtp[k] * e1[k];
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 5, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin16(cs); pin16(e1); pin16(x2); pin16(dcs);
+    bwd_big_level_bf<LDM, 5>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, dcs, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
-    bwd_big_level_bf<LDM, 4, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin16(cs); pin16(e1); pin16(x2); pin16(dcs);
+    bwd_big_level_bf<LDM, 4>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, dcs, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 3, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
+    pin16(cs); pin16(e1); pin16(x2); pin16(dcs);
+    bwd_mid_level_bf<LDM, 3>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, dcs, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" : "+v"(cq), "+v"(gq));
-    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
-    bwd_mid_level_bf<LDM, 2, GD>(cs, gd, Bv, dtp, Cv, dm_, dm_, e1, x2, cq, gq);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("" : "+v"(cq), "+v"(gq));
-    if (GD) pin_group_ends(cs); else pin16(cs); pin16(e1); pin16(x2);
-    // the second direction adds to the first one's ddt: fetch it while the last levels run
+    pin16(cs); pin16(e1); pin16(x2); pin16(dcs);
+    // the second direction adds to the first one's ddt: fetch it while the last level runs
     float old[16];
     if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
-    bwd_small_levels_bf<LDM, GD>(cs, gd, Bv, dtp, Cv, dm_, e1, x2, gq);
-    __builtin_amdgcn_sched_barrier(0);
-    if (TWO_SETS && more) deposit(set ^ 1);  // nobody reads that set before the barrier at the end of this head
+    bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, dcs, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- column phase (as in k_bwd_chunk)
-    pin16(e1); pin16(x2);
-    float dcs[16], val[16];
+    pin16(e1); pin16(x2); pin16(dcs);
+    float val[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       const float E1 = e1[k], X2 = x2[k];
       s.dbc[k * NTHREADS + tid] += dtp[k] * E1;
       s.dbc[(16 + k) * NTHREADS + tid] += X2;
       val[k] = Bv[k] * E1;
-      dcs[k] = Cv[k] * X2 - Bv[k] * dtp[k] * E1;
     }
     dcs[15] += gl;
     {
@@ -1334,7 +1323,6 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
       partA[vec_off(p, u.bt, u.c, u.h) + n] = sumA;
       partBias[vec_off(p, u.bt, u.c, u.h) + n] = sumB;
     }
-    if (TWO_SETS) __syncthreads();  // the next head's tiles are in place, this head's are no longer read
   }
 
   {

@@ -35,9 +35,11 @@
  *    (16 significand bits per operand; relative error of a product <= 2^-16); every other
  *    product is fp32.  With io_dtype = ISSM_BF16 every matrix product takes its operands
  *    rounded once to bf16 (as the reference's kernels cast their dot operands to the input
- *    dtype, issm_triton/issm_cabt_bmm.py:42-43), except x.dS and dy.H, whose fp32 state
- *    operands enter as high and low parts.  Results are bit-reproducible from run to run
- *    (fixed-order reductions, no atomics).
+ *    dtype, issm_triton/issm_cabt_bmm.py:42-43), except x.dS, dy.H and the chunk state
+ *    x^T.(B dt' decay), whose fp32 operands enter as high and low parts; the gradient of
+ *    the running sum of dt'.A is assembled from identically rounded products, so that dA and
+ *    ddt_bias carry no accumulated rounding bias.  Results are bit-reproducible from run to
+ *    run (fixed-order reductions, no atomics).
  *  - Strides: stride[1] * seqlen must stay below 2^30 elements (row byte offsets are 32-bit).
  */
 #ifndef ISSM_H
