@@ -206,6 +206,48 @@ def test_packed_sequences_match_oracle(dtype):
             _check("d" + k, g[k].grad, ins[k].grad, bt)
 
 
+def test_packed_sequences_randomised():
+    """Seeded draws of shapes, options and change points (up to five per batch row, anywhere, repeats allowed) in fp32
+    and bf16 against the oracle's recurrence with resets."""
+    from dest3d_amd import ISSM_chunk_scan_combined
+    rng = torch.Generator().manual_seed(606)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    flip = lambda: bool(torch.randint(0, 2, (1,), generator=rng))
+    for trial in range(8):
+        dtype = torch.bfloat16 if trial % 4 == 3 else torch.float32
+        G = pick(1, 2)
+        H = G * pick(1, 2)
+        Bsz, L_, P, N = pick(1, 3), [pick(2, 200), 64 * pick(1, 4)][trial % 2], pick(1, 64), [pick(1, 200), 64, 128][trial % 3]
+        kw = dict(h0=flip(), softplus=flip(), D=[None, "h", "hp"][pick(0, 2)], z=flip(), bias=flip())
+        case = (Bsz, L_, H, P, N, G, kw, str(dtype))
+        _say(f"randomised seq_idx {trial}: {case}")
+        d = _problem(Bsz, L_, H, P, N, G, seed=700 + trial, **kw)
+        if dtype == torch.bfloat16:
+            for k in ("x", "dt", "B", "C", "z"):
+                d[k] = None if d[k] is None else d[k].bfloat16().float()
+        seq = _seq_ids(Bsz, L_, [[pick(0, L_ - 1) for _ in range(pick(0, 5))] for _ in range(Bsz)])
+        ins = {k: d[k].double().clone().requires_grad_() for k in GRAD_NAMES if d[k] is not None}
+        y_ref, fin_ref = R.issm_scan_sequential(ins["x"], ins["dt"], ins["A"], ins["B"], ins["C"], D=ins.get("D"),
+                                                z=ins.get("z"), dt_bias=ins.get("dt_bias"), initial_states=ins.get("h0"),
+                                                dt_softplus=d["softplus"], dt_limit=d["dt_limit"], seq_idx=seq)
+        ((y_ref * d["dy"].double()).sum() + (fin_ref * d["dfinal"].double()).sum()).backward()
+        cast = lambda t, dt_=dtype: None if t is None else t.to("cuda", dt_).requires_grad_()
+        g = dict(x=cast(d["x"]), dt=cast(d["dt"]), A=cast(d["A"], torch.float32), B=cast(d["B"]), C=cast(d["C"]),
+                 D=cast(d["D"], torch.float32), z=cast(d["z"]), dt_bias=cast(d["dt_bias"], torch.float32),
+                 h0=cast(d["h0"], torch.float32))
+        y, fin = ISSM_chunk_scan_combined(g["x"], g["dt"], g["A"], g["B"], g["C"], 64, D=g["D"], z=g["z"],
+                                          dt_bias=g["dt_bias"], initial_states=g["h0"], seq_idx=seq.cuda(),
+                                          dt_softplus=d["softplus"], dt_limit=d["dt_limit"], return_final_states=True)
+        ((y.float() * d["dy"].cuda()).sum() + (fin * d["dfinal"].cuda()).sum()).backward()
+        torch.cuda.synchronize()
+        ft, bt = (FWD32, BWD32) if dtype == torch.float32 else (FWD16, BWD16)
+        _check(f"out {case}", y, y_ref.detach(), ft)
+        _check(f"final_states {case}", fin, fin_ref.detach(), ft)
+        for k in GRAD_NAMES:
+            if d[k] is not None:
+                _check(f"d{k} {case}", g[k].grad, ins[k].grad, bt)
+
+
 def test_packed_sequences_equal_separate_calls():
     """Two sequences packed into one row give what two calls give, the second without an initial state; a constant
     seq_idx changes nothing (to rounding: a call with seq_idx runs the general kernel variants for every chunk, a call
