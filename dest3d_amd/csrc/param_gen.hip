@@ -15,6 +15,20 @@ namespace issm {
 constexpr int PG_MAXR0 = 12;  // largest H + 2G built (three 4-row steps of the matrix instruction)
 constexpr int PG_M = 16;      // distance encoding width this kernel is built for
 constexpr int PG_TOK = 4;     // tokens per workgroup in the backward (one per wave)
+constexpr int PG_LDT = 20;    // row stride of the backward's 16 x 16 LDS tiles (column-wise reads of four row groups
+                              // fall into different banks; rows stay 8- and 16-byte aligned)
+
+// sum over the 16 lanes that share lane >> 4; valid in the lane with (lane & 15) == 15
+__device__ __forceinline__ float row_sum16_(float v) {
+#define ISSM_PG_DPP_ADD(ctrl) \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+  ISSM_PG_DPP_ADD(0x111);  // row_shr:1
+  ISSM_PG_DPP_ADD(0x112);  // row_shr:2
+  ISSM_PG_DPP_ADD(0x114);  // row_shr:4
+  ISSM_PG_DPP_ADD(0x118);  // row_shr:8
+#undef ISSM_PG_DPP_ADD
+  return v;
+}
 
 template <bool BF>
 __device__ __forceinline__ void load_row16(const void* p, long off, float (&v)[PG_M]) {
@@ -209,10 +223,13 @@ __device__ __forceinline__ float dsoftplus_(float x) { return x <= 20.0f ? sigmo
 // pointer advanced once per trip plus a compile-time offset.  UNR blocks of 16 k have their loads in flight together.
 template <bool BF, bool FULLK, bool HASW>
 __global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
-  constexpr int UNR = HASW ? 2 : 4;
+  constexpr int UNR = (HASW || !BF) ? 2 : 4;
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   typedef typename std::conditional<BF, uint2, f4>::type T4;
   __shared__ float wred[4][16 * PG_M];
+  // per-wave transposition tiles of the FULLK path: effective gradients [row][k] and the dist block [k][m]
+  __shared__ __align__(16) float sg[FULLK ? 4 : 1][FULLK ? UNR : 1][FULLK ? 16 * PG_LDT : 4];
+  __shared__ __align__(16) T sd[FULLK ? 4 : 1][FULLK ? UNR : 1][FULLK ? 16 * PG_LDT : 8];
   const int R0 = p.H + 2 * p.G, R = R0 + (p.has_back ? 2 * p.G : 0);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = lane & 15, q = lane >> 4;
@@ -313,79 +330,94 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
     bs = 0.0f;
     bsb = 0.0f;
     if constexpr (FULLK) {
+      // Every operand is read once, with one 8- or 16-byte load per lane, in the layout whose lane index is the
+      // gradient row (lane (i, q): row i, columns k0 + 4q .. + 3).  The second layout the products need -- lane index
+      // = column -- comes out of a 16 x 16 tile per wave in LDS, written row-wise and read column-wise; so does the
+      // block of dist (16 k x 16 m, loaded as 64 pieces of four adjacent m).  Reading both layouts from global memory
+      // took fourteen 2-byte-per-lane loads per block, and the load pipe, not HBM, set the pace.
       const T* nil = (const T*)p.dist;  // what a lane with no row reads (at least 64 * 16 elements long)
       const T* pa = ok2 ? (const T*)g2 + o2 + 4 * q : nil;
       const T* pab = ok2b ? (const T*)g2b + o2 + 4 * q : nil;
-      const T* pd = (const T*)p.dist + (t * K + 4 * q) * PG_M + i;
-      const T *pg[3], *pgb[3];
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-        pg[s] = okg[s] ? (const T*)g1[s] + o1[s] + i : nil;
-        pgb[s] = okgb[s] ? (const T*)g1b[s] + o1[s] + i : nil;
-      }
-      // HASW: raw in both layouts, weights in both layouts
+      const T* pd = (const T*)p.dist + (t * K + 4 * q + (i >> 2)) * PG_M + 4 * (i & 3);
       const T* pr2 = isdt2 ? (const T*)p.dt_raw + o2 + 4 * q : nil;
-      const T* pr1[3];
-#pragma unroll
-      for (int s = 0; s < 3; ++s) pr1[s] = isdt1[s] ? (const T*)p.dt_raw + o1[s] + i : nil;
       const float* pw2 = HASW ? p.weights + t * K + 4 * q : nullptr;
-      const float* pw1 = HASW ? p.weights + t * K + i : nullptr;
       T* pdd = p.ddist ? (T*)p.ddist + (t * K + i) * PG_M + 4 * q : nullptr;
-      float* pdw = (HASW && p.dweights) ? p.dweights + t * K + i : nullptr;
+      float* pdw = (HASW && p.dweights) ? p.dweights + t * K + 4 * q : nullptr;
       for (int kb = 0; kb < K; kb += 16 * UNR) {
-        T4 ra[UNR], rab[UNR], rr2[UNR];
+        T4 ra[UNR], rab[UNR], rr2[UNR], rd[UNR];
         f4 rw2[UNR];
-        T rd[UNR][4], rg[UNR][3], rgb[UNR][3], rr1[UNR][3];
-        float rw1[UNR];
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
           ra[u] = *(const T4*)(pa + 16 * u);
           if (any_back) rab[u] = *(const T4*)(pab + 16 * u);
-#pragma unroll
-          for (int v = 0; v < 4; ++v) rd[u][v] = pd[(16 * u + v) * PG_M];
-#pragma unroll
-          for (int s = 0; s < 3; ++s) {
-            rg[u][s] = pg[s][16 * u];
-            if (any_back) rgb[u][s] = pgb[s][16 * u];
-            if constexpr (HASW) rr1[u][s] = pr1[s][16 * u];
-          }
+          rd[u] = *(const T4*)(pd + 16 * u * PG_M);
           if constexpr (HASW) {
             rr2[u] = *(const T4*)(pr2 + 16 * u);
             rw2[u] = *(const f4*)(pw2 + 16 * u);
-            rw1[u] = pw1[16 * u];
           }
         }
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-          // rows past R0 hold junk in `a`: they only reach rows of dW that are never read
-          float dv[4], x[3], xb[3], raw1[3];
+          float* S = sg[wave][u];
+          T* D = sd[wave][u];
+          f4 a = ok2 ? widen(ra[u]) : zero4;
+          const f4 ab = (any_back && ok2b) ? widen(rab[u]) : zero4;
+          f4 pw = zero4;  // ddt * softplus(raw): the weight's gradient once summed over the heads
+          if constexpr (HASW) {
+            if (isdt2) {
+              const f4 raw = widen(rr2[u]);
 #pragma unroll
-          for (int v = 0; v < 4; ++v) dv[v] = widen1(rd[u][v]);
-#pragma unroll
-          for (int s = 0; s < 3; ++s) {
-            x[s] = okg[s] ? widen1(rg[u][s]) : 0.0f;
-            xb[s] = (any_back && okgb[s]) ? widen1(rgb[u][s]) : 0.0f;
-            raw1[s] = HASW ? widen1(rr1[u][s]) : 0.0f;
+              for (int v = 0; v < 4; ++v) {
+                const float tt = ex2(raw[v] * LOG2E), uu = 1.0f + tt;
+                const bool big = raw[v] > 20.0f;  // torch's softplus threshold
+                pw[v] = a[v] * (big ? raw[v] : LN2 * __builtin_amdgcn_logf(uu));
+                a[v] *= rw2[u][v] * (big ? 1.0f : tt * __builtin_amdgcn_rcpf(uu));
+              }
+            }
           }
-          block(widen(ra[u]), (any_back && ok2b) ? widen(rab[u]) : zero4, HASW ? widen(rr2[u]) : zero4,
-                HASW ? rw2[u] : zero4, dv, x, xb, raw1, HASW ? rw1[u] : 0.0f,
-                pdd ? pdd + 16 * u * PG_M : nullptr, pdw ? pdw + 16 * u : nullptr, true);
+          bs += (a.x + a.y) + (a.z + a.w);
+          bsb += (ab.x + ab.y) + (ab.z + ab.w);
+          const f4 g = a + ab;
+          *(f4*)(S + i * PG_LDT + 4 * q) = g;
+          *(T4*)(D + (4 * q + (i >> 2)) * PG_LDT + 4 * (i & 3)) = rd[u];
+          // (LDS instructions of one wave are carried out in order: the reads below see the writes above)
+          float dv[4], x[3];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) dv[v] = widen1(D[(4 * q + v) * PG_LDT + i]);
+#pragma unroll
+          for (int s = 0; s < 3; ++s) x[s] = S[(4 * s + q) * PG_LDT + i];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) accW = mfma4(g[v], dv[v], accW);
+          if (pdd != nullptr) {  // uniform
+            f4 dd = zero4;
+#pragma unroll
+            for (int s = 0; s < 3; ++s) dd = mfma4(wA[s], x[s], dd);
+            T* dst = pdd + 16 * u * PG_M;
+            if constexpr (BF) {
+              uint2 w;
+              w.x = pack_bf16(dd.x, dd.y);
+              w.y = pack_bf16(dd.z, dd.w);
+              *(uint2*)dst = w;
+            } else {
+              *(f4*)dst = dd;
+            }
+          }
+          if constexpr (HASW) {
+            if (pdw != nullptr) {  // uniform: sum over the rows = over the 16 lanes that share q
+#pragma unroll
+              for (int v = 0; v < 4; ++v) pw[v] = row_sum16_(pw[v]);
+              if (i == 15) *(f4*)(pdw + 16 * u) = pw;
+            }
+          }
         }
         const int step = 16 * UNR;
         pa += ok2 ? step : 0;
         pab += ok2b ? step : 0;
         pd += step * PG_M;
         if (pdd) pdd += step * PG_M;
-#pragma unroll
-        for (int s = 0; s < 3; ++s) {
-          pg[s] += okg[s] ? step : 0;
-          pgb[s] += okgb[s] ? step : 0;
-          if constexpr (HASW) pr1[s] += isdt1[s] ? step : 0;
-        }
         if constexpr (HASW) {
           pr2 += isdt2 ? step : 0;
           pw2 += step;
-          pw1 += step;
           if (pdw) pdw += step;
         }
       }
