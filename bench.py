@@ -468,6 +468,39 @@ def time_pointnet2_ops(torch, reps=5):
     return res
 
 
+def time_serialization(torch, reps=50):
+    """The Hilbert-curve order (models/dest_module.py:307-397) at the detector's sizes: the curve positions alone
+    (`issm_hilbert_codes`, microseconds and bytes moved), the two orders with their sorts and inverse permutations
+    (`Serialization.forward`), and the gather of the key features into curve order.  HIP events around each call."""
+    from dest3d_amd.serialization import Serialization, hilbert_codes
+    torch.manual_seed(0)
+    res = {}
+
+    def t(fn):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(e0.elapsed_time(e1) / reps * 1e3, 2)
+
+    for name, B, N, C_ in (("keys_8x1024", 8, 1024, 288), ("backbone_8x20000", 8, 20000, 256)):
+        pts = (8 * torch.rand(B, N, 3)).cuda()
+        feat = torch.randn(B, N, C_, device="cuda", dtype=torch.bfloat16)
+        ser = Serialization(order=("xyz", "yxz"))
+        ser(pts)
+        r = {"hilbert_codes_us": t(lambda: hilbert_codes(pts, "xyz")),
+             "codes_bytes": B * N * (12 + 8),   # three float coordinates in, one 64-bit position out
+             "two_orders_with_sorts_us": t(lambda: ser(pts)),
+             "gather_features_us": t(lambda: ser.reorder_points(feat, 0)),
+             "gather_bytes": 2 * B * N * C_ * 2 + B * N * 8}
+        res[name] = r
+    return res
+
+
 def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
@@ -530,6 +563,8 @@ def main():
                     help="time BoxDistFun: the kernels against the same formulas in PyTorch ops, and print the JSON line")
     ap.add_argument("--only-pointnet2", action="store_true",
                     help="time only the backbone's point-set operators and print their JSON line (ms per call)")
+    ap.add_argument("--only-serialization", action="store_true",
+                    help="time the Hilbert-curve order (codes, sorts, feature gather) at the detector's sizes")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc)")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
@@ -550,6 +585,9 @@ def main():
         return
     if args.only_pointnet2:
         print(json.dumps({"pointnet2_ops_ms": time_pointnet2_ops(torch)}))
+        return
+    if args.only_serialization:
+        print(json.dumps({"serialization": time_serialization(torch)}))
         return
     if args.only_layer:
         whole, enc = time_box_dist_layer(torch, args.steps, args.warmup)

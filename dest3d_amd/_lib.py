@@ -28,7 +28,7 @@ EXPORTS = [
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
     "issm_dwconv_partial_rows", "issm_dwconv_silu_fwd", "issm_dwconv_silu_bwd",
     "issm_box_dist_bwd_scratch_bytes", "issm_box_dist_fwd", "issm_box_dist_bwd",
-    "issm_hilbert_codes", "issm_transpose_states",
+    "issm_hilbert_codes", "issm_hilbert_order", "issm_transpose_states",
     "issm_pn2_furthest_point_sampling", "issm_pn2_ball_query", "issm_pn2_group_points", "issm_pn2_group_points_grad",
     "issm_pn2_gather_points", "issm_pn2_gather_points_grad", "issm_pn2_three_nn", "issm_pn2_three_interpolate",
     "issm_pn2_three_interpolate_grad", "issm_pn2_group_points_grad_cl", "issm_pn2_three_interpolate_grad_cl",
@@ -146,6 +146,16 @@ class HilbertArgs(C.Structure):
     ]
 
 
+class HilbertOrderArgs(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("npoint", C.c_int32), ("bits", C.c_int32), ("norder", C.c_int32),
+        ("order", (C.c_int32 * 3) * 6), ("cell", C.c_float), ("points", C.c_void_p), ("index", C.c_void_p),
+        ("inverse", C.c_void_p), ("stream", C.c_void_p),
+    ]
+
+
+HILBERT_ORDER_MAX_POINTS = 4096
+
 _lib: Optional[C.CDLL] = None
 
 
@@ -182,6 +192,7 @@ def load() -> C.CDLL:
     lib.issm_box_dist_bwd_scratch_bytes.argtypes = [C.c_int32] * 6
     lib.issm_hilbert_codes.argtypes = [P(HilbertArgs)]
     lib.issm_transpose_states.argtypes = [P(TransposeArgs)]
+    lib.issm_hilbert_order.argtypes = [P(HilbertOrderArgs)]
     i32, f32 = C.c_int32, C.c_float
     lib.issm_pn2_furthest_point_sampling.argtypes = [i32, i32, i32, vp, vp, vp, vp]
     lib.issm_pn2_ball_query.argtypes = [i32, i32, i32, f32, i32, vp, vp, vp, vp]

@@ -60,6 +60,84 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_codes(HilbertP p) {
   p.codes[id] = hilbert3(g[p.perm[0]], g[p.perm[1]], g[p.perm[2]], p.bits);
 }
 
+// The whole serialization of a sample in one workgroup: minimum corner, curve positions, a stable sort of the
+// positions and the inverse permutation (Serialization.forward, models/dest_module.py:319-345, for all its orders in
+// one launch).  Workgroup = (order, sample).  Keys are (position << 12 | point index): unique, so a bitonic network in
+// LDS sorts them stably; up to 4096 points (32 KB of keys).  The separate steps (a reduction, a launch per order, two
+// library sorts per order) took 75 us per order at 1024 points, nearly all of it launches.
+constexpr int HO_MAXN = 4096, HO_IDXBITS = 12;
+__global__ __launch_bounds__(NTHREADS) void k_hilbert_order(HilbertOrderP p) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  unsigned long long* keys = reinterpret_cast<unsigned long long*>(smem_raw);
+  __shared__ float red[3][NTHREADS / 64];
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x % p.B, o = blockIdx.x / p.B;
+  const float* pts = p.points + (long)b * p.N * 3;
+  // minimum corner of the sample (exact: a minimum does not depend on the order it is taken in)
+  float mn[3] = {INFINITY, INFINITY, INFINITY};
+  for (int j = tid; j < p.N; j += NTHREADS) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) mn[i] = fminf(mn[i], pts[3 * j + i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mn[i] = fminf(mn[i], __shfl_xor(mn[i], d, 64));
+    if ((tid & 63) == 0) red[i][tid >> 6] = mn[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    mn[i] = red[i][0];
+#pragma unroll
+    for (int w = 1; w < NTHREADS / 64; ++w) mn[i] = fminf(mn[i], red[i][w]);
+  }
+  const int cap = (1 << p.bits) - 1;
+  const int p0 = p.perm[o][0], p1 = p.perm[o][1], p2 = p.perm[o][2];
+  for (int j = tid; j < p.NP; j += NTHREADS) {
+    unsigned long long key = ~0ull;  // padding sorts last
+    if (j < p.N) {
+      unsigned g[3];
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        const float v = truncf((pts[3 * j + i] - mn[i]) / p.cell);  // the same correctly rounded division as above
+        int c = v >= (float)cap ? cap : (int)v;
+        g[i] = (unsigned)(c < 0 ? 0 : c);
+      }
+      key = ((unsigned long long)hilbert3(g[p0], g[p1], g[p2], p.bits) << HO_IDXBITS) | (unsigned)j;
+    }
+    keys[j] = key;
+  }
+  __syncthreads();
+  // bitonic network: NP / 2 compare-exchanges per step, every step behind a barrier
+  for (int k = 2; k <= p.NP; k <<= 1) {
+    for (int d = k >> 1; d > 0; d >>= 1) {
+      for (int t = tid; t < (p.NP >> 1); t += NTHREADS) {
+        const int lo = ((t & ~(d - 1)) << 1) | (t & (d - 1)), hi = lo | d;
+        const bool up = (lo & k) == 0;
+        const unsigned long long a = keys[lo], c = keys[hi];
+        if ((a > c) == up) {
+          keys[lo] = c;
+          keys[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  long* index = p.index + ((long)o * p.B + b) * p.N;
+  long* inverse = p.inverse ? p.inverse + ((long)o * p.B + b) * p.N : nullptr;
+  for (int j = tid; j < p.N; j += NTHREADS) {
+    const int src = (int)(keys[j] & ((1u << HO_IDXBITS) - 1u));
+    index[j] = src;
+    if (inverse) inverse[src] = j;
+  }
+}
+
+int launch_hilbert_order(const HilbertOrderP& p, hipStream_t st) {
+  hipLaunchKernelGGL(k_hilbert_order, dim3((unsigned)(p.B * p.norder)), dim3(NTHREADS), (size_t)p.NP * 8, st, p);
+  return (int)hipGetLastError();
+}
+
 int launch_hilbert_codes(const HilbertP& p, hipStream_t st) {
   const long n = (long)p.B * p.N;
   hipLaunchKernelGGL(k_hilbert_codes, dim3((unsigned)((n + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st, p);

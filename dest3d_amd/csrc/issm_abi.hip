@@ -28,6 +28,7 @@ int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, co
 int launch_rmsnorm_fwd(const NormP& p, hipStream_t st);
 int launch_rmsnorm_bwd(const NormP& p, hipStream_t st);
 int launch_hilbert_codes(const HilbertP& p, hipStream_t st);
+int launch_hilbert_order(const HilbertOrderP& p, hipStream_t st);
 struct TrP {
   int B, R, C, in_dt, out_dt;
   const void* in0;
@@ -686,6 +687,36 @@ int issm_hilbert_codes(const issm_hilbert_args* a) {
   for (int i = 0; i < 3; ++i) p.perm[i] = a->order[i];
   p.points = a->points; p.mins = a->mins; p.codes = (long*)a->codes;
   return launched(launch_hilbert_codes(p, (hipStream_t)a->stream), "hilbert_codes");
+}
+
+int issm_hilbert_order(const issm_hilbert_order_args* a) {
+  if (!a) return fail(ISSM_E_NULL, "hilbert_order: args is NULL");
+  if (a->batch < 0 || a->npoint < 0) return fail(ISSM_E_SHAPE, "hilbert_order: bad shape");
+  if (a->norder < 1 || a->norder > 6) return fail(ISSM_E_SHAPE, "hilbert_order: norder = %d (1..6)", a->norder);
+  if (a->bits < 1 || a->bits > 17) return fail(ISSM_E_UNSUPPORTED, "hilbert_order: bits = %d (1..17)", a->bits);
+  if (a->npoint > ISSM_HILBERT_ORDER_MAX_POINTS)
+    return fail(ISSM_E_UNSUPPORTED, "hilbert_order: %d points (at most %d per sample; use issm_hilbert_codes and a sort)",
+                a->npoint, ISSM_HILBERT_ORDER_MAX_POINTS);
+  if (!(a->cell > 0.0f)) return fail(ISSM_E_SHAPE, "hilbert_order: cell must be positive");
+  for (int o = 0; o < a->norder; ++o) {
+    int seen = 0;
+    for (int i = 0; i < 3; ++i) {
+      if (a->order[o][i] < 0 || a->order[o][i] > 2) return fail(ISSM_E_SHAPE, "hilbert_order: order[%d][%d] = %d", o, i, a->order[o][i]);
+      seen |= 1 << a->order[o][i];
+    }
+    if (seen != 7) return fail(ISSM_E_SHAPE, "hilbert_order: order %d is not a permutation of 0, 1, 2", o);
+  }
+  if ((int64_t)a->batch * a->npoint == 0) return ISSM_OK;
+  if (!a->points || !a->index) return fail(ISSM_E_NULL, "hilbert_order: points/index is NULL");
+  if ((int64_t)a->batch * a->norder > 0x7fffffff) return fail(ISSM_E_SHAPE, "hilbert_order: too many samples");
+  HilbertOrderP p;
+  p.B = a->batch; p.N = a->npoint; p.bits = a->bits; p.norder = a->norder; p.cell = a->cell;
+  p.NP = 2;
+  while (p.NP < p.N) p.NP <<= 1;
+  for (int o = 0; o < a->norder; ++o)
+    for (int i = 0; i < 3; ++i) p.perm[o][i] = a->order[o][i];
+  p.points = a->points; p.index = (long*)a->index; p.inverse = (long*)a->inverse;
+  return launched(launch_hilbert_order(p, (hipStream_t)a->stream), "hilbert_order");
 }
 
 // shared checks of the point-set operators: non-negative sizes, work present, pointers given

@@ -104,6 +104,16 @@ struct HilbertP {
   long* codes;          // (B, N)
 };
 
+// the whole serialization in one launch (hilbert.hip): index / inverse (norder, B, N), NP = N rounded up to a power of two
+struct HilbertOrderP {
+  int B, N, NP, bits, norder;
+  int perm[6][3];
+  float cell;
+  const float* points;
+  long* index;
+  long* inverse;  // may be null
+};
+
 // parameters of the box-to-point distance encoding kernels (box_dist.hip)
 struct BoxDistP {
   int B, L, K, D, H, W, dtype, nwg, nwg_bwd;

@@ -43,6 +43,30 @@ def hilbert_codes(points: torch.Tensor, order: str = "xyz", bit: int = 9, cell: 
     return codes
 
 
+def hilbert_order(points: torch.Tensor, orders: Sequence[str] = ("xyz",), bit: int = 9, cell: float = 1.0 / 50.0):
+    """points (B, N, 3), N <= 4096 -> (index, inverse), both (len(orders), B, N) int64: index[o, b] lists the points
+    of sample b along the curve of order o (equal to a stable argsort of ``hilbert_codes``), inverse[o, b] is its
+    inverse permutation.  One kernel launch (libissm_hip.so: issm_hilbert_order)."""
+    for o in orders:
+        if o not in ORDERS:
+            raise NotImplementedError(o)
+    L.require_gpu(points, "points")
+    lib = L.load()
+    p = points.detach().float().contiguous()
+    with torch.cuda.device(p.device):
+        out = torch.empty(2, len(orders), p.shape[0], p.shape[1], dtype=torch.int64, device=p.device)
+        a = L.HilbertOrderArgs()
+        a.batch, a.npoint, a.bits, a.norder = p.shape[0], p.shape[1], bit, len(orders)
+        for j, o in enumerate(orders):
+            for i, v in enumerate(ORDERS[o]):
+                a.order[j][i] = v
+        a.cell = cell
+        a.points, a.index, a.inverse = p.data_ptr(), out[0].data_ptr(), out[1].data_ptr()
+        a.stream = L.current_stream_ptr(p.device)
+        L.check(lib.issm_hilbert_order(C.byref(a)), "issm_hilbert_order")
+    return out[0], out[1]
+
+
 class Serialization(nn.Module):
     def __init__(self, order: Sequence[str] = ("xyz", "yxz"), bit: int = 9):
         super().__init__()
@@ -57,6 +81,12 @@ class Serialization(nn.Module):
         """points (B, N, 3): fills ``index_list`` (per order, the indices that sort the points along the curve) and
         ``reversed_index_list`` (their inverses)   (dest_module.py:319-345)."""
         self.index_list, self.reversed_index_list = [], []
+        if (points.is_cuda and 0 < points.shape[1] <= L.HILBERT_ORDER_MAX_POINTS and self.bit <= 17
+                and len(self.order) <= 6):
+            # minimum corner, curve positions, stable sort and inverse permutation of every order in one launch
+            idx, inv = hilbert_order(points, self.order, self.bit)
+            self.index_list, self.reversed_index_list = list(idx.unbind(0)), list(inv.unbind(0))
+            return
         for o in self.order:
             code = hilbert_codes(points, o, self.bit)
             idx = torch.argsort(code, dim=-1, stable=True)

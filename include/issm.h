@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define ISSM_ABI_VERSION 3
+#define ISSM_ABI_VERSION 4
 #define ISSM_CHUNK 64 /* tokens per internal chunk */
 
 typedef enum issm_status {
@@ -442,6 +442,26 @@ typedef struct issm_hilbert_args {
 } issm_hilbert_args;
 
 int issm_hilbert_codes(const issm_hilbert_args* args);
+
+/* Serialization.forward as a whole (models/dest_module.py:319-345), all orders in one launch: for every order o and
+ * sample b, index[o][b][:] lists the points of the sample along the curve (what torch.argsort of the codes above
+ * returns; points of one cell keep their input order) and inverse[o][b][:] is the inverse permutation (the
+ * reference's second argsort).  The minimum corner is taken inside.  points (B, N, 3) fp32 contiguous; index,
+ * inverse (norder, B, N) int64 contiguous, inverse may be NULL.  N <= ISSM_HILBERT_ORDER_MAX_POINTS and bits <= 17
+ * (ISSM_E_UNSUPPORTED beyond: take issm_hilbert_codes and a library sort). */
+#define ISSM_HILBERT_ORDER_MAX_POINTS 4096
+typedef struct issm_hilbert_order_args {
+  int32_t batch, npoint, bits;
+  int32_t norder; /* 1..6 */
+  int32_t order[6][3];
+  float cell;
+  const float* points;
+  int64_t* index;
+  int64_t* inverse;
+  void* stream;
+} issm_hilbert_order_args;
+
+int issm_hilbert_order(const issm_hilbert_order_args* args);
 
 /* ---- point-set operators of the PointNet++ backbone ---------------------------------------
  * The functions of the reference's `pointnet2._ext` (pointnet2/_ext_src/src/bindings.cpp:8-24), same argument

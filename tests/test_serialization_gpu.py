@@ -85,3 +85,49 @@ def test_rejects_bad_arguments():
     assert lib.issm_hilbert_codes(C.byref(a)) == -2
     a.order[2] = 2
     assert lib.issm_hilbert_codes(C.byref(a)) == -1
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 300, 1000, 1024, 1025, 4096])
+def test_one_launch_order_equals_codes_and_stable_sorts(n):
+    """issm_hilbert_order (minimum corner, positions, stable sort, inverse permutation of every order in one launch)
+    against the separate steps: issm_hilbert_codes and torch's stable argsort, twice.  Many points share a cell (a
+    coarse second half), so the order inside ties is tested too."""
+    from dest3d_amd.serialization import ORDERS, hilbert_codes, hilbert_order
+    print(f"[case] hilbert order n={n}", flush=True)
+    g = torch.Generator().manual_seed(40 + n)
+    pts = 8 * torch.rand(3, n, 3, generator=g)
+    pts[:, n // 2:] = torch.round(pts[:, n // 2:] * 2) / 2      # a 0.5 m lattice: dozens of points per 2 cm cell
+    pts[1, 0] = -3.0                                             # every sample has its own minimum corner
+    pts = pts.cuda()
+    orders = list(ORDERS)
+    idx, inv = hilbert_order(pts, orders, 9)
+    assert idx.shape == inv.shape == (6, 3, n) and idx.dtype == torch.int64
+    for j, o in enumerate(orders):
+        want = torch.argsort(hilbert_codes(pts, o, 9), dim=-1, stable=True)
+        assert torch.equal(idx[j], want), o
+        assert torch.equal(inv[j], torch.argsort(want, dim=-1)), o
+
+
+def test_order_rejects_what_it_does_not_hold():
+    import ctypes as C
+    from dest3d_amd import _lib as L
+    from dest3d_amd.serialization import Serialization
+    lib = L.load()
+    a = L.HilbertOrderArgs()
+    a.batch, a.npoint, a.bits, a.norder, a.cell = 1, 5000, 9, 1, 0.02
+    for i in range(3):
+        a.order[0][i] = i
+    assert lib.issm_hilbert_order(C.byref(a)) == -5 and b"4096" in lib.issm_last_error()
+    a.npoint, a.bits = 100, 18
+    assert lib.issm_hilbert_order(C.byref(a)) == -5
+    a.bits, a.norder = 9, 7
+    assert lib.issm_hilbert_order(C.byref(a)) == -2
+    a.norder = 1
+    assert lib.issm_hilbert_order(C.byref(a)) == -1            # no pointers
+    # the module falls back to codes + library sorts above the limit, with the same result as the oracle
+    torch.manual_seed(1)
+    pts = (8 * torch.rand(1, 5000, 3)).cuda()
+    s = Serialization(order=["zyx"], bit=9)
+    s(pts)
+    _, idx, inv = R.serialize(pts.cpu().numpy(), "zyx", 9)
+    assert (s.index_list[0].cpu().numpy() == idx).all() and (s.reversed_index_list[0].cpu().numpy() == inv).all()
