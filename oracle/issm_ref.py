@@ -53,6 +53,15 @@ def softplus_ref(x: torch.Tensor) -> torch.Tensor:
     return torch.where(x <= 20.0, torch.log1p(torch.exp(torch.clamp(x, max=20.0))), x)
 
 
+def limits_as_fp32(dt_limit):
+    """The reference's kernels take dt_min / dt_max as fp32 scalars (issm_chunk_state.py:55, 98, 210-211; a Python float argument is an fp32 scalar there): the clamp and its
+    backward mask compare against the limits *rounded to fp32*, whatever precision the rest is evaluated in.  A dt
+    that an fp32 caller has already clamped to, say, 0.02 sits exactly on that rounded limit and keeps its gradient;
+    against the unrounded 0.02 it would lie just below and lose it."""
+    import numpy as np
+    return float(np.float32(dt_limit[0])), float(np.float32(dt_limit[1]))
+
+
 def dt_transform(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, INF)):
     """dt' = clamp(softplus?(dt + dt_bias), lo, hi)  (issm_chunk_state.py:84-99).
 
@@ -63,7 +72,7 @@ def dt_transform(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, INF)):
         dt = dt + dt_bias.to(dt.dtype)[None, None]
     if dt_softplus:
         dt = softplus_ref(dt)
-    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    lo, hi = limits_as_fp32(dt_limit)
     return torch.clamp(dt, min=lo, max=hi)
 
 
@@ -217,7 +226,7 @@ def issm_bwd_closed_form(x, dt, A, B, C, chunk, dy, dfinal=None, D=None, dt_bias
     x_, dt_, A_, B_, C_, dy_ = map(f, (x, dt, A, B, C, dy))
     pre = dt_ if dt_bias is None else dt_ + f(dt_bias)[None, None]
     sp = softplus_ref(pre) if dt_softplus else pre
-    lo, hi = float(dt_limit[0]), float(dt_limit[1])
+    lo, hi = limits_as_fp32(dt_limit)
     dtp = torch.clamp(sp, lo, hi)
 
     def pad(t):

@@ -55,7 +55,7 @@ def scan_case(Bsz, L, H, P, N, G, seed, softplus, gate, cuts=None):
     if seq is not None:
         out["seq_idx"] = seq.numpy()
     out.update(dy=dy.numpy(), dfinal=dfinal.numpy(), y=y.detach().numpy(), final=fin.detach().numpy(),
-               softplus=np.array(softplus), dt_limit=np.array(limit))
+               softplus=np.array(softplus), dt_limit=np.array(R.limits_as_fp32(limit)))
     out.update({"grad_" + k: v.grad.numpy() for k, v in leaf.items()})
     return out
 

@@ -206,6 +206,25 @@ def test_packed_sequences_match_oracle(dtype):
             _check("d" + k, g[k].grad, ins[k].grad, bt)
 
 
+def test_dt_already_clamped_by_an_fp32_caller_keeps_its_gradient():
+    """dt = clamp(x, 0.02, 0.3) computed in fp32 and passed with dt_limit = (0.02, 0.3): a third of the entries sit
+    exactly on float32(0.02) or float32(0.3).  They are not *outside* the limits, so their gradient passes, in the
+    kernels (fp32 compare, as in the reference) and in the oracle (limits rounded to fp32)."""
+    _say("dt on the clamp limits")
+    d = _problem(2, 100, 2, 16, 64, 1, seed=31, softplus=False)
+    d["dt"] = torch.clamp(torch.rand(2, 100, 2, 64, generator=torch.Generator().manual_seed(5)) * 0.45 - 0.05, 0.02, 0.3)
+    d["dt_limit"] = (0.02, 0.3)
+    on_limit = ((d["dt"] == d["dt"].min()) | (d["dt"] == d["dt"].max())).float().mean().item()
+    assert on_limit > 0.3
+    y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+    assert (g_ref["dt"][d["dt"] == d["dt"].min()] != 0).any()
+    y, fin, g, _ = _run_operator(d, torch.float32)
+    _check("out", y, y_ref, FWD32)
+    for k in GRAD_NAMES:
+        if d[k] is not None:
+            _check("d" + k, g[k], g_ref[k], BWD32)
+
+
 def test_packed_sequences_randomised():
     """Seeded draws of shapes, options and change points (up to five per batch row, anywhere, repeats allowed) in fp32
     and bf16 against the oracle's recurrence with resets."""

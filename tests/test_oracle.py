@@ -334,3 +334,21 @@ def test_bench_generator_draws_the_same_problem_as_the_tests_generator():
     b = bench.synthetic_inputs(torch, 2, 24, 3, 4, 8, G=1, seed=1235, h0_std=0.1)
     for k in b:
         assert torch.equal(a[k], b[k]), k
+
+
+def test_clamp_limits_are_the_fp32_roundings_the_kernels_receive():
+    """A dt that an fp32 caller clamped to 0.02 equals float32(0.02) = 0.0199999995529...: it sits on the limit the
+    reference's kernels compare with (their dt_min is an fp32 scalar) and keeps its gradient; against the double 0.02
+    it would count as clamped.  One element below and one above for contrast."""
+    import numpy as np
+    lim = float(np.float32(0.02))
+    dt = torch.tensor([lim, float(np.nextafter(np.float32(0.02), np.float32(0))), 0.05], dtype=torch.float64).reshape(1, 3, 1, 1)
+    dt.requires_grad_()
+    out = R.dt_transform(dt, None, False, (0.02, 0.3))
+    out.sum().backward()
+    assert out.flatten().tolist() == [lim, lim, 0.05]
+    assert dt.grad.flatten().tolist() == [1.0, 0.0, 1.0]
+    x = torch.randn(1, 3, 1, 2, dtype=torch.float64)
+    A, B, C = -torch.ones(1, 1, dtype=torch.float64), torch.ones(1, 3, 1, 1, dtype=torch.float64), torch.ones(1, 3, 1, 1, dtype=torch.float64)
+    g = R.issm_bwd_closed_form(x, dt.detach(), A, B, C, 4, torch.ones_like(x), dt_limit=(0.02, 0.3))
+    assert g["ddt"].flatten()[0] != 0 and g["ddt"].flatten()[1] == 0
