@@ -1553,6 +1553,7 @@ __device__ __forceinline__ void colsum_block(const float* __restrict__ src, int 
   float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   if (c < ncols) {
     int j = g;
+#pragma unroll 2
     for (; j + 24 < J; j += 32) {
       a0 += src[(long)j * ncols + c];
       a1 += src[(long)(j + 8) * ncols + c];
@@ -1574,9 +1575,38 @@ __device__ __forceinline__ void colsum_block(const float* __restrict__ src, int 
 // dD[h] = sum over units and p of partD[(j*H + h)*P + p]: one block per head.
 __device__ __forceinline__ void dd_scalar_block(const float* __restrict__ partD, int J, int H, int P,
                                                 float* __restrict__ dD, int h, float* red) {
-  float a = 0.0f;
-  for (int e = threadIdx.x; e < J * P; e += NTHREADS) a += partD[((long)(e / P) * H + h) * P + (e % P)];
-  red[threadIdx.x] = a;
+  // element e = j P + p of the head's (J, P) slab; a thread takes e = tid, tid + 256, ...: (j, p) advance without a
+  // division, and four elements are requested before any is added (with 8 blocks in the launch the latency of a
+  // load is the run time: one element per trip made this the longest block of the kernel)
+  const int dj = NTHREADS / P, dp = NTHREADS % P;
+  int jj = (int)threadIdx.x / P, pp = (int)threadIdx.x % P;
+  const long row = (long)H * P;
+  const float* src = partD + (long)h * P;
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  auto next = [&](int& j_, int& p_) {
+    p_ += dp;
+    j_ += dj + (p_ >= P ? 1 : 0);
+    p_ -= p_ >= P ? P : 0;
+  };
+  while (jj < J) {
+    int j1 = jj, p1 = pp;
+    next(j1, p1);
+    int j2 = j1, p2 = p1;
+    next(j2, p2);
+    int j3 = j2, p3 = p2;
+    next(j3, p3);
+    const float v0 = src[jj * row + pp];   // (rows past the end read row 0 and add nothing: no branch around a load)
+    const float v1 = src[(j1 < J ? j1 : 0) * row + p1];
+    const float v2 = src[(j2 < J ? j2 : 0) * row + p2];
+    const float v3 = src[(j3 < J ? j3 : 0) * row + p3];
+    a0 += v0;
+    a1 += j1 < J ? v1 : 0.0f;
+    a2 += j2 < J ? v2 : 0.0f;
+    a3 += j3 < J ? v3 : 0.0f;
+    jj = j3; pp = p3;
+    next(jj, pp);
+  }
+  red[threadIdx.x] = (a0 + a1) + (a2 + a3);
   __syncthreads();
   for (int o = NTHREADS / 2; o > 0; o >>= 1) {
     if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
