@@ -250,11 +250,6 @@ __device__ __forceinline__ void pin16(float (&a)[16]) {
                "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
 }
 __device__ __forceinline__ void pin4(f4& a) { asm volatile("" : "+v"(a)); }
-// first and last row of each of the lane's four groups (what is left of a running sum once the in-group decays exist)
-__device__ __forceinline__ void pin_group_ends(float (&a)[16]) {
-  asm volatile("" : "+v"(a[0]), "+v"(a[3]), "+v"(a[4]), "+v"(a[7]), "+v"(a[8]), "+v"(a[11]), "+v"(a[12]), "+v"(a[15]));
-}
-
 // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of logical
 // ids so that units sharing B/C tiles (the heads of one chunk) share an L2.
 __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
