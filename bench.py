@@ -39,8 +39,15 @@ SHAPE = dict(B=8, L=1024, H=8, P=32, N=256, G=1, cs=64)
 
 # The scan workloads this script can time: the headline (configs[1], fp32), its variants, and the baseline's other scan
 # configurations (configs[3]: long sequence; configs[4]: large state).  shape overrides SHAPE.
+# Unless a workload says `presoftplus`, dt is handed over raw with dt_softplus=True and a (H, N) dt_bias of zeros: bias,
+# softplus and clamp run inside the kernels (issm_chunk_state.py:84-99).  `presoftplus` is the module's call pattern
+# (models/dest_module.py:600-611): dt = softplus(dt_raw) computed by the caller, dt_softplus=False, no bias.
+# `fwd_only` times the forward alone (configs[0], the reference's own forward-only harness test_issm.py:113-135).
+# Every workload runs with the library's internal chunk of 64 tokens, whatever chunk_size the configuration names.
 WORKLOADS = {
     "headline": dict(shape={}, ndir=2, dtype="float32"),
+    "headline_module_call_pattern": dict(shape={}, ndir=2, dtype="float32", presoftplus=True),
+    "config0_gpu_forward_only_B2": dict(shape=dict(B=2), ndir=1, dtype="float32", fwd_only=True),
     "uni_fp32": dict(shape={}, ndir=1, dtype="float32"),
     "uni_bf16": dict(shape={}, ndir=1, dtype="bfloat16"),
     "bidir_bf16": dict(shape={}, ndir=2, dtype="bfloat16"),
@@ -71,7 +78,7 @@ def synthetic_inputs(torch, Bsz, L, H, P, N, G=1, seed=1234, h0_std=0.0):
     return dict(x=x, dt_raw=dt_raw, A=A, B=Bm, C=Cm, D=D, h0=h0, dy=dy, dfinal=dfinal)
 
 
-def make_problem(torch, shape, ndir, dtype, seed=1235, h0_std=0.0):
+def make_problem(torch, shape, ndir, dtype, seed=1235, h0_std=0.0, presoftplus=False):
     SHAPE = shape
     I = synthetic_inputs(torch, SHAPE["B"], SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=seed,
                          h0_std=h0_std)
@@ -85,7 +92,12 @@ def make_problem(torch, shape, ndir, dtype, seed=1235, h0_std=0.0):
         t["dy"].append(torch.randn(I["x"].shape, generator=g))
         t["dfinal"].append(torch.randn(I["dfinal"].shape, generator=g))
     out = {k: [v.to(dev, dtype if k in ("x", "B", "C", "dy") else torch.float32) for v in vs] for k, vs in t.items()}
-    out["dt"] = torch.nn.functional.softplus(I["dt_raw"]).to(dev, dtype)   # module call pattern: dt already softplus'ed
+    if presoftplus:   # module call pattern: dt already softplus'ed by the caller
+        out["dt"] = torch.nn.functional.softplus(I["dt_raw"]).to(dev, dtype)
+        out["dt_bias"] = None
+    else:             # the kernels apply bias -> softplus -> clamp
+        out["dt"] = I["dt_raw"].to(dev, dtype)
+        out["dt_bias"] = torch.zeros(SHAPE["H"], SHAPE["N"], device=dev)
     out["A"] = I["A"].to(dev)
     out["D"] = I["D"].to(dev)
     out["h0"] = I["h0"].to(dev)
@@ -96,16 +108,17 @@ class Runner:
     """Forward + backward through the C ABI with preallocated buffers (no autograd, no allocation
     in the timed region): exactly the kernels ISSMChunkScanCombinedFn launches."""
 
-    def __init__(self, torch, ndir, dtype, shape=None, h0_std=0.0):
+    def __init__(self, torch, ndir, dtype, shape=None, h0_std=0.0, presoftplus=False, fwd_only=False):
         from dest3d_amd import _lib as L
         from dest3d_amd.issm_combined import _Problem
         self.torch, self.L, self.lib = torch, L, L.load()
         self.ndir = ndir
         SHAPE = self.shape = dict(globals()["SHAPE"], **(shape or {}))
         self.elt = 2 if dtype == torch.bfloat16 else 4
-        t = self.t = make_problem(torch, SHAPE, ndir, dtype, h0_std=h0_std)
-        self.prob = _Problem(t["x"], t["dt"], t["A"], t["B"], t["C"], SHAPE["cs"], t["D"], [None] * ndir, None,
-                             t["h0"], None, False, (0.0, float("inf")))
+        self.fwd_only = fwd_only
+        t = self.t = make_problem(torch, SHAPE, ndir, dtype, h0_std=h0_std, presoftplus=presoftplus)
+        self.prob = _Problem(t["x"], t["dt"], t["A"], t["B"], t["C"], SHAPE["cs"], t["D"], [None] * ndir, t["dt_bias"],
+                             t["h0"], None, not presoftplus, (0.0, float("inf")))
         a = self.a = self.prob.args()
         dev = "cuda"
         B_, L_, H, P, N, G = (SHAPE[k] for k in ("B", "L", "H", "P", "N", "G"))
@@ -117,6 +130,7 @@ class Runner:
         self.dC = [e(B_, L_, G, N, dt=dtype) for _ in range(ndir)]
         self.ddt = e(B_, L_, H, N, dt=dtype)
         self.dA, self.dD, self.dh0 = e(H, N), e(H), e(B_, H, P, N)
+        self.dbias = e(H, N) if t["dt_bias"] is not None else None
         self.ws = self.prob.workspace(a, bwd=False)
         self.bws = self.prob.workspace(a, bwd=True)
         for i in range(ndir):
@@ -127,6 +141,7 @@ class Runner:
             a.dx[i], a.dB[i], a.dC[i] = (L.tensor_desc(v[i]) for v in (self.dx, self.dB, self.dC))
         a.ddt = L.tensor_desc(self.ddt)
         a.dA, a.dD, a.dh0 = self.dA.data_ptr(), self.dD.data_ptr(), self.dh0.data_ptr()
+        a.ddt_bias = L.ptr(self.dbias)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
         a.saved = self.ws.data_ptr()
         a.bwd_workspace, a.bwd_workspace_bytes = self.bws.data_ptr(), self.bws.numel()
@@ -134,7 +149,8 @@ class Runner:
 
     def step(self):
         self.L.check(self.lib.issm_scan_fwd(C.byref(self.a)), "fwd")
-        self.L.check(self.lib.issm_scan_bwd(C.byref(self.a)), "bwd")
+        if not self.fwd_only:
+            self.L.check(self.lib.issm_scan_bwd(C.byref(self.a)), "bwd")
 
     def time_steps(self, steps, warmup):
         torch = self.torch
@@ -322,33 +338,47 @@ def workload_report(run, step_us, reps=20):
 
 
 def cpu_baseline(torch):
-    """Chunked pure-PyTorch formulation (oracle.issm_scan_chunked, fp32, autograd backward) on
-    the host cores, on a bounded sample: 2 of the 8 batch elements, one direction, 2 repetitions
-    (about 15-30 s); scaled by 8 (= 4 x batch, 2 x directions) to the workload's unit."""
+    """Chunked pure-PyTorch formulation (oracle.issm_scan_chunked after oracle.dt_transform, fp32, autograd backward)
+    on the host cores, on a bounded sample: 2 of the 8 batch elements, one direction, 2 repetitions (about 15-30 s);
+    scaled by 8 (= 4 x batch, 2 x directions) to the workload's unit.  Threads: the host share of one GPU on the
+    measurement machines is 16 cores (OMP_NUM_THREADS there), so that many are used even where os.cpu_count() reports
+    the whole machine; both numbers are in the record."""
     from oracle import issm_ref as R
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    host = os.cpu_count() or 1
+    try:
+        host = min(host, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    cores = min(host, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or host)
     torch.set_num_threads(cores)
     I = R.make_inputs(2, SHAPE["L"], SHAPE["H"], SHAPE["P"], SHAPE["N"], SHAPE["G"], seed=1235)
-    ins = [I["x"].clone().requires_grad_(), torch.nn.functional.softplus(I["dt_raw"]).requires_grad_(),
+    bias = torch.zeros(SHAPE["H"], SHAPE["N"])
+    ins = [I["x"].clone().requires_grad_(), I["dt_raw"].clone().requires_grad_(),
            I["A"].clone().requires_grad_(), I["B"].clone().requires_grad_(), I["C"].clone().requires_grad_()]
+
+    def fwd(x, dt_raw, A, B, C_):
+        return R.issm_scan_chunked(x, R.dt_transform(dt_raw, bias, True), A, B, C_, SHAPE["cs"])
+
     best = float("inf")
     for _ in range(2):
         for t in ins:
             t.grad = None
         t0 = time.perf_counter()
-        y, fin = R.issm_scan_chunked(*ins, SHAPE["cs"])
+        y, fin = fwd(*ins)
         ((y * I["dy"]).sum() + (fin * I["dfinal"]).sum()).backward()
         best = min(best, time.perf_counter() - t0)
     # configs[0] as BASELINE.json states it: forward only, B=2, the same formulation, no gradient bookkeeping
     with torch.no_grad():
-        fwd = float("inf")
+        f = float("inf")
         for _ in range(2):
             t0 = time.perf_counter()
-            R.issm_scan_chunked(*[t.detach() for t in ins], SHAPE["cs"])
-            fwd = min(fwd, time.perf_counter() - t0)
-    return {"value": best * 8 * 1e6, "unit": "us/call", "cores": cores, "kind": "port",
-            "sample": "B=2 of 8, one direction, fwd+bwd, fp32, best of 2; scaled x8 to B=8 bidirectional",
-            "config0_forward_only_B2_us": round(fwd * 1e6, 1)}
+            fwd(*[t.detach() for t in ins])
+            f = min(f, time.perf_counter() - t0)
+    return {"value": best * 8 * 1e6, "unit": "us/call", "cores": cores, "host_cpu_count": os.cpu_count(),
+            "kind": "port",
+            "sample": "B=2 of 8, one direction, fwd+bwd incl. bias/softplus/clamp of dt, fp32, best of 2; scaled x8 to "
+                      "B=8 bidirectional",
+            "config0_forward_only_B2_us": round(f * 1e6, 1)}
 
 
 def time_box_dist_layer(torch, steps=10, warmup=3):
@@ -501,6 +531,75 @@ def time_serialization(torch, reps=50):
     return res
 
 
+def layer_compulsory_bytes(nlayers=1, with_encoding=False, B=8, L=1024, K=256, d_model=288, d_dist=16, elt=2):
+    """Compulsory HBM bytes of a forward + backward step through `nlayers` MultiHeadISSMScan layers at the configs[2]
+    shape if nothing but the layer's own inputs, outputs and their gradients crossed HBM (dt, B, C and every scan
+    intermediate staying on chip): per layer and pass, the distance encoding `dist` (B, L, K, 16) and the locality
+    weights (B, L, K) fp32 are read once, key (B, L, d) and query (B, K, d) features are read and written once; the
+    backward also reads the two output gradients, writes the two input gradients and writes d(dist).  With the
+    encoding: BoxDistFun writes `dist` and the weights once and its backward reads the summed d(dist) once (positions
+    and the table are negligible)."""
+    e_dist, e_w = B * L * K * d_dist * elt, B * L * K * 4
+    e_feat = (B * L + B * K) * d_model * elt
+    fwd = e_dist + e_w + 2 * e_feat
+    bwd = e_dist + e_w + 2 * e_feat + 2 * e_feat + e_dist
+    total = nlayers * (fwd + bwd)
+    if with_encoding:
+        total += e_dist + e_w + e_dist
+    return total
+
+
+def time_layer_stack(torch, steps=5, warmup=2, nlayers=6):
+    """configs[2] as a whole: BoxDistFun + local_weight once, then `nlayers` MultiHeadISSMScan layers as a residual
+    stack (models/dest_detector.py:207-235 calls the decoder layers on one shared encoding), bf16, forward + backward
+    from a scalar loss, eager; microseconds per step."""
+    from dest3d_amd.box_dist import BoxDistFun
+    from dest3d_amd.scan_module import MultiHeadISSMScan
+    torch.manual_seed(0)
+    bd = BoxDistFun(out_dim=16).cuda().bfloat16()
+    stack = torch.nn.ModuleList(MultiHeadISSMScan(d_model=288, d_state=256, d_dist=16, chunk_size=256, nheads=8,
+                                                  expand=1) for _ in range(nlayers)).cuda().bfloat16()
+    key = torch.randn(8, 1024, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    query = torch.randn(8, 256, 288, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    key_pos = 8.0 * torch.rand(8, 1024, 3, device="cuda")
+    query_pos = torch.cat([8.0 * torch.rand(8, 256, 3, device="cuda"), 0.2 + 2.0 * torch.rand(8, 256, 3, device="cuda")], -1)
+    zero_angle = torch.zeros(8, 256, device="cuda")
+    g_key, g_query = torch.randn_like(key) / 64, torch.randn_like(query) / 64
+
+    def step():
+        for mod in (stack, bd):
+            mod.zero_grad(set_to_none=True)
+        key.grad = query.grad = None
+        dist, weights = bd(key_pos, query_pos[..., :3], query_pos[..., 3:], zero_angle, weight_query_pos=query_pos)
+        hk, hq = key, query
+        for layer in stack:
+            ok, oq = layer(hk, hq, dist, key_pos, weights)
+            hk, hq = hk + ok, hq + oq
+        torch.autograd.backward((hk, hq), (g_key, g_query))
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e6
+
+
+def caller_rooflines(variants):
+    """The caller-side timings against the HBM time of their compulsory bytes (layer_compulsory_bytes)."""
+    rows = {"detector_layer_bf16_fwd_bwd": (1, False), "detector_layer_bf16_fwd_bwd_as_hip_graph": (1, False),
+            "box_dist_plus_layer_bf16_fwd_bwd": (1, True), "detector_six_layers_plus_box_dist_bf16_fwd_bwd": (6, True)}
+    out = {}
+    for k, (nl, enc) in rows.items():
+        if k in variants:
+            nb = layer_compulsory_bytes(nl, enc)
+            out[k] = {"us": variants[k], "compulsory_mb": round(nb / 1e6, 1), "bound": "hbm",
+                      "frac": round(nb / (variants[k] * 1e-6) / (PEAK_HBM_GBS * 1e9), 4)}
+    return out
+
+
 def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
@@ -548,6 +647,25 @@ def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
         step()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps * 1e6
+
+
+def make_runner(torch, name):
+    spec = WORKLOADS[name]
+    return Runner(torch, spec["ndir"], getattr(torch, spec["dtype"]), spec["shape"], spec.get("h0_std", 0.0),
+                  presoftplus=spec.get("presoftplus", False), fwd_only=spec.get("fwd_only", False))
+
+
+def workload_text(name):
+    """What a workload runs, in words (the `config.workload` of its JSON line)."""
+    spec = WORKLOADS[name]
+    sh = dict(SHAPE, **spec["shape"])
+    return ("B={B} L={L} H={H} P={P} N={N} G={G}".format(**sh) + ", "
+            + ("forward only" if spec.get("fwd_only") else "fwd+bwd") + ", "
+            + ("bidirectional pair (fused)" if spec["ndir"] == 2 else "one direction") + ", "
+            + ("fp32 I/O" if spec["dtype"] == "float32" else "bf16 I/O, fp32 states and accumulation") + ", "
+            + ("dt pre-softplused by the caller (dt_softplus=False, no dt_bias)" if spec.get("presoftplus")
+               else "dt_softplus=True (in-kernel), dt_bias (H,N) zeros, dt_limit (0, inf)")
+            + ", internal chunk 64" + (", h0 ~ N(0, %g)" % spec["h0_std"] if spec.get("h0_std") else ", h0 = 0"))
 
 
 def main():
@@ -605,13 +723,13 @@ def main():
         torch.cuda.synchronize()
     if args.workload:
         # one workload's step loop only (what the profiles under profiles/ are taken from)
-        spec = WORKLOADS[args.workload]
-        r = Runner(torch, spec["ndir"], getattr(torch, spec["dtype"]), spec["shape"], spec.get("h0_std", 0.0))
+        r = make_runner(torch, args.workload)
         us = r.time_steps(args.steps, args.warmup)
-        print(json.dumps({"workload": args.workload, "us_per_step": round(us, 2), "steps": args.steps,
-                          "warmup": args.warmup, **({} if args.no_variants else workload_report(r, us))}))
+        rep = {} if (args.no_variants or r.fwd_only) else workload_report(r, us)
+        print(json.dumps({"workload": args.workload, "config": {"workload": workload_text(args.workload)},
+                          "us_per_step": round(us, 2), "steps": args.steps, "warmup": args.warmup, **rep}))
         return
-    run = Runner(torch, 2, torch.float32)
+    run = make_runner(torch, "headline")
     us = run.time_steps(args.steps, args.warmup)
     pct = run.step_percentiles(max(args.steps, 20))
     rep = workload_report(run, us)
@@ -630,10 +748,11 @@ def main():
             if name == "headline":
                 continue
             big = bool(spec["shape"].get("L", 0) > 4096 or spec["shape"].get("N", 0) > 256)
-            r = Runner(torch, spec["ndir"], getattr(torch, spec["dtype"]), spec["shape"], spec.get("h0_std", 0.0))
+            r = make_runner(torch, name)
             v = r.time_steps(5 if big else max(args.steps // 2, 5), 2 if big else 5)
             variants[name] = round(v, 2)
-            if name in ("bidir_bf16", "long_sequence_B2_L16384_uni_bf16", "large_state_B16_L2048_H16_P64_N512_bidir_fp32"):
+            if name in ("headline_module_call_pattern", "bidir_bf16", "long_sequence_B2_L16384_uni_bf16",
+                        "large_state_B16_L2048_H16_P64_N512_bidir_fp32"):
                 variant_rooflines[name] = workload_report(r, v, reps=5 if big else 20)
             del r
             torch.cuda.empty_cache()
@@ -641,12 +760,13 @@ def main():
         variants["detector_layer_bf16_fwd_bwd_as_hip_graph"] = round(time_module_layer(torch, as_graph=True), 2)
         variants["detector_layer_fp32_fwd_bwd"] = round(time_module_layer(torch, dtype=torch.float32), 2)
         variants["box_dist_plus_layer_bf16_fwd_bwd"] = round(time_box_dist_layer(torch)[0], 2)
+        variants["detector_six_layers_plus_box_dist_bf16_fwd_bwd"] = round(time_layer_stack(torch), 2)
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[1]: B=8 L=1024 H=8 P=32 N=256 G=1 chunk=64, fwd+bwd, bidirectional pair "
-                               "(fused), fp32 I/O, fp32 MFMA accumulate"},
+        "config": {"workload": "configs[1]: " + workload_text("headline"),
+                   "variants": {k: workload_text(k) for k in WORKLOADS if k != "headline"}},
         "roofline": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in roof.items()},
         "step_us_percentiles": pct,
         "stages_us": stages,
@@ -654,6 +774,7 @@ def main():
         "step_roofline": rep["step_roofline"],
         "variants_us": variants,
         "variant_rooflines": variant_rooflines,
+        "caller_rooflines": caller_rooflines(variants),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch)
