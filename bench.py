@@ -219,6 +219,7 @@ class Runner:
         st, csl, cabt = f(Bt, nc + 1, H, P, N), f(Bt, nc, H, N), f(Bt, nc, H, 64, 64)
         dst, dm, gn, dh0d = f(Bt, nc, H, P, N), f(Bt, nc, H, 64, 64), f(Bt, nc, H, N), f(nd, B_, H, P, N)
         pa, pb, pd = f(Bt * nc, H, N), f(Bt * nc, H, N), f(Bt * nc * H, P)
+        redo = torch.zeros(lib.issm_bwd_chunk_redo_ints(C.byref(a)), dtype=torch.int32, device="cuda")
         p = lambda t: t.data_ptr()
         stages = [
             ("chunk_local", lambda: lib.issm_stage_chunk_local(C.byref(a), p(st), p(csl), p(cabt))),
@@ -226,7 +227,7 @@ class Runner:
             ("chunk_scan", lambda: lib.issm_stage_chunk_scan(C.byref(a), p(st), p(cabt), None)),
             ("bwd_dstates", lambda: lib.issm_stage_bwd_dstates(C.byref(a), None, p(dst), p(dm))),
             ("state_passing_bwd", lambda: lib.issm_stage_state_passing_bwd(C.byref(a), p(st), p(csl), p(dst), p(gn), p(dh0d))),
-            ("bwd_chunk", lambda: [lib.issm_stage_bwd_chunk(C.byref(a), d, None, p(st), p(dst), p(dm), p(gn), p(pa), p(pb))
+            ("bwd_chunk", lambda: [lib.issm_stage_bwd_chunk(C.byref(a), d, None, p(st), p(dst), p(dm), p(gn), p(pa), p(pb), p(redo))
                                    for d in range(nd)][-1]),
             ("bwd_dx", lambda: lib.issm_stage_bwd_dx(C.byref(a), None, p(dst), p(cabt), p(pd))),
             ("bwd_reduce", lambda: lib.issm_stage_bwd_reduce(C.byref(a), p(pa), p(pb), p(pd), p(dh0d))),

@@ -22,7 +22,8 @@ EXPORTS = [
     "issm_abi_version", "issm_last_error", "issm_fwd_workspace_bytes", "issm_bwd_workspace_bytes",
     "issm_scan_fwd", "issm_scan_bwd", "issm_stage_chunk_local", "issm_stage_state_passing_fwd",
     "issm_stage_chunk_scan", "issm_stage_bwd_gate", "issm_stage_bwd_dstates",
-    "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_stage_bwd_dx", "issm_stage_bwd_reduce",
+    "issm_stage_state_passing_bwd", "issm_stage_bwd_chunk", "issm_bwd_chunk_redo_ints", "issm_stage_bwd_dx",
+    "issm_stage_bwd_reduce",
     "issm_rmsnorm_bwd_blocks", "issm_gated_rmsnorm_fwd", "issm_gated_rmsnorm_bwd",
     "issm_gated_rmsnorm_bwd_noalloc",
     "issm_param_gen_bwd_blocks", "issm_param_gen_fwd", "issm_param_gen_bwd",
@@ -182,7 +183,9 @@ def load() -> C.CDLL:
     lib.issm_stage_bwd_gate.argtypes = [P(ScanArgs), vp, vp]
     lib.issm_stage_bwd_dstates.argtypes = [P(ScanArgs), vp, vp, vp]
     lib.issm_stage_state_passing_bwd.argtypes = [P(ScanArgs), vp, vp, vp, vp, vp]
-    lib.issm_stage_bwd_chunk.argtypes = [P(ScanArgs), C.c_int, vp, vp, vp, vp, vp, vp, vp]
+    lib.issm_stage_bwd_chunk.argtypes = [P(ScanArgs), C.c_int, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.issm_bwd_chunk_redo_ints.argtypes = [P(ScanArgs)]
+    lib.issm_bwd_chunk_redo_ints.restype = C.c_size_t
     lib.issm_stage_bwd_dx.argtypes = [P(ScanArgs), vp, vp, vp, vp]
     lib.issm_stage_bwd_reduce.argtypes = [P(ScanArgs), vp, vp, vp, vp]
     lib.issm_rmsnorm_bwd_blocks.argtypes = [C.c_int64]

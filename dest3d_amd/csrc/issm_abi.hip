@@ -19,7 +19,10 @@ int launch_bwd_dstates(const KP& p, const float* dy_ws, float* dstates, float* d
 int launch_state_bwd(const KP& p, const float* states, const float* cs_last, float* dstates, float* g_last,
                      float* dh0_dir, hipStream_t st);
 int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
-                     const float* g_last, float* partA, float* partBias, hipStream_t st);
+                     const float* g_last, float* partA, float* partBias, int* redo, int* redo_pending, hipStream_t st);
+int launch_bwd_chunk_redo(const KP& p, int ndirs, const float* dy_ws, const float* states, const float* dstates,
+                          const float* dm, const float* g_last, float* partA, float* partBias, const int* redo,
+                          hipStream_t st);
 int launch_bwd_dx(const KP& p, const float* dy_ws, const float* dstates, const float* cabt, float* partD,
                   hipStream_t st);
 int launch_bwd_reduce(const KP& p, const float* partA, const float* partBias, const float* partD,
@@ -90,7 +93,7 @@ struct FwdWs {
   size_t states, cs_last, cabt, out_x, total;  // offsets in floats
 };
 struct BwdWs {
-  size_t dstates, dm, g_last, dh0_dir, partA, partBias, partD, dy_ws, total;
+  size_t dstates, dm, g_last, dh0_dir, partA, partBias, partD, redo, dy_ws, total;
 };
 
 static int nchunks(const issm_dims& d) { return (d.seqlen + ISSM_CHUNK - 1) / ISSM_CHUNK; }
@@ -118,6 +121,7 @@ static BwdWs bwd_layout(const issm_dims& d, bool has_z) {
   w.partA = o; o += align64(Bt * nc * H * N);
   w.partBias = o; o += align64(Bt * nc * H * N);
   w.partD = o; o += align64(Bt * nc * H * P);
+  w.redo = o; o += align64(Bt * nc * H * ((N + ISSM_CHUNK - 1) / ISSM_CHUNK));  // one int per direction, workgroup and head
   w.dy_ws = o; if (has_z) o += align64(Bt * d.seqlen * H * P);
   w.total = o;
   return w;
@@ -330,9 +334,15 @@ int issm_stage_state_passing_bwd(const issm_scan_args* a, const float* states, c
                   "state_passing_bwd");
 }
 
+size_t issm_bwd_chunk_redo_ints(const issm_scan_args* a) {
+  if (check_dims(a)) return 0;
+  const issm_dims& d = a->dims;
+  return (size_t)d.batch * d.ndir * nchunks(d) * d.nheads * ((d.dstate + ISSM_CHUNK - 1) / ISSM_CHUNK);
+}
+
 int issm_stage_bwd_chunk(const issm_scan_args* a, int dir, const float* dy_gated, const float* states,
                          const float* dstates, const float* dm, const float* g_last, float* part_a,
-                         float* part_bias) {
+                         float* part_bias, int32_t* redo) {
   int rc = check_common(a);
   if (rc) return rc;
   if ((rc = check_dout(a, dy_gated))) return rc;
@@ -340,8 +350,15 @@ int issm_stage_bwd_chunk(const issm_scan_args* a, int dir, const float* dy_gated
   if (!states || !dstates || !dm || !g_last || !part_a || !part_bias) return fail(ISSM_E_NULL, "bwd_chunk: NULL buffer");
   KP p = make_kp(a);
   p.dir0 = dir;
-  return launched(launch_bwd_chunk(p, dy_gated, states, dstates, dm, g_last, part_a, part_bias, (hipStream_t)a->stream),
-                  "bwd_chunk");
+  int pending = 0;
+  if ((rc = launched(launch_bwd_chunk(p, dy_gated, states, dstates, dm, g_last, part_a, part_bias, redo, &pending,
+                                      (hipStream_t)a->stream),
+                     "bwd_chunk")))
+    return rc;
+  if (!pending) return ISSM_OK;
+  return launched(launch_bwd_chunk_redo(p, 1, dy_gated, states, dstates, dm, g_last, part_a, part_bias, redo,
+                                        (hipStream_t)a->stream),
+                  "bwd_chunk (redo)");
 }
 
 int issm_stage_bwd_dx(const issm_scan_args* a, const float* dy_gated, const float* dstates, const float* cabt,
@@ -393,14 +410,21 @@ int issm_scan_bwd(const issm_scan_args* a) {
                                       ws + bw.dh0_dir, st),
                      "state_passing_bwd")))
     return rc;
+  int* redo = reinterpret_cast<int*>(ws + bw.redo);
+  int pending = 0;
   for (int dir = 0; dir < p.ndir; ++dir) {
     KP pd = p;
     pd.dir0 = dir;
     if ((rc = launched(launch_bwd_chunk(pd, dy, sv + fw.states, ws + bw.dstates, ws + bw.dm, ws + bw.g_last,
-                                        ws + bw.partA, ws + bw.partBias, st),
+                                        ws + bw.partA, ws + bw.partBias, redo, &pending, st),
                        "bwd_chunk")))
       return rc;
   }
+  if (pending &&
+      (rc = launched(launch_bwd_chunk_redo(p, p.ndir, dy, sv + fw.states, ws + bw.dstates, ws + bw.dm, ws + bw.g_last,
+                                           ws + bw.partA, ws + bw.partBias, redo, st),
+                     "bwd_chunk (redo)")))
+    return rc;
   if ((rc = launched(launch_bwd_dx(p, dy, ws + bw.dstates, sv + fw.cabt, ws + bw.partD, st), "bwd_dx"))) return rc;
   return launched(launch_bwd_reduce(p, ws + bw.partA, ws + bw.partBias, ws + bw.partD, ws + bw.dh0_dir, a->dA,
                                     a->dt_bias ? a->ddt_bias : nullptr, a->D ? a->dD : nullptr, a->dh0, st),

@@ -115,30 +115,32 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
 #pragma unroll
         for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
       }
-      if (IOB) {
-        // bf16 inputs: the block goes out as one symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] (8 KB at the
-        // start of the unit's 16 KB): the F sums of k_bwd_chunk_bf contract over the columns of dM and the G sums over
-        // its rows, and with T both are rows of one tile, contiguous for a lane's 8 k-slots.
+      {
+        // The block goes out as the symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] (8 KB at the start of the
+        // unit's 16 KB): the F sums of the chunk backward contract over the columns of dM and the G sums over its rows,
+        // and with T both are rows of one tile, contiguous for a lane's k-slots.  bf16 inputs: T is dM rounded to
+        // bf16.  fp32 inputs: a second matrix of the same shape follows in the next 8 KB with the bf16 rounding of what
+        // the first one left, dM = hi + lo to 16 significand bits.
         uint16_t* mb = reinterpret_cast<uint16_t*>(m);
         const int sc = j * 16 + cm, l0 = wave * 16 + 4 * g4;
-        const unsigned w0 = pack_bf16(acc[0], acc[1]), w1 = pack_bf16(acc[2], acc[3]);
-        const uint16_t h[4] = {(uint16_t)w0, (uint16_t)(w0 >> 16), (uint16_t)w1, (uint16_t)(w1 >> 16)};
-        if (j < wave) {  // a block below the diagonal blocks: whole, and whole again mirrored
 #pragma unroll
-          for (int r = 0; r < 4; ++r) mb[(l0 + r) * CS + sc] = h[r];
-          *(uint2*)(mb + sc * CS + l0) = make_uint2(w0, w1);
-        } else {  // a diagonal block: the lane's entries on or below the diagonal, each mirrored
+        for (int half = 0; half < (IOB ? 1 : 2); ++half) {
+          const unsigned w0 = pack_bf16(acc[0], acc[1]), w1 = pack_bf16(acc[2], acc[3]);
+          const uint16_t h[4] = {(uint16_t)w0, (uint16_t)(w0 >> 16), (uint16_t)w1, (uint16_t)(w1 >> 16)};
+          if (j < wave) {  // a block below the diagonal blocks: whole, and whole again mirrored
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            if (sc <= l0 + r) mb[(l0 + r) * CS + sc] = h[r];
-            if (sc < l0 + r) mb[sc * CS + l0 + r] = h[r];
+            for (int r = 0; r < 4; ++r) mb[(l0 + r) * CS + sc] = h[r];
+            *(uint2*)(mb + sc * CS + l0) = make_uint2(w0, w1);
+          } else {  // a diagonal block: the lane's entries on or below the diagonal, each mirrored
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              if (sc <= l0 + r) mb[(l0 + r) * CS + sc] = h[r];
+              if (sc < l0 + r) mb[sc * CS + l0 + r] = h[r];
+            }
           }
-        }
-      } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int l = wave * 16 + 4 * g4 + r, sc = j * 16 + cm;
-          m[l * CS + sc] = sc <= l ? acc[r] : 0.0f;
+          for (int r = 0; r < 4; ++r) acc[r] -= bf16_to_f(h[r]);
+          mb += CS * CS;
         }
       }
     }
@@ -641,7 +643,7 @@ __device__ __forceinline__ void bwd_small_levels(const float (&cs)[16], const fl
 
 // partA, partBias: (Bt*nc, H, N) per-unit partial sums of dA and ddt_bias
 template <int PT, bool IOB, bool DTB, bool FULL>
-__device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+__device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias, const int* __restrict__ redo, const int dir_here, const bool mirror) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -651,14 +653,28 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
   const int cm = lane & 15, g4 = lane >> 4;
   const int nsl = (p.N + NS - 1) / NS;
   Unit u;
+  // `redo` (one word per direction, workgroup and head, written by the tile-base kernel): only the marked heads are
+  // evaluated here, and their ddt / dB / dC are added to what that kernel left (zero, or the other direction's share).
+  // `mirror`: the workgroup's chunk index counts from the other end -- the chunk of this direction that covers the
+  // same tokens as the un-mirrored chunk of the other direction (one workgroup then adds both directions' shares to
+  // those tokens' ddt one after the other, and no two workgroups ever update one address).
   int id = xcd_remap(blockIdx.x, gridDim.x);
   const int ns = id % nsl;
   id /= nsl;
   u.g = id % p.G;
   id /= p.G;
-  u.c = p.c_lo + id % p.ncl;
+  const int cj = id % p.ncl;
+  u.c = p.c_lo + (mirror ? p.ncl - 1 - cj : cj);
   u.b = id / p.ncl;
-  u.dir = p.dir0;
+  if (redo) {
+    const int nblk = p.B * p.ncl * p.G * nsl;
+    const int wg = ((u.b * p.ncl + (u.c - p.c_lo)) * p.G + u.g) * nsl + ns;  // as the tile-base kernel counts them
+    redo += (dir_here * nblk + wg) * p.hpg;
+    int any = 0;
+    for (int hh = 0; hh < p.hpg; ++hh) any |= redo[hh];
+    if (!any) return;
+  }
+  u.dir = dir_here;
   u.bt = u.b * p.ndir + u.dir;
   u.h = u.g * p.hpg;
   const int n = ns * NS + wave * 16 + cm;
@@ -678,9 +694,10 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
   for (int hh = 0; hh < p.hpg; ++hh) {
+    if (redo && !redo[hh]) continue;
     // the reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
     // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first
-    u.h = u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh);
+    u.h = u.g * p.hpg + (dir_here ? p.hpg - 1 - hh : hh);
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
     lane_load_ln<DTB>(p.dt, u.b, u.h, n, vn, g4, rm, raw);
@@ -696,7 +713,7 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
       asm volatile("" : "+v"(tq));
       dy_load<IOB, PT, FULL>(p, u, dy_ws, dv, tq);
       lp_load<IOB, PT, FULL>(p, u, p.x[u.dir], xv, tq);
-      tril_load(dm + sq_off(p, u.bt, u.c, u.h), mv, tq);
+      tril_load_hl(dm + sq_off(p, u.bt, u.c, u.h), mv, tq);
       __syncthreads();  // the previous head no longer reads the LDS tiles
       lp_store_split<PT, LDS_>(dv, s.dys.hi, s.dys.lo, tq);
       lp_store_split<PT, LDS_>(xv, s.xs.hi, s.xs.lo, tq);
@@ -816,7 +833,7 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
     pin16(cs); pin16(e1); pin16(x2);
     // the second direction adds to the first one's ddt: fetch it while the last levels run
     float old[16];
-    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
+    if ((redo || dir_here > 0) && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
     bwd_small_levels(cs, Bd, Cv, s.dms(), e1, x2, gq);
     __builtin_amdgcn_sched_barrier(0);
@@ -872,7 +889,7 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
       sumA += da * dtp[k];
       val[k] = (val[k] + da * An) * dfac[k];
       if (rm.full || rowk(k) < lim) sumB += val[k];
-      if (p.dir0 > 0) val[k] += old[k];
+      if (redo || dir_here > 0) val[k] += old[k];
     }
     if (p.ddt.ptr) lane_store_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, val);
     sumA = scan_g_incl(sumA, g4);
@@ -890,20 +907,34 @@ __device__ __forceinline__ void k_bwd_chunk_body(const KP& p, const float* __res
       vb[k] = s.dbc[k * NTHREADS + tid];
       vc[k] = s.dbc[(16 + k) * NTHREADS + tid];
     }
+    if (redo) {
+      float ob[16], oc[16];
+      if (p.dB[u.dir].ptr) lane_load_ln<IOB>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, ob);
+      if (p.dC[u.dir].ptr) lane_load_ln<IOB>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, oc);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        vb[k] += ob[k];
+        vc[k] += oc[k];
+      }
+    }
     if (p.dB[u.dir].ptr) lane_store_ln<IOB>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, vb);
     if (p.dC[u.dir].ptr) lane_store_ln<IOB>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
   }
 }
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
-  k_bwd_chunk_body<PT, IOB, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias, const int* __restrict__ redo, int ndirs) {
+  // (ndirs > 1 only with `redo`: the marked heads of directions p.dir0, p.dir0 + 1, .. one after the other)
+  for (int d = 0; d < ndirs; ++d) {
+    if (d) __syncthreads();
+    k_bwd_chunk_body<PT, IOB, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, redo, p.dir0 + d, d > 0);
+  }
 }
 // One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
 // for the last one (uniform per workgroup).
 template <int PT, bool IOB, bool DTB>
 __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_mixed(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
-  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_body<PT, IOB, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
-  else k_bwd_chunk_body<PT, IOB, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_body<PT, IOB, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, nullptr, p.dir0, false);
+  else k_bwd_chunk_body<PT, IOB, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, nullptr, p.dir0, false);
 }
 
 
@@ -1101,7 +1132,7 @@ __device__ __forceinline__ void bwd_small_levels_bf(const float (&cs)[16], const
 }
 
 template <int PT, bool DTB, bool FULL>
-__device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
+__device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias, const int* __restrict__ redo, const int dir_here, const bool mirror) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdChunkBfSmem<PT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
@@ -1111,14 +1142,28 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
   const int cm = lane & 15, g4 = lane >> 4;
   const int nsl = (p.N + NS - 1) / NS;
   Unit u;
+  // `redo` (one word per direction, workgroup and head, written by the tile-base kernel): only the marked heads are
+  // evaluated here, and their ddt / dB / dC are added to what that kernel left (zero, or the other direction's share).
+  // `mirror`: the workgroup's chunk index counts from the other end -- the chunk of this direction that covers the
+  // same tokens as the un-mirrored chunk of the other direction (one workgroup then adds both directions' shares to
+  // those tokens' ddt one after the other, and no two workgroups ever update one address).
   int id = xcd_remap(blockIdx.x, gridDim.x);
   const int ns = id % nsl;
   id /= nsl;
   u.g = id % p.G;
   id /= p.G;
-  u.c = p.c_lo + id % p.ncl;
+  const int cj = id % p.ncl;
+  u.c = p.c_lo + (mirror ? p.ncl - 1 - cj : cj);
   u.b = id / p.ncl;
-  u.dir = p.dir0;
+  if (redo) {
+    const int nblk = p.B * p.ncl * p.G * nsl;
+    const int wg = ((u.b * p.ncl + (u.c - p.c_lo)) * p.G + u.g) * nsl + ns;  // as the tile-base kernel counts them
+    redo += (dir_here * nblk + wg) * p.hpg;
+    int any = 0;
+    for (int hh = 0; hh < p.hpg; ++hh) any |= redo[hh];
+    if (!any) return;
+  }
+  u.dir = dir_here;
   u.bt = u.b * p.ndir + u.dir;
   u.h = u.g * p.hpg;
   const int n = ns * NS + wave * 16 + cm;
@@ -1136,7 +1181,7 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
 
   // The reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
   // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first.
-  auto head_of = [&](int hh) { return u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh); };
+  auto head_of = [&](int hh) { return u.g * p.hpg + (dir_here ? p.hpg - 1 - hh : hh); };
   // a head's tiles on their way from global memory to LDS: raw bf16 pairs (x, dy) and the thread's two 16-byte pieces
   // of T (rows tq >> 3 and 32 + (tq >> 3), columns 8 (tq & 7) .. + 7)
   uint2 nx[PT], ny[PT];
@@ -1166,6 +1211,7 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
   };
 
   for (int hh = 0; hh < p.hpg; ++hh) {
+    if (redo && !redo[hh]) continue;
     u.h = head_of(hh);
     // ---- global loads of this head
     float raw[16], dsv[KP_], hv[KP_];
@@ -1257,7 +1303,7 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
     pin16(cs); pin16(e1); pin16(x2); pin16(dcs);
     // the second direction adds to the first one's ddt: fetch it while the last level runs
     float old[16];
-    if (p.dir0 > 0 && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
+    if ((redo || dir_here > 0) && p.ddt.ptr) lane_load_ln<DTB>(p.ddt, u.b, u.h, n, vn, g4, rm, old);
     __builtin_amdgcn_sched_barrier(0);
     bwd_mid_level_bf<LDM, 2>(cs, Bv, dtp, Cv, dm_, dm_, e1, x2, dcs, cq, gq);
     __builtin_amdgcn_sched_barrier(0);
@@ -1312,7 +1358,7 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
       val[k] = (val[k] + da * An) * dfac[k];
       if (rm.full || rowk(k) < lim) sumB += val[k];
     }
-    if (p.dir0 > 0 && p.ddt.ptr) {
+    if ((redo || dir_here > 0) && p.ddt.ptr) {
 #pragma unroll
       for (int k = 0; k < 16; ++k) val[k] += old[k];
     }
@@ -1332,20 +1378,33 @@ __device__ __forceinline__ void k_bwd_chunk_bf_body(const KP& p, const float* __
       vb[k] = s.dbc[k * NTHREADS + tid];
       vc[k] = s.dbc[(16 + k) * NTHREADS + tid];
     }
+    if (redo) {
+      float ob[16], oc[16];
+      if (p.dB[u.dir].ptr) lane_load_ln<true>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, ob);
+      if (p.dC[u.dir].ptr) lane_load_ln<true>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, oc);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        vb[k] += ob[k];
+        vc[k] += oc[k];
+      }
+    }
     if (p.dB[u.dir].ptr) lane_store_ln<true>(p.dB[u.dir], u.b, u.g, n, vn, g4, rm, vb);
     if (p.dC[u.dir].ptr) lane_store_ln<true>(p.dC[u.dir], u.b, u.g, n, vn, g4, rm, vc);
   }
 }
 template <int PT, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
-  k_bwd_chunk_bf_body<PT, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+__global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias, const int* __restrict__ redo, int ndirs) {
+  for (int d = 0; d < ndirs; ++d) {
+    if (d) __syncthreads();
+    k_bwd_chunk_bf_body<PT, DTB, FULL>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, redo, p.dir0 + d, d > 0);
+  }
 }
 // One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
 // for the last one (uniform per workgroup).
 template <int PT, bool DTB>
 __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf_mixed(KP p, const float* __restrict__ dy_ws, const float* __restrict__ states, const float* __restrict__ dstates, const float* __restrict__ dm, const float* __restrict__ g_last, float* __restrict__ partA, float* __restrict__ partBias) {
-  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_bf_body<PT, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
-  else k_bwd_chunk_bf_body<PT, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+  if (p.c_lo + (xcd_remap(blockIdx.x, gridDim.x) / ((p.N + NS - 1) / NS) / p.G) % p.ncl == p.nc - 1) k_bwd_chunk_bf_body<PT, DTB, false>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, nullptr, p.dir0, false);
+  else k_bwd_chunk_bf_body<PT, DTB, true>(p, dy_ws, states, dstates, dm, g_last, partA, partBias, nullptr, p.dir0, false);
 }
 
 
@@ -1692,27 +1751,62 @@ int launch_state_bwd(const KP& p, const float* states, const float* cs_last, flo
 
 template <int PT, bool IOB, bool DTB, bool FULL, bool MIXED>
 static int launch_bwd_chunk_t(const KP& p, int blocks, const float* dy_ws, const float* states, const float* dstates,
-                              const float* dm, const float* g_last, float* partA, float* partBias, hipStream_t st) {
-  if constexpr (IOB) {  // bf16 inputs: every product on the bf16 matrix instructions
+                              const float* dm, const float* g_last, float* partA, float* partBias, const int* redo,
+                              int ndirs, hipStream_t st) {
+  if constexpr (MIXED) {  // (never with `redo`: the tile-base kernel takes complete tiles only)
+    if constexpr (IOB) {
+      const size_t sm = sizeof(BwdChunkBfSmem<PT>);
+      if (int e = set_lds(&k_bwd_chunk_bf_mixed<PT, DTB>, sm)) return e;
+      hipLaunchKernelGGL((k_bwd_chunk_bf_mixed<PT, DTB>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+    } else {
+      const size_t sm = sizeof(BwdChunkSmem<PT>);
+      if (int e = set_lds(&k_bwd_chunk_mixed<PT, false, DTB>, sm)) return e;
+      hipLaunchKernelGGL((k_bwd_chunk_mixed<PT, false, DTB>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+    }
+  } else if constexpr (IOB) {  // bf16 inputs: every product on the bf16 matrix instructions
     const size_t sm = sizeof(BwdChunkBfSmem<PT>);
-    constexpr auto kern = MIXED ? &k_bwd_chunk_bf_mixed<PT, DTB> : &k_bwd_chunk_bf<PT, DTB, FULL>;
-    if (int e = set_lds(kern, sm)) return e;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+    if (int e = set_lds(&k_bwd_chunk_bf<PT, DTB, FULL>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk_bf<PT, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias, redo, ndirs);
   } else {
     const size_t sm = sizeof(BwdChunkSmem<PT>);
-    constexpr auto kern = MIXED ? &k_bwd_chunk_mixed<PT, false, DTB> : &k_bwd_chunk<PT, false, DTB, FULL>;
-    if (int e = set_lds(kern, sm)) return e;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias);
+    if (int e = set_lds(&k_bwd_chunk<PT, false, DTB, FULL>, sm)) return e;
+    hipLaunchKernelGGL((k_bwd_chunk<PT, false, DTB, FULL>), dim3(blocks), dim3(NTHREADS), sm, st, p, dy_ws, states, dstates, dm, g_last, partA, partBias, redo, ndirs);
   }
   return 0;
 }
 
+bool bwd_tile_available(const KP& p, const float* dy_ws);
+int launch_bwd_tile(const KP& p, const float* states, const float* dstates, const float* dm, const float* g_last,
+                    float* partA, float* partBias, int* redo, hipStream_t st);
+
+// Chunk backward of direction p.dir0.  With a `redo` buffer (issm_bwd_chunk_redo_ints words) the tile-base kernel
+// (issm_bwd_tile.hip) does the work and marks the heads outside its range; launch_bwd_chunk_redo then evaluates those
+// with the level-hierarchy kernel.  Without one, or for calls the tile-base kernel is not built for (ragged tiles, packed
+// sequences, a gate, mixed input types), the level-hierarchy kernel evaluates everything and *redo_pending stays 0.
 int launch_bwd_chunk(const KP& p, const float* dy_ws, const float* states, const float* dstates, const float* dm,
-                     const float* g_last, float* partA, float* partBias, hipStream_t st) {
+                     const float* g_last, float* partA, float* partBias, int* redo, int* redo_pending, hipStream_t st) {
+  const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
+  if (redo && bwd_tile_available(p, dy_ws)) {
+    if (redo_pending) *redo_pending = 1;
+    return launch_bwd_tile(p, states, dstates, dm, g_last, partA, partBias, redo, st);
+  }
+  ISSM_DISPATCH(p, {
+    if (int e = launch_bwd_chunk_t<PT_, IOB_, DTB_, FULL_, MIXED_>(p, blocks, dy_ws, states, dstates, dm, g_last, partA,
+                                                                  partBias, nullptr, 1, st))
+      return e;
+  });
+  return (int)hipGetLastError();
+}
+
+// The level-hierarchy kernel over the heads the tile-base launches of directions p.dir0 .. p.dir0 + ndirs - 1 marked in
+// `redo` (ordinary inputs mark none, and its workgroups return at once).
+int launch_bwd_chunk_redo(const KP& p, int ndirs, const float* dy_ws, const float* states, const float* dstates,
+                          const float* dm, const float* g_last, float* partA, float* partBias, const int* redo,
+                          hipStream_t st) {
   const int blocks = p.B * p.nc * p.G * ((p.N + NS - 1) / NS);
   ISSM_DISPATCH(p, {
     if (int e = launch_bwd_chunk_t<PT_, IOB_, DTB_, FULL_, MIXED_>(p, blocks, dy_ws, states, dstates, dm, g_last, partA,
-                                                                  partBias, st))
+                                                                  partBias, redo, ndirs, st))
       return e;
   });
   return (int)hipGetLastError();

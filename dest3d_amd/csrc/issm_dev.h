@@ -22,6 +22,12 @@
 #include <stdint.h>
 #include <type_traits>
 
+// A wave-uniform value made opaque to the optimizer (its multiples are then formed next to their use instead of being
+// hoisted out of loops into scarce scalar registers).  A translation unit may define its own form before including this.
+#ifndef ISSM_OPAQUE_S
+#define ISSM_OPAQUE_S(x) asm volatile("" : "+s"(x))
+#endif
+
 namespace issm {
 
 constexpr int CS = 64;         // tokens per chunk
@@ -532,7 +538,7 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
     // integer add per element.
     const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
     unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
-    asm volatile("" : "+s"(ks));
+    ISSM_OPAQUE_S(ks);
     const char* qb = (const char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) r[k] = *(const T*)(qb + (lo + (unsigned)(16 * (k >> 2) + (k & 3)) * ks));
@@ -547,7 +553,7 @@ __device__ __forceinline__ void lane_load_ln(const TensorD& t, int b, int third,
     const int rmax = rm.nvalid - 1 - 4 * g4;  // last existing row, relative to the lane's row 0 (may be negative)
     const unsigned lo = (unsigned)(rm.base * (int)t.s1 + (vn ? n : 0)) * (unsigned)sizeof(T);
     unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
-    asm volatile("" : "+s"(ks));
+    ISSM_OPAQUE_S(ks);
     const char* qb = (const char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -569,7 +575,7 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
   if (rm.full) {
     const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
     unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
-    asm volatile("" : "+s"(ks));
+    ISSM_OPAQUE_S(ks);
     char* qb = (char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -581,7 +587,7 @@ __device__ __forceinline__ void lane_store_ln(const TensorD& t, int b, int third
     const int rmax = rm.nvalid - 1 - 4 * g4;
     const unsigned lo = (unsigned)(rm.base * (int)t.s1 + n) * (unsigned)sizeof(T);
     unsigned ks = (unsigned)(rm.step * (int)t.s1) * (unsigned)sizeof(T);
-    asm volatile("" : "+s"(ks));
+    ISSM_OPAQUE_S(ks);
     char* qb = (char*)q;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -600,7 +606,7 @@ __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int 
   if (full) {
     const unsigned lo = (unsigned)(4 * g4 * N + n) * 4u;
     unsigned nb = (unsigned)N * 4u;
-    asm volatile("" : "+s"(nb));
+    ISSM_OPAQUE_S(nb);
     const char* sb = (const char*)src;
 #pragma unroll
     for (int q = 0; q < CNT; ++q) out[q] = *(const float*)(sb + (lo + (unsigned)(16 * (q >> 2) + (q & 3)) * nb));
@@ -610,7 +616,7 @@ __device__ __forceinline__ void lane_load_pn(const float* __restrict__ src, int 
     const int pmax = P - 1 - 4 * g4;
     const unsigned lo = (unsigned)(4 * g4 * N + (vn ? n : 0)) * 4u;
     unsigned nb = (unsigned)N * 4u;
-    asm volatile("" : "+s"(nb));
+    ISSM_OPAQUE_S(nb);
     const char* sb = (const char*)src;
 #pragma unroll
     for (int q = 0; q < CNT; ++q)
@@ -634,20 +640,17 @@ __device__ __forceinline__ Coef lane_coef(const KP& p, int h, int n, bool vn) {
   c.bias = (vn && p.dt_bias) ? p.dt_bias[h * p.N + n] : 0.0f;
   return c;
 }
-template <bool WANT_DFAC>
-__device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn, int cm, int g4, const RowMap& rm,
-                                           const float (&raw)[16], float (&dtp)[16], float (&cs)[16],
-                                           float (&dfac)[16]) {
-  const float A2 = cf.A * LOG2E;
-  const float bias = cf.bias;
-  // softplus and its derivative share one exponential: with t = e^pre, softplus = log(1 + t) and sigmoid = t / (1 + t);
-  // above the reference's threshold of 20 both are replaced (identity, 1).  F_NOCLAMP: the limits are (0, inf) and
-  // softplus is on, so the clamp and its mask cannot act and are skipped.
+// dt transform of CNT values that already include the bias: softplus -> clamp; dfac (if WANT_DFAC) receives
+// d dt' / d dt.  Softplus and its derivative share one exponential: with t = e^pre, softplus = log(1 + t) and
+// sigmoid = t / (1 + t); above the reference's threshold of 20 both are replaced (identity, 1).  F_NOCLAMP: the limits
+// are (0, inf) and softplus is on, so the clamp and its mask cannot act and are skipped.
+template <bool WANT_DFAC, int CNT>
+__device__ __forceinline__ void dt_transform(const KP& p, const float (&pre_)[CNT], float (&dtp)[CNT], float (&dfac)[CNT]) {
   if (p.flags & F_SOFTPLUS) {
     if (p.flags & F_NOCLAMP) {
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const float pre = raw[k] + bias;
+      for (int k = 0; k < CNT; ++k) {
+        const float pre = pre_[k];
         const float t = ex2(pre * LOG2E), u = 1.0f + t;
         const bool big = pre > 20.0f;
         dtp[k] = big ? pre : LN2 * __builtin_amdgcn_logf(u);
@@ -655,8 +658,8 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
       }
     } else {
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const float pre = raw[k] + bias;
+      for (int k = 0; k < CNT; ++k) {
+        const float pre = pre_[k];
         const float t = ex2(pre * LOG2E), u = 1.0f + t;
         const bool big = pre > 20.0f;
         const float sp = big ? pre : LN2 * __builtin_amdgcn_logf(u);
@@ -666,17 +669,34 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
     }
   } else {
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const float sp = raw[k] + bias;
+    for (int k = 0; k < CNT; ++k) {
+      const float sp = pre_[k];
       dtp[k] = __builtin_amdgcn_fmed3f(sp, p.dt_min, p.dt_max);
       if (WANT_DFAC) dfac[k] = (sp < p.dt_min || sp > p.dt_max) ? 0.0f : 1.0f;
     }
   }
+}
+// dt transform (bias -> softplus -> clamp) of the lane's 16 rows.  Rows past the end of the sequence and absent columns
+// come out as dt' = 0.
+template <bool WANT_DFAC>
+__device__ __forceinline__ void lane_dt(const KP& p, const Coef& cf, bool vn, int g4, const RowMap& rm,
+                                        const float (&raw)[16], float (&dtp)[16], float (&dfac)[16]) {
+  float pre[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) pre[k] = raw[k] + cf.bias;
+  dt_transform<WANT_DFAC, 16>(p, pre, dtp, dfac);
   if (!rm.full) {  // rows past the end of the sequence and absent columns behave as dt' = 0
 #pragma unroll
     for (int k = 0; k < 16; ++k)
       if (!(vn && lane_row(k, g4) < rm.nvalid)) dtp[k] = 0.0f;
   }
+}
+template <bool WANT_DFAC>
+__device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn, int cm, int g4, const RowMap& rm,
+                                           const float (&raw)[16], float (&dtp)[16], float (&cs)[16],
+                                           float (&dfac)[16]) {
+  const float A2 = cf.A * LOG2E;
+  lane_dt<WANT_DFAC>(p, cf, vn, g4, rm, raw, dtp, dfac);
   // Running sum down the 64 rows: in the lane over its four rows of each tile, then across the four lane groups
   // of a tile, then across the tiles.  The cross-lane steps of the four tiles do not depend on each other, so each
   // step is issued for all four before any result is used (a cross-lane fetch goes through the LDS pipe: taken tile
@@ -726,6 +746,64 @@ __device__ __forceinline__ float lane_prep(const KP& p, const Coef& cf, bool vn,
   }
   return carry;
 }
+
+// Running sums of a = dt' A log2(e) restarted at every 16-row tile: pc[k] = sum of a over the rows of k's tile up to and
+// including k's row, tt[J] = the whole tile's sum (the same on the four lanes of a column).  Used by the kernels that
+// write a decay exp2(cs[l] - cs[s]) as  exp2(pc[l]) . exp2(base(tile of l) - base(tile of s)) . exp2(-pc[s])  with
+// base(J) = tt[0] + .. + tt[J-1]: two exponentials per element and ten per column serve every pair of rows of the chunk.
+__device__ __forceinline__ void lane_tile_sums(float A2, int cm, int g4, const RowMap& rm, const float (&dtp)[16],
+                                               float (&pc)[16], float (&tt)[4]) {
+  float c[4], v[4], t[4];
+  if (rm.full || rm.cut == 0) {
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      float a = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a += dtp[4 * J + j] * A2;
+        pc[4 * J + j] = a;
+      }
+      c[J] = a;
+    }
+  } else {  // packed sequences: the sum drops by SEQ_CUT at every row where the sequence id changes
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      const unsigned bits = (unsigned)(rm.cut >> (16 * J + 4 * g4)) & 15u;
+      float a = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        a += dtp[4 * J + j] * A2 - (((bits >> j) & 1u) ? SEQ_CUT : 0.0f);
+        pc[4 * J + j] = a;
+      }
+      c[J] = a;
+    }
+  }
+#pragma unroll
+  for (int J = 0; J < 4; ++J) t[J] = __shfl_up(c[J], 16, 64);
+#pragma unroll
+  for (int J = 0; J < 4; ++J) v[J] = g4 >= 1 ? c[J] + t[J] : c[J];
+#pragma unroll
+  for (int J = 0; J < 4; ++J) t[J] = __shfl_up(v[J], 32, 64);
+#pragma unroll
+  for (int J = 0; J < 4; ++J) v[J] = g4 >= 2 ? v[J] + t[J] : v[J];  // inclusive over the lane groups
+#pragma unroll
+  for (int J = 0; J < 4; ++J) tt[J] = __shfl(v[J], cm + 48, 64);    // tile totals
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    const float add = v[J] - c[J];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pc[4 * J + j] += add;
+  }
+}
+
+// v_mfma_f32_16x16x16_bf16: lane (m, g4) supplies k = 4 g4 .. 4 g4 + 3 -- in the column-lane layout exactly the lane's
+// four rows of one 16-row tile.
+typedef short sh4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f4 mfma_bf16k(bf4 a, bf4 b, f4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(sh4, a), __builtin_bit_cast(sh4, b), c, 0, 0, 0);
+}
+// an fp32 value cut to 16 significand bits (towards zero): it then splits into two bf16 numbers exactly
+__device__ __forceinline__ float trunc16(float v) { return __uint_as_float(__float_as_uint(v) & 0xffffff00u); }
 
 // ------------------------------------------------------------------ cooperative tile loaders
 // The unit's (64 x P) tile of a (B,L,H,P) tensor, zero padded to 16*PT columns: registers, then
@@ -864,6 +942,22 @@ __device__ __forceinline__ void tril_load(const float* __restrict__ src, f4 (&v)
   for (int i = 0; i < 4; ++i) {
     const int e = tid + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
     v[i] = (s4 <= l) ? *(const f4*)(src + l * CS + s4) : (f4){0, 0, 0, 0};
+  }
+}
+// The same lower triangle from the pair of symmetric bf16 matrices (hi at src, lo 8 KB behind it, each 64 x 64) that
+// k_bwd_dstates writes for fp32 inputs: dM = hi + lo.
+__device__ __forceinline__ void tril_load_hl(const float* __restrict__ src, f4 (&v)[4], int tid = threadIdx.x) {
+  const uint16_t* hi = reinterpret_cast<const uint16_t*>(src);
+  const uint16_t* lo = hi + CS * CS;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = tid + i * NTHREADS, l = e >> 4, s4 = (e & 15) * 4;
+    const uint2 a = *(const uint2*)(hi + l * CS + s4), b = *(const uint2*)(lo + l * CS + s4);
+    const f4 w = {__uint_as_float(a.x << 16) + __uint_as_float(b.x << 16),
+                  __uint_as_float(a.x & 0xffff0000u) + __uint_as_float(b.x & 0xffff0000u),
+                  __uint_as_float(a.y << 16) + __uint_as_float(b.y << 16),
+                  __uint_as_float(a.y & 0xffff0000u) + __uint_as_float(b.y & 0xffff0000u)};
+    v[i] = (s4 <= l) ? w : (f4){0, 0, 0, 0};
   }
 }
 __device__ __forceinline__ void tril_store(const f4 (&v)[4], float* dst, int tid = threadIdx.x) {

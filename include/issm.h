@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define ISSM_ABI_VERSION 4
+#define ISSM_ABI_VERSION 5
 #define ISSM_CHUNK 64 /* tokens per internal chunk */
 
 typedef enum issm_status {
@@ -181,9 +181,10 @@ int issm_stage_chunk_scan(const issm_scan_args* args, const float* states, const
 int issm_stage_bwd_gate(const issm_scan_args* args, const float* out_x, float* dy_gated);
 /* issm_stage_bwd_dstates: dH_c = dy^T . (C*exp(cs)) into dstates (Bt,nc,H,P,N) and
  *   dM = tril(dy . x^T) into dm (Bt,nc,H,64,64); either output may be NULL.  `dy` is args->dout
- *   unless dy_gated is given.  With io_dtype = ISSM_BF16 a block of dm holds, in the first 8 of its 16 KB, the
- *   symmetric 64 x 64 bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] instead of the fp32 lower triangle -- the form
- *   issm_stage_bwd_chunk reads for bf16 inputs.  Replaces _chunk_scan_bwd_dstates (issm_chunk_scan.py:380-512) and
+ *   unless dy_gated is given.  A 16 KB block of dm holds the symmetric 64 x 64 bf16 matrix
+ *   T[i][j] = dM[max(i,j)][min(i,j)] in its first 8 KB (the form issm_stage_bwd_chunk reads: the sums over rows and
+ *   over columns of dM both become row reads) and, for io_dtype = ISSM_F32, a second such matrix in the other 8 KB
+ *   holding the bf16 rounding of what the first left: dM = hi + lo to 16 significand bits.  Replaces _chunk_scan_bwd_dstates (issm_chunk_scan.py:380-512) and
  *   _chunk_scan_bwd_dcb (issm_chunk_scan.py:790-900). */
 int issm_stage_bwd_dstates(const issm_scan_args* args, const float* dy_gated, float* dstates, float* dm);
 /* issm_stage_state_passing_bwd: reverse recurrence in place (dstates[c] becomes dS_c, the gradient
@@ -200,10 +201,18 @@ int issm_stage_state_passing_bwd(const issm_scan_args* args, const float* states
  *   (issm_chunk_scan.py:515-657), _chunk_scan_chunk_state_bwd_dt (issm_combined.py:398-557),
  *   _bmm_CABT_dbc_chunk_bwd (issm_cabt_bmm.py:454-673), _chunk_scan_bwd_ddAcs_stable
  *   (issm_chunk_scan.py:903-1031) and the elementwise part of _chunk_cumsum_bwd
- *   (issm_chunk_state.py:107-231). */
+ *   (issm_chunk_state.py:107-231).
+ *   `redo` (issm_bwd_chunk_redo_ints(args) ints, contents irrelevant on entry, or NULL): with it the sums with the
+ *   decay inside run in tile-base form (two exponentials per element, every block of the chunk a plain matrix
+ *   product) wherever a 16-row tile's total decay stays below 2^96, and the level-hierarchy kernel, which has no such
+ *   limit, evaluates only the (workgroup, head) pairs the buffer then marks; NULL: the level-hierarchy kernel
+ *   evaluates everything.  Same results to rounding either way. */
 int issm_stage_bwd_chunk(const issm_scan_args* args, int dir, const float* dy_gated,
                          const float* states, const float* dstates, const float* dm,
-                         const float* g_last, float* part_a, float* part_bias);
+                         const float* g_last, float* part_a, float* part_bias, int32_t* redo);
+/* Number of ints issm_stage_bwd_chunk's `redo` buffer needs (batch * directions * chunks * heads * 64-column slices;
+ *   each direction uses its own part); 0 on bad dimensions.  No counterpart in the reference. */
+size_t issm_bwd_chunk_redo_ints(const issm_scan_args* args);
 /* issm_stage_bwd_dx: dx and the per-unit partial sums part_d (Bt*nc*H,P) of dD.  Replaces
  *   _chunk_scan_chunk_state_bwd_dx (issm_combined.py:183-395). */
 int issm_stage_bwd_dx(const issm_scan_args* args, const float* dy_gated, const float* dstates,

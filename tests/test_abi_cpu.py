@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported(lib):
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/issm.h but not exported"
     assert sorted(L.EXPORTS) == names
-    assert lib.issm_abi_version() == 4
+    assert lib.issm_abi_version() == 5
 
 
 def test_struct_layout_matches_header(lib):

@@ -480,7 +480,9 @@ def test_stage_entry_points_match_oracle_intermediates(shape):
     L.check(lib.issm_stage_bwd_dstates(C.byref(a), None, dst.data_ptr(), dm.data_ptr()), "dstates")
     torch.cuda.synchronize()
     _check("dH", dst, ref["dH"], BWD32)
-    _check("dM", torch.tril(dm), ref["dM"], BWD32)
+    # dM leaves the kernel as a pair of symmetric bf16 matrices per unit, dM = hi + lo to 16 bits (include/issm.h)
+    halves = dm.view(torch.bfloat16).reshape(Bsz, nc, H, 2, 64, 64).float()
+    _check("dM", torch.tril(halves[:, :, :, 0] + halves[:, :, :, 1]), ref["dM"], BWD32)
     g_next, dh0d = f(Bsz, nc, H, N), f(1, Bsz, H, P, N)
     L.check(lib.issm_stage_state_passing_bwd(C.byref(a), states.data_ptr(), cs_last.data_ptr(), dst.data_ptr(),
                                              g_next.data_ptr(), dh0d.data_ptr()), "sp_bwd")
@@ -491,8 +493,9 @@ def test_stage_entry_points_match_oracle_intermediates(shape):
     ddt, dB, dC, dx = f(Bsz, L_, H, N), f(Bsz, L_, G, N), f(Bsz, L_, G, N), f(Bsz, L_, H, P)
     pa, pb, pd = f(Bsz * nc, H, N), f(Bsz * nc, H, N), f(Bsz * nc * H, P)
     a.ddt, a.dB[0], a.dC[0], a.dx[0] = (L.tensor_desc(t) for t in (ddt, dB, dC, dx))
+    redo = torch.full((lib.issm_bwd_chunk_redo_ints(C.byref(a)),), -1, dtype=torch.int32, device=dev)
     L.check(lib.issm_stage_bwd_chunk(C.byref(a), 0, None, states.data_ptr(), dst.data_ptr(), dm.data_ptr(),
-                                     g_next.data_ptr(), pa.data_ptr(), pb.data_ptr()), "bwd_chunk")
+                                     g_next.data_ptr(), pa.data_ptr(), pb.data_ptr(), redo.data_ptr()), "bwd_chunk")
     L.check(lib.issm_stage_bwd_dx(C.byref(a), None, dst.data_ptr(), cabt.data_ptr(), pd.data_ptr()), "bwd_dx")
     dA, dbias, dD, dh0 = f(H, N), f(H, N), f(H), f(Bsz, H, P, N)
     a.dA, a.ddt_bias, a.dD, a.dh0 = dA.data_ptr(), dbias.data_ptr(), dD.data_ptr(), dh0.data_ptr()
@@ -792,9 +795,13 @@ def test_large_bidirectional_fp32_shape():
 
 def test_extreme_decay_is_finite_and_accurate():
     """Decays that underflow within a few rows (|dt' A| up to ~3000 per step) and rows that do not decay at all
-    (dt' = 0) in the same chunk: the level factors never exceed 1, so nothing may overflow.  Accuracy bar here:
-    1e-3 instead of 1e-4 / 1e-3 -- with running sums of dt' A in the thousands, one fp32 ulp of the sum (the
-    reference keeps it in fp32 as well, issm_chunk_state.py:84-104) is already ~5e-4 in the exponent."""
+    (dt' = 0) in the same chunk: the level factors never exceed 1, so nothing may overflow (every head here is outside
+    the tile-base kernel's range and falls to the level-hierarchy kernel).  Accuracy bar here: 1e-3 instead of
+    1e-4 / 1e-3 -- with running sums of dt' A in the thousands, one fp32 ulp of the sum (the reference keeps it in fp32 as
+    well, issm_chunk_state.py:84-104) is already ~5e-4 in the exponent.  dA is one sum per (head, state) over all tokens of
+    terms of both signs that nearly cancel here (condition number ~5000 against the intra-chunk matrix dM = dy x^T): dM
+    reaches the kernels with 16 significand bits, which alone is worth 2e-2 of max |dA| on this input (1.7e-3 with an
+    fp32 dM), hence its own bar."""
     _say("extreme decay")
     d = _problem(1, 192, 2, 32, 64, 1, seed=21, softplus=False)
     g = torch.Generator().manual_seed(22)
@@ -809,7 +816,7 @@ def test_extreme_decay_is_finite_and_accurate():
     _check("final_states", fin, fin_ref, 1e-3)
     for k in GRAD_NAMES:
         if d[k] is not None:
-            _check("d" + k, gr[k], g_ref[k], 1e-2 if k in ("dt", "A") else 1e-3)
+            _check("d" + k, gr[k], g_ref[k], 5e-2 if k == "A" else 1e-2 if k == "dt" else 1e-3)
 
 
 def test_hip_graph_replays_match_eager():
