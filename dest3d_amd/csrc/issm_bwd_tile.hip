@@ -406,7 +406,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
     }
 
     // ---- the rest of the column phase: suffix sums over the rows, ddt, the partial sums
-    dcs[15] += g4 == 3 ? gl_keep : 0.0f;
+    // (fresh opaque lane coordinates: the cross-lane fetch addresses are formed here rather than kept across the loop and
+    // reloaded from scratch behind the requests in flight)
+    int cm2 = cm, g42 = g4;
+    asm volatile("" : "+v"(cm2), "+v"(g42));
+    dcs[15] += g42 == 3 ? gl_keep : 0.0f;
     {
       // suffix sums up the 64 rows; the cross-lane steps of the four tiles are issued together
       float c[4], v[4], t[4];
@@ -423,13 +427,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
 #pragma unroll
       for (int J = 0; J < 4; ++J) t[J] = __shfl_down(c[J], 16, 64);
 #pragma unroll
-      for (int J = 0; J < 4; ++J) v[J] = g4 <= 2 ? c[J] + t[J] : c[J];
+      for (int J = 0; J < 4; ++J) v[J] = g42 <= 2 ? c[J] + t[J] : c[J];
 #pragma unroll
       for (int J = 0; J < 4; ++J) t[J] = __shfl_down(v[J], 32, 64);
 #pragma unroll
-      for (int J = 0; J < 4; ++J) v[J] = g4 <= 1 ? v[J] + t[J] : v[J];  // inclusive from the last lane group down
+      for (int J = 0; J < 4; ++J) v[J] = g42 <= 1 ? v[J] + t[J] : v[J];  // inclusive from the last lane group down
 #pragma unroll
-      for (int J = 0; J < 4; ++J) t[J] = __shfl(v[J], cm, 64);           // tile totals
+      for (int J = 0; J < 4; ++J) t[J] = __shfl(v[J], cm2, 64);           // tile totals
       float carry = 0.0f;  // sum over all rows after the current tile
 #pragma unroll
       for (int J = 3; J >= 0; --J) {
@@ -455,8 +459,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
     sumA = scan_g_incl(sumA, g4);
     sumB = scan_g_incl(sumB, g4);
     if (g4 == 3) {
-      partA[vec_off(p, u.bt, u.c, u.h) + n] = sumA;
-      partBias[vec_off(p, u.bt, u.c, u.h) + n] = sumB;
+      // (an opaque copy of the column: the two per-lane addresses are then formed here instead of being kept, as 64-bit
+      // values, across the head loop -- a reload from scratch at this point would wait for every request in flight)
+      int nq = n;
+      asm volatile("" : "+v"(nq));
+      partA[vec_off(p, u.bt, u.c, u.h) + nq] = sumA;
+      partBias[vec_off(p, u.bt, u.c, u.h) + nq] = sumB;
     }
   }
 

@@ -421,6 +421,73 @@ def test_biscan_matches_two_flipped_scans_and_oracle():
     assert torch.equal(fl(y2), o[1]) and torch.equal(l2, o[3])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_heads_outside_the_tile_kernel_range_are_redone_by_the_level_kernel(dtype):
+    """Complete tiles, both directions, four heads in two groups: head 1 decays by far more than 2^96 per 16 rows
+    everywhere, head 3 only inside one stretch of tokens, heads 0 and 2 nowhere.  The chunk backward then runs partly in
+    the tile-base kernel and partly in the level-hierarchy kernel -- per (workgroup, head), in either direction or both
+    -- and the two write one ddt / dB / dC together; everything against the fp64 oracle, and the marks themselves
+    through the stage entry point."""
+    from dest3d_amd import ISSM_biscan_combined
+    _say(f"heads in and out of the tile kernel's range, {dtype}")
+    Bsz, L_, H, P, N, G = 2, 192, 4, 32, 128, 2
+    d = _problem(Bsz, L_, H, P, N, G, seed=61, softplus=False)
+    d["dt"] = d["dt"].abs()
+    d["A"][1] = -80.0 * (1.0 + torch.rand(N, generator=torch.Generator().manual_seed(1)))
+    d["dt"][:, 70:110, 3] *= 80.0
+    g = torch.Generator().manual_seed(62)
+    d["x_b"] = torch.randn(d["x"].shape, generator=g)
+    d["B_b"] = torch.randn(d["B"].shape, generator=g) / math.sqrt(N)
+    d["C_b"] = torch.randn(d["C"].shape, generator=g) / math.sqrt(N)
+    dy_b = torch.randn(d["x"].shape, generator=g)
+    dl_b = torch.randn(d["h0"].shape, generator=g)
+    io = ("x", "x_b", "dt", "B", "B_b", "C", "C_b")
+    names = list(io) + ["A", "D", "h0"]
+    q = {k: (d[k].to(dtype).float() if k in io else d[k]) for k in names}     # what the kernels are handed
+    ref_in = {k: q[k].double().clone().requires_grad_() for k in names}
+    yf, yb, lf, lb = R.issm_biscan_ref(ref_in["x"], ref_in["x_b"], ref_in["dt"], ref_in["A"], ref_in["B"],
+                                       ref_in["B_b"], ref_in["C"], ref_in["C_b"], D=ref_in["D"],
+                                       initial_states=ref_in["h0"])
+    ((yf * d["dy"].double()).sum() + (yb * dy_b.double()).sum() + (lf * d["dfinal"].double()).sum()
+     + (lb * dl_b.double()).sum()).backward()
+    dev = "cuda"
+    gi = {k: q[k].to(dev, dtype if k in io else torch.float32).requires_grad_() for k in names}
+    o = ISSM_biscan_combined(gi["x"], gi["x_b"], gi["dt"], gi["A"], gi["B"], gi["B_b"], gi["C"], gi["C_b"], 64,
+                             D=gi["D"], initial_states=gi["h0"])
+    ((o[0].float() * d["dy"].to(dev)).sum() + (o[1].float() * dy_b.to(dev)).sum() + (o[2] * d["dfinal"].to(dev)).sum()
+     + (o[3] * dl_b.to(dev)).sum()).backward()
+    torch.cuda.synchronize()
+    # (fp32 bars as in test_extreme_decay_is_finite_and_accurate: running sums in the thousands cost fp32 exponent bits)
+    fwd, bwd = (1e-3, 1e-2) if dtype == torch.float32 else (2e-2, 5e-2)
+    for name, a, b in zip(("y_f", "y_b", "last_f", "last_b"), o, (yf, yb, lf, lb)):
+        _check(name, a, b, fwd)
+    for k in names:
+        _check("d" + k, gi[k].grad, ref_in[k].grad, 5e-2 if k == "A" else bwd)
+    # the marks: one direction through the stage entry point, on intermediates of the right shapes
+    if dtype == torch.float32:
+        dd = dict(d, z=None, dt_bias=None)
+        L, prob, a = _stage_args(dd)
+        lib = L.load()
+        nc = L_ // 64
+        f = lambda *s_: torch.zeros(s_, device=dev)
+        states, dst, dm, gn = f(Bsz, nc + 1, H, P, N), f(Bsz, nc, H, P, N), f(Bsz, nc, H, 64, 64), f(Bsz, nc, H, N)
+        ddt, dB, dC = f(Bsz, L_, H, N), f(Bsz, L_, G, N), f(Bsz, L_, G, N)
+        pa, pb = f(Bsz * nc, H, N), f(Bsz * nc, H, N)
+        dyd = d["dy"].to(dev)
+        a.dout[0] = L.tensor_desc(dyd)
+        a.ddt, a.dB[0], a.dC[0] = (L.tensor_desc(t) for t in (ddt, dB, dC))
+        redo = torch.full((lib.issm_bwd_chunk_redo_ints(C.byref(a)),), -1, dtype=torch.int32, device=dev)
+        L.check(lib.issm_stage_bwd_chunk(C.byref(a), 0, None, states.data_ptr(), dst.data_ptr(), dm.data_ptr(),
+                                         gn.data_ptr(), pa.data_ptr(), pb.data_ptr(), redo.data_ptr()), "bwd_chunk")
+        torch.cuda.synchronize()
+        marks = redo.view(Bsz, nc, G, N // 64, H // G).cpu()      # (batch, chunk, group, slice, head of the group)
+        assert set(marks.unique().tolist()) == {0, 1}
+        assert bool((marks[..., 0] == 0).all()), "heads 0 and 2 stay in the tile-base kernel"
+        assert bool((marks[:, :, 0, :, 1] == 1).all()), "head 1 is out of range everywhere"
+        assert bool((marks[:, 1, 1, :, 1] == 1).all()) and bool((marks[:, 0, 1, :, 1] == 0).all()), \
+            "head 3 is out of range only in the chunk that holds tokens 70..109"
+
+
 def _stage_args(d, ndir=1):
     """ScanArgs + device tensors for direct stage calls (single direction, fp32)."""
     from dest3d_amd import _lib as L
