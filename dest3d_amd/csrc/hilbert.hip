@@ -40,6 +40,15 @@ __device__ __forceinline__ long hilbert3(unsigned x0, unsigned x1, unsigned x2, 
   return h;
 }
 
+// Cell index of a truncated quotient: [0, cap], with NaN (a NaN coordinate, or Inf - Inf) sent to cell 0 by an explicit
+// test instead of reaching the float-to-int conversion, whose result for NaN is not defined.
+__device__ __forceinline__ unsigned cell_index(float v, int cap) {
+  return v >= (float)cap ? (unsigned)cap : (v > 0.0f ? (unsigned)(int)v : 0u);
+}
+// Minimum that keeps a NaN once seen, as torch.amin does (fminf would drop it): a sample with a NaN coordinate then
+// gets the same corner, and so the same cells, from the one-workgroup kernel and from the host-side reduction.
+__device__ __forceinline__ float min_keep_nan(float a, float b) { return a != a ? a : (b != b ? b : fminf(a, b)); }
+
 __global__ __launch_bounds__(NTHREADS) void k_hilbert_codes(HilbertP p) {
   const long id = (long)blockIdx.x * NTHREADS + threadIdx.x;
   if (id >= (long)p.B * p.N) return;
@@ -53,9 +62,7 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_codes(HilbertP p) {
     // a correctly rounded division, as torch.div(..., rounding_mode="trunc") performs on the host: this file is built
     // without fast-math, which would turn it into a multiplication by an approximate reciprocal and move points that
     // sit exactly on a cell boundary into the neighbouring cell
-    const float v = truncf((q[i] - mn[i]) / p.cell);
-    int c = v >= (float)cap ? cap : (int)v;
-    g[i] = (unsigned)(c < 0 ? 0 : c);
+    g[i] = cell_index(truncf((q[i] - mn[i]) / p.cell), cap);
   }
   p.codes[id] = hilbert3(g[p.perm[0]], g[p.perm[1]], g[p.perm[2]], p.bits);
 }
@@ -77,12 +84,12 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_order(HilbertOrderP p) {
   float mn[3] = {INFINITY, INFINITY, INFINITY};
   for (int j = tid; j < p.N; j += NTHREADS) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) mn[i] = fminf(mn[i], pts[3 * j + i]);
+    for (int i = 0; i < 3; ++i) mn[i] = min_keep_nan(mn[i], pts[3 * j + i]);
   }
 #pragma unroll
   for (int i = 0; i < 3; ++i) {
 #pragma unroll
-    for (int d = 32; d > 0; d >>= 1) mn[i] = fminf(mn[i], __shfl_xor(mn[i], d, 64));
+    for (int d = 32; d > 0; d >>= 1) mn[i] = min_keep_nan(mn[i], __shfl_xor(mn[i], d, 64));
     if ((tid & 63) == 0) red[i][tid >> 6] = mn[i];
   }
   __syncthreads();
@@ -90,7 +97,7 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_order(HilbertOrderP p) {
   for (int i = 0; i < 3; ++i) {
     mn[i] = red[i][0];
 #pragma unroll
-    for (int w = 1; w < NTHREADS / 64; ++w) mn[i] = fminf(mn[i], red[i][w]);
+    for (int w = 1; w < NTHREADS / 64; ++w) mn[i] = min_keep_nan(mn[i], red[i][w]);
   }
   const int cap = (1 << p.bits) - 1;
   const int p0 = p.perm[o][0], p1 = p.perm[o][1], p2 = p.perm[o][2];
@@ -100,9 +107,7 @@ __global__ __launch_bounds__(NTHREADS) void k_hilbert_order(HilbertOrderP p) {
       unsigned g[3];
 #pragma unroll
       for (int i = 0; i < 3; ++i) {
-        const float v = truncf((pts[3 * j + i] - mn[i]) / p.cell);  // the same correctly rounded division as above
-        int c = v >= (float)cap ? cap : (int)v;
-        g[i] = (unsigned)(c < 0 ? 0 : c);
+        g[i] = cell_index(truncf((pts[3 * j + i] - mn[i]) / p.cell), cap);  // the same correctly rounded division as above
       }
       key = ((unsigned long long)hilbert3(g[p0], g[p1], g[p2], p.bits) << HO_IDXBITS) | (unsigned)j;
     }

@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "../../include/issm.h"
@@ -235,6 +236,8 @@ static int launched(int hip_err, const char* what) {
   return fail(ISSM_E_LAUNCH, "%s: %s", what, hipGetErrorString((hipError_t)hip_err));
 }
 
+static void norm_scratch_warm(hipStream_t stream);  // further down, with the allocation-free backward it serves
+
 extern "C" {
 
 int issm_abi_version(void) { return ISSM_ABI_VERSION; }
@@ -450,8 +453,9 @@ static int norm_params(const issm_norm_args* a, NormP* p, bool bwd) {
   if (bwd && a->z && !a->dz) return fail(ISSM_E_NULL, "rmsnorm bwd: dz is NULL");
   if (a->layer_norm && !a->mean) return fail(ISSM_E_NULL, "layernorm: mean is NULL");
   if (bwd && a->bias && (!a->db_partial || !a->db)) return fail(ISSM_E_NULL, "norm bwd with bias: db_partial/db is NULL");
-  if (a->bias && a->ncols > 8192 && !(a->ncols / gs == 1 && (a->ncols & 3) == 0 && a->ncols <= 1024))
-    return fail(ISSM_E_UNSUPPORTED, "norm with bias: ncols %d > 8192", a->ncols);
+  // only the backward stages the bias partial sums next to the weight's in LDS; the forward has no such limit
+  if (bwd && a->bias && a->ncols > 8192 && !(a->ncols / gs == 1 && (a->ncols & 3) == 0 && a->ncols <= 1024))
+    return fail(ISSM_E_UNSUPPORTED, "norm bwd with bias: ncols %d > 8192", a->ncols);
   p->rows = a->rows; p->ncols = a->ncols; p->gs = gs; p->ngroups = a->ncols / gs;
   p->dt = a->dtype; p->wdt = a->weight_dtype; p->nbg = a->norm_before_gate; p->eps = a->eps;
   p->x = a->x; p->z = a->z; p->w = a->w; p->xs = a->x_row_stride; p->zs = a->z_row_stride;
@@ -467,6 +471,7 @@ int issm_gated_rmsnorm_fwd(const issm_norm_args* a) {
   NormP p;
   int rc = norm_params(a, &p, false);
   if (rc) return rc;
+  norm_scratch_warm((hipStream_t)a->stream);
   return launched(launch_rmsnorm_fwd(p, (hipStream_t)a->stream), "rmsnorm_fwd");
 }
 
@@ -474,6 +479,7 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* a) {
   NormP p;
   int rc = norm_params(a, &p, true);
   if (rc) return rc;
+  norm_scratch_warm((hipStream_t)a->stream);
   return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd");
 }
 
@@ -491,22 +497,50 @@ static __device__ __align__(256) float g_norm_scratch[ISSM_NORM_SCRATCH_FLOATS];
 static constexpr int kMaxDevices = 64;
 static std::mutex g_norm_scratch_mutex;
 static float* g_norm_scratch_ptr[kMaxDevices];  // [device]: address of that device's copy, once looked up
+static std::atomic<bool> g_norm_scratch_known[kMaxDevices];  // set after the pointer: a cheap test for norm_scratch_warm
 
-static int norm_scratch_ptr(float** out) {
+// The look-up may load the code object and so must not run while `stream` records a graph: a first call on a device
+// that arrives under capture is refused (one eager call per device, of this entry point or of any other of the
+// library's normalisation calls, comes first -- those resolve the address on the way, see norm_scratch_warm).
+static int norm_scratch_ptr(float** out, hipStream_t stream) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(ISSM_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
   if (dev < 0 || dev >= kMaxDevices) return fail(ISSM_E_UNSUPPORTED, "device index %d outside 0..%d", dev, kMaxDevices - 1);
   std::lock_guard<std::mutex> lock(g_norm_scratch_mutex);
   if (!g_norm_scratch_ptr[dev]) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(ISSM_E_UNSUPPORTED,
+                  "rmsnorm bwd without allocation: the first call on device %d came while its stream records a graph; "
+                  "make one eager call of a normalisation entry point on this device before the capture", dev);
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_norm_scratch));  // of the current device's copy
     if (e != hipSuccess || !ptr)
       return fail(ISSM_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
     g_norm_scratch_ptr[dev] = (float*)ptr;
+    g_norm_scratch_known[dev].store(true, std::memory_order_release);
   }
   *out = g_norm_scratch_ptr[dev];
   return ISSM_OK;
+}
+// Called by the other normalisation entry points: resolves the current device's address when that is possible now
+// (not under capture), silently otherwise, so that a model whose forward ran eagerly once can capture the
+// allocation-free backward without a warm-up call of its own.
+static void norm_scratch_warm(hipStream_t stream) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return;
+  }
+  if (g_norm_scratch_known[dev].load(std::memory_order_acquire)) return;
+  float* unused = nullptr;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return;
+  }
+  if (norm_scratch_ptr(&unused, stream) != ISSM_OK) g_err[0] = 0;
 }
 
 extern "C" {
@@ -530,7 +564,7 @@ int issm_gated_rmsnorm_bwd_noalloc(const issm_norm_args* a) {
   NormP p;
   int rc = norm_params(&b, &p, true);
   if (rc) return rc;
-  if ((rc = norm_scratch_ptr(&scratch))) return rc;
+  if ((rc = norm_scratch_ptr(&scratch, (hipStream_t)a->stream))) return rc;
   p.dw_partial = scratch;  // every launched block writes its whole row of partials before the sum reads it
   p.db_partial = scratch + part;
   return launched(launch_rmsnorm_bwd(p, (hipStream_t)a->stream), "rmsnorm_bwd_noalloc");

@@ -497,7 +497,7 @@ __device__ __forceinline__ float scan_g_incl_rev(float v, int g4) {
 struct RowMap {
   int base, step, nvalid;
   bool full;
-  unsigned long long cut;  // bit r: the sequence id changes between rows r - 1 and r of the chunk (scan order); uniform
+  unsigned long long cut;  // bit r: the sequence id changes between rows r - 1 and r of the chunk (scan order; the initial states count as id 0); uniform
 };
 template <bool FULL>
 __device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4, int n0) {
@@ -512,11 +512,13 @@ __device__ __forceinline__ RowMap make_rowmap(const KP& p, const Unit& u, int g4
   if (!FULL && p.seq_idx) {  // packed sequences take the kernels' general variants
     // lane = row of the chunk in scan order; its predecessor in scan order may be the previous chunk's last row
     const int row = u.c * CS + (int)(threadIdx.x & 63);
+    // The initial states belong to sequence id 0 (issm_chunk_scan.py:123 and issm_state_passing.py:91 start from id 0):
+    // a row whose first id is not 0 is cut off from them, like a row from a predecessor of another id.
     bool changes = false;
-    if (row > 0 && row < p.L) {
+    if (row < p.L) {
       const long t = u.dir ? p.L - 1 - row : row, tp = u.dir ? t + 1 : t - 1;
       const int* q = p.seq_idx + (long)u.b * p.seq_s0;
-      changes = q[t * p.seq_s1] != q[tp * p.seq_s1];
+      changes = q[t * p.seq_s1] != (row > 0 ? q[tp * p.seq_s1] : 0);
     }
     r.cut = __ballot(changes);
   }

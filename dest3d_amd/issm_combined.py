@@ -248,7 +248,10 @@ def ISSM_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias
         z: (batch, seqlen, nheads, headdim)
         dt_bias: (nheads, dstate)
         initial_states: (batch, nheads, headdim, dstate)
-        seq_idx: (batch, seqlen) integer ids of the sequences packed into a row, or None
+        seq_idx: (batch, seqlen) integer ids of the sequences packed into a row, or None.  The ids of a row must
+            not decrease.  initial_states count as id 0 (issm_chunk_scan.py:123): they feed the first sequence of a
+            row whose ids start at 0 and nothing in a row whose ids start higher.  Every change of id is a cut
+            (the reference's equality masks would reconnect a repeated id inside a chunk only; not reproduced).
         dt_softplus: whether to apply softplus to dt (+ dt_bias)
     Return:
         out: (batch, seqlen, nheads, headdim)  [, final_states (batch, nheads, headdim, dstate) fp32]

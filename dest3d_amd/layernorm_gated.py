@@ -53,12 +53,16 @@ class LayerNormFn(torch.autograd.Function):
             z2 = _rows(z.detach().to(kdt))
         w = weight.detach()
         w = w if w.dtype in (torch.float32, torch.bfloat16) else w.float()
-        w = w.contiguous()
         assert w.shape == (shape[-1],)
         b = None
         if bias is not None:
             assert bias.shape == (shape[-1],)
-            b = bias.detach().to(w.dtype).contiguous()   # the kernels read weight and bias in one dtype
+            # The kernels read weight and bias in one dtype, the reference's widen each to fp32 on its own
+            # (layernorm_gated.py:77-80): where the two differ both go to fp32, so that neither is rounded.
+            if bias.dtype != w.dtype:
+                w = w.float()
+            b = bias.detach().to(w.dtype).contiguous()
+        w = w.contiguous()
         gs = shape[-1] if group_size is None else group_size
         assert shape[-1] % gs == 0
         with torch.cuda.device(x.device):

@@ -131,7 +131,12 @@ typedef struct issm_scan_args {
    * set.  Tokens of a batch row whose values differ belong to different sequences packed into that row, and no
    * state passes from one to the next: wherever seq_idx changes from a token to its successor the running sum of
    * dt'.A takes an extra -128 ln 2, i.e. every decay across the change is multiplied by 2^-128 (3e-39: zero at fp32
-   * resolution, where the reference's kernels multiply by an exact 0).  The backward must be given the same array. */
+   * resolution, where the reference's kernels multiply by an exact 0).  The backward must be given the same array.
+   * Contract: the ids of a row must not decrease.  The initial states count as id 0, as in the reference
+   * (issm_chunk_scan.py:123 takes 0 as the id before the first chunk, issm_state_passing.py:91 starts from 0): they
+   * feed the first sequence of a row whose ids start at 0 and nothing in a row whose ids start higher (dh0 of that
+   * row is then 0).  Ids that decrease are not rejected; the reference's equality masks would reconnect equal ids
+   * inside a chunk but not across chunks, and that mix is not reproduced: here every change of id is a cut. */
   const int32_t* seq_idx;
   int64_t seq_idx_stride[2]; /* element strides of (batch, seqlen) */
 } issm_scan_args;
@@ -277,7 +282,11 @@ int issm_gated_rmsnorm_bwd(const issm_norm_args* args);
  * up to 512 columns always fit).  The function calls no
  * hipMalloc / hipFree or other allocating routine.  All calls on one GPU share that GPU's array: two calls that
  * overlap in time on one GPU (different streams or host threads) race; calls on one stream are ordered and safe.
- * Nothing in the array has to be cleared between calls (every partial that is read was written by the same call). */
+ * Nothing in the array has to be cleared between calls (every partial that is read was written by the same call).
+ * The array's device address is looked up once per device, on the first eager call there of this function or of
+ * issm_gated_rmsnorm_fwd / issm_gated_rmsnorm_bwd; that look-up may load code and is kept out of graph capture: if the
+ * very first normalisation call on a device arrives while args->stream is recording, this function returns
+ * ISSM_E_UNSUPPORTED and launches nothing.  Make one eager call per device before capturing. */
 #define ISSM_NORM_SCRATCH_FLOATS (2048 * 1024)
 int issm_gated_rmsnorm_bwd_noalloc(const issm_norm_args* args);
 

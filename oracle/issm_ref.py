@@ -96,7 +96,11 @@ def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
     seq_idx (B,L), optional: ids of the sequences packed into a row (issm_combined.py:29).  Where the id changes
     from one token to the next no state is carried over -- what the reference's kernels obtain by zeroing every
     decay between tokens of different ids (issm_chunk_state.py, issm_state_passing.py, issm_chunk_scan.py and
-    issm_cabt_bmm.py:14 under HAS_SEQ_IDX).
+    issm_cabt_bmm.py:14 under HAS_SEQ_IDX).  The initial states count as id 0 (issm_chunk_scan.py:123 loads 0 as the id
+    before the first chunk, issm_state_passing.py:91 starts from 0): a row whose ids start above 0 never sees them.
+    Ids must not decrease along a row: the reference's kernels compare ids by equality, so a later token with an
+    earlier id would be reconnected inside a chunk (issm_cabt_bmm.py:146-148) but not across chunks; that mix is not
+    restated here and the HIP path rejects nothing but documents the same contract.
 
     Returns (out (B,L,H,P), final_states (B,H,P,N)).
     """
@@ -116,8 +120,9 @@ def issm_scan_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None,
     dts, Bs, Cs, xs = dtp.unbind(1), Bh.unbind(1), Ch.unbind(1), x_.unbind(1)
     for t in range(L):
         decay = torch.exp(dts[t] * A_[None])                          # (B,H,N)
-        if seq_idx is not None and t > 0:
-            decay = decay * (seq_idx[:, t] == seq_idx[:, t - 1]).to(dtype)[:, None, None]
+        if seq_idx is not None:
+            prev = seq_idx[:, t - 1] if t > 0 else torch.zeros_like(seq_idx[:, 0])   # initial states carry id 0
+            decay = decay * (seq_idx[:, t] == prev).to(dtype)[:, None, None]
         inject = (dts[t] * Bs[t])[:, :, None, :] * xs[t][..., None]
         h = decay[:, :, None, :] * h + inject
         ys.append(torch.einsum("bhpn,bhn->bhp", h, Cs[t]))

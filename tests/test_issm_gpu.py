@@ -171,18 +171,22 @@ def _seq_ids(Bsz, L, cuts):
     return s
 
 
+@pytest.mark.parametrize("first_id", [0, 1])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_packed_sequences_match_oracle(dtype):
+def test_packed_sequences_match_oracle(dtype, first_id):
     """seq_idx (issm_combined.py:29): several sequences packed into a batch row; no state crosses a change of id.
     Changes inside a chunk, at a chunk's first row, at its last row, in adjacent rows and in the ragged last chunk;
-    row 1 of the batch has no change at all.  Every gradient against the oracle's recurrence with resets."""
-    _say(f"operator with seq_idx {dtype}")
+    row 1 of the batch has no change at all.  Every gradient against the oracle's recurrence with resets.
+    first_id = 1: the ids of batch row 0 start at 1, so its initial states (which count as id 0,
+    issm_chunk_scan.py:123) reach no token and receive a zero gradient; batch row 1 still starts at 0."""
+    _say(f"operator with seq_idx {dtype} first id {first_id}")
     L_ = 64 * 3 + 21
     d = _problem(2, L_, 2, 32, 96, 1, seed=77, D="h", z=True)
     if dtype == torch.bfloat16:
         for k in ("x", "dt", "B", "C", "z"):
             d[k] = d[k].bfloat16().float()
     seq = _seq_ids(2, L_, [[5, 40, 41, 64, 127, 130, 200], []])
+    seq[0] += first_id
     ins = {k: d[k].double().clone().requires_grad_() for k in GRAD_NAMES if d[k] is not None}
     y_ref, fin_ref = R.issm_scan_sequential(ins["x"], ins["dt"], ins["A"], ins["B"], ins["C"], D=ins["D"], z=ins["z"],
                                             dt_bias=ins["dt_bias"], initial_states=ins["h0"],
@@ -204,6 +208,9 @@ def test_packed_sequences_match_oracle(dtype):
     for k in GRAD_NAMES:
         if d[k] is not None:
             _check("d" + k, g[k].grad, ins[k].grad, bt)
+    if first_id:
+        # the kernels multiply a decay across a change of id by 2^-128 where the reference multiplies by 0
+        assert ins["h0"].grad[0].abs().max() == 0 and g["h0"].grad[0].abs().max() < 1e-30
 
 
 def test_dt_already_clamped_by_an_fp32_caller_keeps_its_gradient():
@@ -667,6 +674,35 @@ def test_properties_at_benchmark_shape():
     _check("final[0]", fg, fr, FWD32)
     for k in ins:
         _check("d" + k, gi[k].grad, ins[k].grad, BWD32)
+
+
+def test_forward_only_at_the_cpu_runnable_configuration():
+    """The reference's own CPU-runnable case on the GPU: forward only, fp32, B=2, L=1024, H=8, P=32, N=256, G=1, the
+    chunk size 64, dt through softplus with dt_bias inside the
+    kernels, zero initial states, no autograd graph.  Both batch elements are checked against the sequential fp64 oracle
+    and against the chunked restatement of the reference's formulation (oracle/issm_ref.py: issm_scan_chunked)."""
+    from dest3d_amd import ISSM_chunk_scan_combined as op
+    _say("config0 forward only B=2")
+    I = R.make_inputs(2, 1024, 8, 32, 256, seed=77)
+    dev = "cuda"
+    t = {k: v.to(dev) for k, v in I.items()}
+    bias = I["dt_bias"]
+    h0 = torch.zeros(2, 8, 32, 256)
+    with torch.no_grad():
+        y, fin = op(t["x"], t["dt_raw"], t["A"], t["B"], t["C"], 64, D=t["D"], dt_bias=bias.to(dev),
+                    initial_states=h0.to(dev), dt_softplus=True, return_final_states=True)
+        torch.cuda.synchronize()
+    assert not y.requires_grad and y.dtype == torch.float32
+    dbl = {k: v.double() for k, v in I.items()}
+    yr, fr = R.issm_scan_sequential(dbl["x"], dbl["dt_raw"], dbl["A"], dbl["B"], dbl["C"], D=dbl["D"],
+                                    dt_bias=bias.double(), initial_states=h0.double(), dt_softplus=True)
+    _check("y", y, yr, FWD32)
+    _check("final", fin, fr, FWD32)
+    yc, fc = R.issm_scan_chunked(dbl["x"], R.dt_transform(dbl["dt_raw"], bias.double(), True), dbl["A"], dbl["B"],
+                                 dbl["C"], 64, initial_states=h0.double())
+    yc = yc + dbl["D"][None, None, :, None] * dbl["x"]
+    _check("y vs chunked", y, yc, FWD32)
+    _check("final vs chunked", fin, fc, FWD32)
 
 
 def test_benchmark_shape_bf16_bidirectional():

@@ -287,9 +287,11 @@ def test_layernorm_form_against_the_library_routines():
     torch.testing.assert_close(R.gated_rmsnorm_ref(x, w, bias=b), R.gated_rmsnorm_ref(x, w) + b, rtol=1e-13, atol=1e-13)
 
 
-def test_packed_sequences_are_independent_runs():
-    """seq_idx: a row that packs three sequences gives, segment by segment, what three separate runs give (the later
-    ones without an initial state) -- outputs, final state and gradients; ids need not start at zero."""
+@pytest.mark.parametrize("first_id", [0, 4])
+def test_packed_sequences_are_independent_runs(first_id):
+    """seq_idx: a row that packs three sequences gives, segment by segment, what three separate runs give -- outputs,
+    final state and gradients.  The initial states count as id 0 (issm_chunk_scan.py:123, issm_state_passing.py:91):
+    they feed the first sequence when its id is 0 and nothing when the ids start higher."""
     torch.manual_seed(3)
     Bsz, L, H, P, N = 1, 11, 2, 3, 4
     x = torch.randn(Bsz, L, H, P, dtype=torch.float64, requires_grad=True)
@@ -297,23 +299,58 @@ def test_packed_sequences_are_independent_runs():
     A = -torch.rand(H, N, dtype=torch.float64) * 3
     Bm = torch.randn(Bsz, L, 1, N, dtype=torch.float64)
     Cm = torch.randn(Bsz, L, 1, N, dtype=torch.float64)
-    h0 = torch.randn(Bsz, H, P, N, dtype=torch.float64)
-    seq = torch.tensor([[4, 4, 4, 7, 7, 7, 7, 7, 9, 9, 9]])
+    h0 = torch.randn(Bsz, H, P, N, dtype=torch.float64, requires_grad=True)
+    seq = torch.tensor([[0, 0, 0, 3, 3, 3, 3, 3, 5, 5, 5]]) + first_id
     y, fin = R.issm_scan_sequential(x, dt, A, Bm, Cm, initial_states=h0, seq_idx=seq)
     w = torch.randn_like(y)
-    gx, gdt = torch.autograd.grad((y * w).sum() + fin.sum(), (x, dt))
+    gx, gdt, gh0 = torch.autograd.grad((y * w).sum() + fin.sum(), (x, dt, h0))
     ys, gxs, gdts = [], [], []
     for lo, hi in ((0, 3), (3, 8), (8, 11)):
         xs = x.detach()[:, lo:hi].clone().requires_grad_()
         dts = dt.detach()[:, lo:hi].clone().requires_grad_()
-        yi, fi = R.issm_scan_sequential(xs, dts, A, Bm[:, lo:hi], Cm[:, lo:hi], initial_states=h0 if lo == 0 else None)
+        h0s = h0.detach().clone().requires_grad_()
+        yi, fi = R.issm_scan_sequential(xs, dts, A, Bm[:, lo:hi], Cm[:, lo:hi],
+                                        initial_states=h0s if lo == 0 and first_id == 0 else None)
         loss = (yi * w[:, lo:hi]).sum() + (fi.sum() if hi == L else 0.0)
-        a, b = torch.autograd.grad(loss, (xs, dts))
+        a, b = torch.autograd.grad(loss, (xs, dts), retain_graph=True)
+        if lo == 0:
+            gh0s = torch.autograd.grad(loss, h0s)[0] if first_id == 0 else torch.zeros_like(h0)
         ys.append(yi.detach()); gxs.append(a); gdts.append(b)
     torch.testing.assert_close(y.detach(), torch.cat(ys, 1), rtol=1e-12, atol=1e-12)
     torch.testing.assert_close(fin.detach(), fi.detach(), rtol=1e-12, atol=1e-12)
     torch.testing.assert_close(gx, torch.cat(gxs, 1), rtol=1e-12, atol=1e-12)
     torch.testing.assert_close(gdt, torch.cat(gdts, 1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(gh0, gh0s, rtol=1e-12, atol=1e-12)
+
+
+def test_packed_sequences_match_the_id_equality_masks_of_the_reference_kernels():
+    """The reference has no reset: each of its kernels multiplies a decay by [id == id'] -- token pairs inside a chunk
+    (issm_cabt_bmm.py:146-148), a token against the id before its chunk for the incoming state, with 0 before the first
+    chunk (issm_chunk_scan.py:123,133), and chunk ends against each other in the state passing (issm_state_passing.py:
+    91-99).  For ids that never decrease all of these say "same sequence", so  y_l = sum_{s<=l} [id_l == id_s] C_l
+    decay(l,s) dt_s B_s x_s + [id_l == 0 == every id before l] C_l decay(l,-1) h0,  evaluated here pair by pair."""
+    torch.manual_seed(5)
+    L, P, N = 9, 2, 3
+    x = torch.randn(1, L, 1, P, dtype=torch.float64)
+    dt = torch.rand(1, L, 1, N, dtype=torch.float64) * 0.5
+    A = -torch.rand(1, N, dtype=torch.float64) * 2
+    Bm = torch.randn(1, L, 1, N, dtype=torch.float64)
+    Cm = torch.randn(1, L, 1, N, dtype=torch.float64)
+    h0 = torch.randn(1, 1, P, N, dtype=torch.float64)
+    for ids in ([0, 0, 0, 1, 1, 2, 2, 2, 2], [1, 1, 1, 1, 2, 2, 2, 3, 3], [0] * 9, [2] * 9):
+        y, _ = R.issm_scan_sequential(x, dt, A, Bm, Cm, initial_states=h0, seq_idx=torch.tensor([ids]))
+        a = dt[0, :, 0] * A[0]                                       # (L, N)
+        for l in range(L):
+            for p_ in range(P):
+                acc = 0.0
+                for n in range(N):
+                    for s_ in range(l + 1):
+                        if ids[l] == ids[s_]:
+                            acc += (Cm[0, l, 0, n] * torch.exp(a[s_ + 1:l + 1, n].sum()) * dt[0, s_, 0, n]
+                                    * Bm[0, s_, 0, n] * x[0, s_, 0, p_]).item()
+                    if ids[l] == 0:
+                        acc += (Cm[0, l, 0, n] * torch.exp(a[:l + 1, n].sum()) * h0[0, 0, p_, n]).item()
+                assert abs(acc - y[0, l, 0, p_].item()) < 1e-12, (ids, l, p_)
 
 
 def test_make_inputs_is_deterministic_and_in_range():

@@ -86,6 +86,36 @@ def test_gated_layernorm_and_bias_fwd_bwd(shape, gs, nbg, use_z, rms, use_b, dty
         _check("dz", zg.grad, zr.grad, bt)
 
 
+def test_bias_in_another_dtype_than_the_weight_is_not_rounded():
+    """A bf16 weight with an fp32 bias (layernorm_gated.py:77-80 widens each to fp32 on its own): the bias must enter
+    with all its fp32 bits.  The bias here is 1 + 2^-12 per column, which bf16 would round to 1; x = 0 and no gate make
+    the output the bias itself."""
+    from dest3d_amd import layernorm_fn
+    _say("layernorm bf16 weight, fp32 bias")
+    x = torch.zeros(4, 256, device="cuda")
+    w = torch.ones(256, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    b = torch.full((256,), 1.0 + 2.0 ** -12, device="cuda", requires_grad=True)
+    y = layernorm_fn(x, w, b, None, 1e-5, None, True, False)
+    assert torch.equal(y, b.detach().expand(4, 256))
+    y.sum().backward()
+    assert w.grad.dtype == torch.bfloat16 and b.grad.dtype == torch.float32
+    assert torch.equal(b.grad, torch.full((256,), 4.0, device="cuda"))
+
+
+def test_forward_with_a_bias_has_no_column_limit_of_the_backward():
+    """9000 columns with a bias: the forward runs (it stages nothing in LDS); only a backward would be refused."""
+    from dest3d_amd import layernorm_fn
+    _say("layernorm forward 9000 columns with bias")
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 9000, generator=g)
+    w = torch.randn(9000, generator=g)
+    b = torch.randn(9000, generator=g)
+    with torch.no_grad():
+        y = layernorm_fn(x.cuda(), w.cuda(), b.cuda(), None, 1e-5, None, True, False)
+    ref = torch.nn.functional.layer_norm(x.double(), (9000,), w.double(), b.double(), 1e-5)
+    _check("y", y, ref, FWD32)
+
+
 def test_layernorm_module_matches_torch_layer_norm():
     """The LayerNorm module without a gate is torch's own layer_norm (the library routine), forward and backward."""
     from issm_triton.layernorm_gated import LayerNorm

@@ -108,6 +108,27 @@ def test_one_launch_order_equals_codes_and_stable_sorts(n):
         assert torch.equal(inv[j], torch.argsort(want, dim=-1)), o
 
 
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
+def test_non_finite_coordinates_sort_alike_in_the_one_launch_kernel_and_in_the_separate_steps(bad):
+    """A NaN or infinite coordinate (a corrupt point): no conversion of NaN to an integer, and the one-launch kernel
+    agrees with issm_hilbert_codes + a stable argsort -- the path longer samples take -- on index and inverse.  The
+    minimum corner keeps a NaN the way torch.amin does, so both see the same cells; the result is a permutation."""
+    from dest3d_amd.serialization import ORDERS, hilbert_codes, hilbert_order
+    print(f"[case] hilbert order with a {bad} coordinate", flush=True)
+    g = torch.Generator().manual_seed(7)
+    pts = 8 * torch.rand(3, 500, 3, generator=g)
+    pts[0, 17, 1] = bad                    # sample 0: one bad coordinate; sample 1: a whole bad point; sample 2: clean
+    pts[1, 250] = bad
+    pts = pts.cuda()
+    orders = list(ORDERS)
+    idx, inv = hilbert_order(pts, orders, 9)
+    for j, o in enumerate(orders):
+        want = torch.argsort(hilbert_codes(pts, o, 9), dim=-1, stable=True)
+        assert torch.equal(idx[j], want), o
+        assert torch.equal(inv[j], torch.argsort(want, dim=-1)), o
+        assert torch.equal(torch.sort(idx[j], dim=-1).values, torch.arange(500, device="cuda").expand(3, 500))
+
+
 def test_order_rejects_what_it_does_not_hold():
     import ctypes as C
     from dest3d_amd import _lib as L

@@ -59,7 +59,10 @@ def test_noalloc_rmsnorm_bwd_equals_the_buffered_entry_point_twice_in_a_row():
     for rows, ncols, dtype, gated, layer in [(8192, 288, torch.bfloat16, True, False), (300, 288, torch.bfloat16, True, False),
                                              (4096, 1024, torch.float32, True, False), (7, 50, torch.float32, False, False),
                                              (4096, 512, torch.float32, True, True), (33, 288, torch.bfloat16, True, True),
-                                             (1, 288, torch.float32, True, False)]:
+                                             (1, 288, torch.float32, True, False),
+                                             # a bias case, then a larger case without one: its weight partials cover
+                                             # the part of the array where the bias partials of the call before lie
+                                             (2048, 512, torch.float32, True, True), (4096, 1024, torch.float32, True, False)]:
         print(f"[case] rmsnorm bwd noalloc rows={rows} ncols={ncols} {dtype} gated={gated} layer={layer}", flush=True)
         got = _run(lib, L, rows, ncols, dtype, gated, 5 + rows, noalloc=True, layer=layer)
         want = _run(lib, L, rows, ncols, dtype, gated, 5 + rows, noalloc=False, layer=layer)
@@ -94,3 +97,104 @@ def test_noalloc_rmsnorm_bwd_rejects_what_does_not_fit():
     a.rstd = rstd.data_ptr()
     a.dy, a.dy_row_stride, a.dx, a.dx_row_stride, a.dw, a.db = x1.data_ptr(), 1024, x1.data_ptr(), 1024, dw.data_ptr(), dw.data_ptr()
     assert lib.issm_gated_rmsnorm_bwd_noalloc(C.byref(a)) == -6 and b"weight and bias" in lib.issm_last_error()
+
+
+def _prepared(lib, L, rows, ncols, dtype, seed, layer):
+    """Forward done, every backward buffer allocated: what is left is the backward call itself."""
+    from dest3d_amd import layernorm_gated as N
+    g = torch.Generator().manual_seed(seed)
+    t = dict(x=torch.randn(rows, ncols, generator=g).to(dtype).cuda(), z=torch.randn(rows, ncols, generator=g).to(dtype).cuda(),
+             w=(1.0 + 0.1 * torch.randn(ncols, generator=g)).cuda(), dy=torch.randn(rows, ncols, generator=g).to(dtype).cuda(),
+             b=(0.1 * torch.randn(ncols, generator=g)).cuda() if layer else None)
+    t["y"] = torch.empty_like(t["x"])
+    t["rstd"] = torch.empty(rows, dtype=torch.float32, device="cuda")
+    t["mean"] = torch.empty(rows, dtype=torch.float32, device="cuda")
+    for k in ("dx", "dz"):
+        t[k] = torch.full_like(t["x"], float("nan"))
+    for k in ("dw", "db"):
+        t[k] = torch.full((ncols,), float("nan"), device="cuda")
+    t["part"] = torch.empty(2, lib.issm_rmsnorm_bwd_blocks(rows), ncols, dtype=torch.float32, device="cuda")
+
+    def args():
+        a = N._norm_args(t["x"], t["z"], t["w"], 1e-5, None, False, t["b"], layer)   # stream = torch's current one
+        a.y, a.y_row_stride, a.rstd = t["y"].data_ptr(), t["y"].stride(0), t["rstd"].data_ptr()
+        if layer:
+            a.mean, a.db = t["mean"].data_ptr(), t["db"].data_ptr()
+        a.dy, a.dy_row_stride = t["dy"].data_ptr(), t["dy"].stride(0)
+        a.dx, a.dx_row_stride = t["dx"].data_ptr(), t["dx"].stride(0)
+        a.dz, a.dz_row_stride = t["dz"].data_ptr(), t["dz"].stride(0)
+        a.dw = t["dw"].data_ptr()
+        return a
+    L.check(lib.issm_gated_rmsnorm_fwd(C.byref(args())), "fwd")
+    return t, args
+
+
+def _buffered(lib, L, t, args, layer):
+    a = args()
+    a.dw_partial = t["part"][0].data_ptr()
+    if layer:
+        a.db_partial = t["part"][1].data_ptr()
+    L.check(lib.issm_gated_rmsnorm_bwd(C.byref(a)), "bwd")
+    torch.cuda.synchronize()
+    return {k: t[k].clone() for k in ("dx", "dz", "dw") + (("db",) if layer else ())}
+
+
+@pytest.mark.parametrize("layer", [False, True])
+def test_noalloc_rmsnorm_bwd_allocates_nothing_and_takes_null_partial_buffers(layer):
+    """What the entry point is for: between the state before and after the call neither the driver's free memory
+    (which also sees allocations made behind torch's back) nor torch's own count moves, with dw_partial and
+    db_partial both NULL."""
+    from dest3d_amd import _lib as L
+    lib = L.load()
+    print(f"[case] rmsnorm bwd noalloc allocation check layer={layer}", flush=True)
+    t, args = _prepared(lib, L, 3000, 288, torch.bfloat16, 41, layer)
+    want = _buffered(lib, L, t, args, layer)
+    a = args()
+    a.dw_partial = a.db_partial = None
+    L.check(lib.issm_gated_rmsnorm_bwd_noalloc(C.byref(a)), "warm-up")     # first call on the device resolves the address
+    torch.cuda.synchronize()
+    for k in ("dx", "dz", "dw", "db"):
+        t[k].fill_(float("nan"))
+    torch.cuda.synchronize()
+    free0, alloc0, resv0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    L.check(lib.issm_gated_rmsnorm_bwd_noalloc(C.byref(a)), "bwd_noalloc")
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == resv0
+    for k, v in want.items():
+        assert torch.equal(t[k], v), k
+
+
+def test_noalloc_rmsnorm_bwd_in_a_hip_graph_replays_like_eager():
+    """The callers the entry point names record it into a graph.  After one eager call on the device (which resolves
+    the scratch array's address; a first call under capture is refused), the call is captured and replayed three
+    times on changed inputs, with eager work and synchronisations of the program's own between the replays; every
+    replay must equal the buffered entry point on the same inputs bit for bit."""
+    from dest3d_amd import _lib as L
+    lib = L.load()
+    print("[case] rmsnorm bwd noalloc under graph capture", flush=True)
+    t, args = _prepared(lib, L, 2500, 288, torch.bfloat16, 43, True)
+    a = args()
+    a.dw_partial = a.db_partial = None
+    L.check(lib.issm_gated_rmsnorm_bwd_noalloc(C.byref(a)), "warm-up")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ac = args()                                       # picks up the capturing stream
+            ac.dw_partial = ac.db_partial = None
+            L.check(lib.issm_gated_rmsnorm_bwd_noalloc(C.byref(ac)), "bwd_noalloc under capture")
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.Generator().manual_seed(99)
+    for rep in range(3):
+        t["dy"].copy_(torch.randn(t["dy"].shape, generator=g).to(t["dy"].dtype))
+        want = _buffered(lib, L, t, args, True)             # eager work of the program's own, then a synchronisation
+        for k in ("dx", "dz", "dw", "db"):
+            t[k].fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, v in want.items():
+            assert torch.equal(t[k], v), (rep, k)
