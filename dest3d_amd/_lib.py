@@ -217,7 +217,7 @@ def load() -> C.CDLL:
     lib.issm_param_gen_fwd.argtypes = [P(PGenArgs)]
     lib.issm_param_gen_bwd.argtypes = [P(PGenArgs)]
     for name in EXPORTS:
-        if name != "issm_last_error":
+        if name != "issm_last_error" and not name.endswith("_redo_ints"):
             getattr(lib, name).restype = C.c_int
     lib.issm_box_dist_bwd_scratch_bytes.restype = C.c_int64
     _lib = lib

@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libissm_hip.so")
-SOURCES = ["issm_abi.hip", "issm_fwd.hip", "issm_bwd.hip", "issm_bwd_tile.hip", "rmsnorm_gated.hip", "param_gen.hip", "dwconv_silu.hip", "box_dist.hip", "box_dist_sorted.hip", "hilbert.hip", "pointnet2_ops.hip", "transpose_states.hip"]
+SOURCES = ["issm_abi.hip", "issm_fwd.hip", "issm_fwd_tile.hip", "issm_bwd.hip", "issm_bwd_tile.hip", "rmsnorm_gated.hip", "param_gen.hip", "dwconv_silu.hip", "box_dist.hip", "box_dist_sorted.hip", "hilbert.hip", "pointnet2_ops.hip", "transpose_states.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",

@@ -169,7 +169,10 @@ int issm_scan_bwd(const issm_scan_args* args);
  * issm_stage_chunk_local: dt transform + cumsum, chunk states and C.A.B^T in one pass
  *   over dt.  Replaces _chunk_cumsum_fwd (issm_chunk_state.py:11-104), _chunk_state_fwd
  *   (issm_chunk_state.py:234-356) and _bmm_CABT_chunk_fwd (issm_cabt_bmm.py:7-153).
- *   states / cabt may be NULL to skip that product. */
+ *   states / cabt may be NULL to skip that product.
+ *   Launches made of complete 64 x 64 tiles run a kernel that writes every decay as a product of per-tile factors
+ *   (valid while no 16-row tile's sum of dt'.A.log2(e) falls below -100) and computes the chunks outside that range
+ *   with the general formulation in the same launch. */
 int issm_stage_chunk_local(const issm_scan_args* args, float* states, float* cs_last, float* cabt);
 /* issm_stage_state_passing_fwd: H_0 = h0, H_{c+1} = exp(cs_last_c) * H_c + S_c, in place
  *   (states[c] becomes H_c); final = H_nc.  Replaces _state_passing_fwd

@@ -511,6 +511,8 @@ def _stage_args(d, ndir=1):
     # head dimensions that leave threads of the state-passing kernels without a row of their own (stand-ins that only
     # load): 20 of 32 rows and 40 of 64 with 32-column slices, 36 of 48 with 64-column slices and many workgroups
     (1, 150, 2, 20, 64, 1), (1, 150, 2, 40, 96, 1), (4, 130, 8, 36, 512, 1),
+    # complete 64 x 64 tiles only: the kernels written for them (row-lane chunk_local, tile-base bwd_chunk)
+    (2, 192, 4, 32, 128, 2), (1, 128, 2, 36, 64, 1), (1, 128, 2, 64, 192, 1),
 ], ids=lambda s: "B%dL%dH%dP%dN%dG%d" % s)
 def test_stage_entry_points_match_oracle_intermediates(shape):
     """chunk_local -> state_passing -> chunk_scan and the backward stages, each against the
