@@ -977,3 +977,41 @@ def test_randomised_shapes_fp32_match_oracle():
                 assert g[k] is None
                 continue
             _check(f"d{k} {case}", g[k], g_ref[k], BWD32)
+
+
+@pytest.mark.parametrize("L_", [256, 230], ids=["complete_tiles", "ragged"])
+def test_nearly_undamped_scan_keeps_the_parameter_gradients(L_):
+    """dt' between 1e-6 and 5e-5 (what tiny locality weights make of it): every decay is within 1e-3 of 1, the scan is
+    nearly a plain running sum, and dA, dB, dC are sums whose terms carry a factor dt'.
+
+    (i) dt' handed over as it is (dt_softplus=False): every output and gradient at the usual fp32 bars.
+    (ii) dt' made inside the kernels by softplus of pre-activations in [-14, -10].  The reference evaluates softplus as
+    log(exp(x) + 1) in fp32 (softplus.py:9-11), and so do the kernels (with the hardware's exp2 / log2): for exp(x) near
+    1e-5 the rounding of 1 + exp(x) alone is worth up to 1 % of the result, so dt' -- and with it dA, dB, dC and the final
+    states, all proportional to dt' here -- differs from the exact softplus of the fp64 oracle by 1e-3 .. 1e-2.  That is
+    a property of the formula, not of the scan (part (i) runs the same scan at 1e-5); the test states the bound.  The
+    reference's module applies softplus in PyTorch and hands dt over as in (i) (dest_module.py:553-559)."""
+    _say(f"nearly undamped scan L={L_}")
+    g = torch.Generator().manual_seed(92)
+    d = _problem(2, L_, 4, 32, 128, 1, seed=91, D="h", softplus=False, h0=False)
+    d["dt"] = torch.rand(2, L_, 4, 128, generator=g) * 4.9e-5 + 1e-6
+    d["dt_limit"] = (0.0, float("inf"))
+    y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+    y, fin, gk, _ = _run_operator(d, torch.float32)
+    _check("out", y, y_ref, FWD32)
+    _check("final_states", fin, fin_ref, FWD32)
+    for k in GRAD_NAMES:
+        if d[k] is not None:
+            _check("d" + k, gk[k], g_ref[k], BWD32)
+    # (ii)
+    d = _problem(2, L_, 4, 32, 128, 1, seed=93, D="h", softplus=True, h0=False, bias=False)
+    d["dt"] = torch.rand(2, L_, 4, 128, generator=g) * 4.0 - 14.0
+    d["dt_limit"] = (0.0, float("inf"))
+    y, fin, gk, _ = _run_operator(d, torch.float32)
+    y_ref, fin_ref, g_exact = _oracle(d, GRAD_NAMES)
+    _check("out | in-kernel softplus", y, y_ref, FWD32)          # dominated by D x
+    _check("dx | in-kernel softplus", gk["x"], g_exact["x"], BWD32)
+    worst = max(max(_err(gk[k], g_exact[k])) for k in ("A", "B", "C"))
+    worst = max(worst, max(_err(fin, fin_ref)))
+    print(f"    against the exact softplus: worst of final states, dA, dB, dC = {worst:.3e}", flush=True)
+    assert 2e-4 < worst < 3e-2
