@@ -13,6 +13,7 @@
 
 namespace issm {
 int launch_chunk_local(const KP& p, float* states, float* cs_last, float* cabt, hipStream_t st);
+bool bwd_tile_available(const KP& p, const float* dy_ws);
 int launch_state_fwd(const KP& p, float* states, const float* cs_last, hipStream_t st);
 int launch_chunk_scan(const KP& p, const float* states, const float* cabt, float* out_x, hipStream_t st);
 int launch_bwd_gate(const KP& p, const float* out_x, float* dy_ws, hipStream_t st);
@@ -94,7 +95,7 @@ struct FwdWs {
   size_t states, cs_last, cabt, out_x, total;  // offsets in floats
 };
 struct BwdWs {
-  size_t dstates, dm, g_last, dh0_dir, partA, partBias, partD, redo, dy_ws, total;
+  size_t dstates, dm, g_last, dh0_dir, partA, partBias, partD, redo, dy_ws, ddt_part, total;
 };
 
 static int nchunks(const issm_dims& d) { return (d.seqlen + ISSM_CHUNK - 1) / ISSM_CHUNK; }
@@ -111,7 +112,8 @@ static FwdWs fwd_layout(const issm_dims& d, bool has_z) {
   return w;
 }
 
-static BwdWs bwd_layout(const issm_dims& d, bool has_z) {
+// ddt_part: with two directions and a bf16 ddt, the first direction's share of ddt in fp32 ((B, L, H, N))
+static BwdWs bwd_layout(const issm_dims& d, bool has_z, bool ddt_part) {
   const size_t Bt = (size_t)d.batch * d.ndir, nc = nchunks(d), H = d.nheads, P = d.headdim, N = d.dstate;
   BwdWs w;
   size_t o = 0;
@@ -124,9 +126,11 @@ static BwdWs bwd_layout(const issm_dims& d, bool has_z) {
   w.partD = o; o += align64(Bt * nc * H * P);
   w.redo = o; o += align64(Bt * nc * H * ((N + ISSM_CHUNK - 1) / ISSM_CHUNK));  // one int per direction, workgroup and head
   w.dy_ws = o; if (has_z) o += align64(Bt * d.seqlen * H * P);
+  w.ddt_part = o; if (ddt_part) o += align64((size_t)d.batch * d.seqlen * H * N);
   w.total = o;
   return w;
 }
+static bool wants_ddt_part(const issm_scan_args* a) { return a->dims.ndir == 2 && a->dt_dtype == ISSM_BF16; }
 
 static int check_dims(const issm_scan_args* a) {
   if (!a) return fail(ISSM_E_NULL, "args is NULL");
@@ -255,7 +259,7 @@ int issm_bwd_workspace_bytes(const issm_scan_args* a, size_t* out) {
   int rc = check_dims(a);
   if (rc) return rc;
   if (!out) return fail(ISSM_E_NULL, "out is NULL");
-  *out = bwd_layout(a->dims, a->z[0].ptr != nullptr).total * sizeof(float);
+  *out = bwd_layout(a->dims, a->z[0].ptr != nullptr, wants_ddt_part(a)).total * sizeof(float);
   return ISSM_OK;
 }
 
@@ -392,7 +396,7 @@ int issm_scan_bwd(const issm_scan_args* a) {
   if (rc) return rc;
   const bool has_z = a->z[0].ptr != nullptr;
   const FwdWs fw = fwd_layout(a->dims, has_z);
-  const BwdWs bw = bwd_layout(a->dims, has_z);
+  const BwdWs bw = bwd_layout(a->dims, has_z, wants_ddt_part(a));
   if (!a->saved) return fail(ISSM_E_WORKSPACE, "saved forward workspace is NULL");
   if (!a->bwd_workspace || a->bwd_workspace_bytes < bw.total * sizeof(float))
     return fail(ISSM_E_WORKSPACE, "backward workspace: need %zu bytes, got %zu", bw.total * sizeof(float),
@@ -415,8 +419,16 @@ int issm_scan_bwd(const issm_scan_args* a) {
     return rc;
   int* redo = reinterpret_cast<int*>(ws + bw.redo);
   int pending = 0;
+  KP pc = p;
+  if (wants_ddt_part(a) && bwd_tile_available(p, dy)) {
+    // both directions go through the tile-base kernel: the first one's share of the bf16 ddt travels in fp32
+    pc.ddt_part.ptr = ws + bw.ddt_part;
+    pc.ddt_part.s2 = p.N;
+    pc.ddt_part.s1 = (long)p.H * p.N;
+    pc.ddt_part.s0 = (long)p.L * p.H * p.N;
+  }
   for (int dir = 0; dir < p.ndir; ++dir) {
-    KP pd = p;
+    KP pd = pc;
     pd.dir0 = dir;
     if ((rc = launched(launch_bwd_chunk(pd, dy, sv + fw.states, ws + bw.dstates, ws + bw.dm, ws + bw.g_last,
                                         ws + bw.partA, ws + bw.partBias, redo, &pending, st),

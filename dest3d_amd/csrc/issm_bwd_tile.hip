@@ -47,8 +47,9 @@ struct BwdTileSmem {
 __device__ __forceinline__ bf8 cat_bf4(bf4 a, bf4 b) { return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7); }
 
 // PNF: the head dimension fills its 16-row tiles (P == 16 PT); ACC: ddt holds the other direction's share already and
-// this launch adds to it.
-template <int PT, bool IOB, bool PNF, bool ACC>
+// this launch adds to it; P32 (bf16 only): that share travels in fp32 through p.ddt_part -- the first direction's launch
+// writes it there, the second reads it from there and writes the once-rounded sum to ddt.
+template <int PT, bool IOB, bool PNF, bool ACC, bool P32>
 __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __restrict__ states,
                                                           const float* __restrict__ dstates,
                                                           const float* __restrict__ dm,
@@ -396,12 +397,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
     // rest of this head, which only waits for the predecessor's values (requested before them)
     const float gl_keep = l_gl;
     float old[16];
-    if constexpr (ACC) lane_load_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, old);
+    if constexpr (ACC) {
+      if constexpr (P32) lane_load_ln<false>(p.ddt_part, u.b, u.h, n, true, g4, rm, old);
+      else lane_load_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, old);
+    }
     request(head_of(min(hh + 1, p.hpg - 1)));  // (unconditional: the last head is requested again and not used)
     __builtin_amdgcn_sched_barrier(0);
     if (skip) {
       // the level-hierarchy kernel adds this head's share to ddt later: it must find the other direction's, or zero
-      if constexpr (!ACC) lane_store_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, val);  // (val is all zero here)
+      if constexpr (!ACC) {  // (val is all zero here)
+        if constexpr (P32) lane_store_ln<false>(p.ddt_part, u.b, u.h, n, true, g4, rm, val);
+        else lane_store_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, val);
+      } else if constexpr (P32) {
+        lane_store_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, old);  // the other direction's share moves into ddt
+      }
       continue;
     }
 
@@ -455,7 +464,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
 #pragma unroll
       for (int k = 0; k < 16; ++k) val[k] += old[k];
     }
-    lane_store_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, val);
+    if constexpr (!ACC && P32) lane_store_ln<false>(p.ddt_part, u.b, u.h, n, true, g4, rm, val);
+    else lane_store_ln<IOB>(p.ddt, u.b, u.h, n, true, g4, rm, val);
     sumA = scan_g_incl(sumA, g4);
     sumB = scan_g_incl(sumB, g4);
     if (g4 == 3) {
@@ -508,8 +518,14 @@ static int launch_bwd_tile_t(const KP& p, int blocks, const float* states, const
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(NTHREADS), sm, st, p, states, dstates, dm, g_last, partA, partBias, redo);
     return 0;
   };
-  if (pnf) return acc ? go(&k_bwd_tile<PT, IOB, true, true>) : go(&k_bwd_tile<PT, IOB, true, false>);
-  return acc ? go(&k_bwd_tile<PT, IOB, false, true>) : go(&k_bwd_tile<PT, IOB, false, false>);
+  if constexpr (IOB) {
+    if (p.ddt_part.ptr) {
+      if (pnf) return acc ? go(&k_bwd_tile<PT, IOB, true, true, true>) : go(&k_bwd_tile<PT, IOB, true, false, true>);
+      return acc ? go(&k_bwd_tile<PT, IOB, false, true, true>) : go(&k_bwd_tile<PT, IOB, false, false, true>);
+    }
+  }
+  if (pnf) return acc ? go(&k_bwd_tile<PT, IOB, true, true, false>) : go(&k_bwd_tile<PT, IOB, true, false, false>);
+  return acc ? go(&k_bwd_tile<PT, IOB, false, true, false>) : go(&k_bwd_tile<PT, IOB, false, false, false>);
 }
 
 int launch_bwd_tile(const KP& p, const float* states, const float* dstates, const float* dm, const float* g_last,

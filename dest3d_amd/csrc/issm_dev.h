@@ -55,6 +55,9 @@ struct KP {
   float dt_min, dt_max;
   TensorD x[2], Bm[2], Cm[2], z[2], out[2], dout[2], dx[2], dB[2], dC[2], dz[2];
   TensorD dt, ddt, h0;
+  // Two directions with a bf16 ddt: the first direction's share of ddt travels in fp32 through this (B, L, H, N) buffer
+  // instead of through ddt itself, so that the sum of the two is rounded to bf16 once (null: it travels through ddt).
+  TensorD ddt_part;
   const float* A;
   const float* D;
   const float* dt_bias;

@@ -146,7 +146,9 @@ int issm_abi_version(void);
 /* Message of the calling thread's most recent failure ("" if none). */
 const char* issm_last_error(void);
 
-/* Workspace sizes for a problem (only args->dims and args->z[0].ptr are read). */
+/* Workspace sizes for a problem (only args->dims, args->z[0].ptr and args->dt_dtype are read: with two directions and
+ * a bf16 ddt the backward workspace also holds the first direction's share of ddt in fp32, so that the sum of the two
+ * directions is rounded to bf16 once). */
 int issm_fwd_workspace_bytes(const issm_scan_args* args, size_t* out);
 int issm_bwd_workspace_bytes(const issm_scan_args* args, size_t* out);
 

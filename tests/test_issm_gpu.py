@@ -760,7 +760,7 @@ def test_benchmark_shape_bf16_bidirectional():
         _check(f"d{k} fused vs single direction", g[k].grad, part.grad, 1e-2)
     for k in ("A", "D", "h0"):
         _check(f"d{k} fused vs sum of parts", g[k].grad, a[k].grad + r[k].grad, 1e-5)
-    # ddt leaves in bf16: the fused call rounds the first direction's part before the second is added
+    # ddt leaves in bf16: the fused call rounds the fp32 sum of the two directions once, the two calls round each part
     _check("ddt fused vs sum of parts", g["dt"].grad, a["dt"].grad.float() + r["dt"].grad.float(), 1e-2)
     del o2, g2_, a, r, y1, y2
     # oracle on (b, h) = (5, 3), both directions through the fused call on strided views
@@ -1015,3 +1015,44 @@ def test_nearly_undamped_scan_keeps_the_parameter_gradients(L_):
     worst = max(worst, max(_err(fin, fin_ref)))
     print(f"    against the exact softplus: worst of final states, dA, dB, dC = {worst:.3e}", flush=True)
     assert 2e-4 < worst < 3e-2
+
+
+def test_bidirectional_bf16_ddt_is_the_once_rounded_sum_of_the_two_directions():
+    """ddt is shared by the two directions.  With a bf16 ddt the first direction's share travels in fp32 (through the
+    backward workspace) and the second direction's launch writes bf16(share 1 + share 2): one rounding.  The fp32 share
+    of direction 1 is read from the workspace of this call; the fp32 share of direction 2 from the workspace of a second
+    call whose direction 1 is this call's direction 2 on flipped tokens (equal to fp32 rounding: another instantiation
+    of the kernel).  The returned ddt must lie within half a bf16 unit in the last place of the fp32 sum of the two
+    -- everywhere; rounding the first share to bf16 before the addition, as a shared bf16 ddt would, breaks that in a
+    visible fraction of the elements (checked, so that the test is known to tell the two apart)."""
+    import bench
+    _say("bidirectional bf16 ddt: single rounding")
+    shape = dict(B=2, L=192, H=2, P=32, N=128, G=1, cs=64)
+    r1 = bench.Runner(torch, 2, torch.bfloat16, shape=shape, h0_std=0.1)
+    r2 = bench.Runner(torch, 2, torch.bfloat16, shape=shape, h0_std=0.1)
+    fl = lambda v: torch.flip(v, dims=[1])
+    for k in ("x", "B", "C", "dy"):
+        r2.t[k][0].copy_(fl(r1.t[k][1]))
+        r2.t[k][1].copy_(fl(r1.t[k][0]))
+    r2.t["dfinal"][0].copy_(r1.t["dfinal"][1])
+    r2.t["dfinal"][1].copy_(r1.t["dfinal"][0])
+    r2.t["dt"].copy_(fl(r1.t["dt"]))
+    n = shape["B"] * shape["L"] * shape["H"] * shape["N"]
+    share = []
+    for r in (r1, r2):
+        r.step()
+        torch.cuda.synchronize()
+        tail = r.bws.view(torch.float32)[-((n + 63) // 64 * 64):][:n]     # last region of the backward workspace
+        share.append(tail.view(shape["B"], shape["L"], shape["H"], shape["N"]).clone())
+    assert torch.isfinite(share[0]).all() and share[0].abs().max() > 0
+    for ra, p_own, p_other in ((r1, share[0], fl(share[1])), (r2, share[1], fl(share[0]))):
+        total = p_own.double() + p_other.double()
+        got = ra.ddt.double()
+        ulp = torch.exp2(torch.floor(torch.log2(got.abs().clamp_min(1e-30))) - 7)      # bf16: 8 significand bits
+        slack = 0.5 * ulp * 1.001 + 4e-6 * (p_own.abs() + p_other.abs()).double()      # + the second share's fp32 noise
+        once = (got - total).abs() <= slack
+        assert once.all(), f"{(~once).sum().item()} of {n} elements are further than half a bf16 ulp from the fp32 sum"
+        twice = (p_own.to(torch.bfloat16).float() + p_other).to(torch.bfloat16).double()  # what a shared bf16 ddt gives
+        frac = ((twice - total).abs() > slack).double().mean().item()
+        print(f"    rounded twice, {100 * frac:.1f} % of the elements would miss the bound", flush=True)
+        assert frac > 0.01
