@@ -246,26 +246,29 @@ class Runner:
         return res
 
 
-KERNEL_OF_STAGE = {"chunk_local": "k_chunk_local", "state_passing_fwd": "k_state_fwd_full", "chunk_scan": "k_chunk_scan",
-                   "bwd_dstates": "k_bwd_dstates", "state_passing_bwd": "k_state_bwd_full", "bwd_chunk": "k_bwd_chunk",
+KERNEL_OF_STAGE = {"chunk_local": "k_local_tile", "state_passing_fwd": "k_state_fwd_full", "chunk_scan": "k_chunk_scan",
+                   "bwd_dstates": "k_bwd_dstates", "state_passing_bwd": "k_state_bwd_full", "bwd_chunk": "k_bwd_tile",
                    "bwd_dx": "k_bwd_dx", "bwd_reduce": "k_bwd_reduce"}
 
 
 def measured_traffic(stage):
-    """HBM bytes per launch of a stage's kernel at the headline workload, as the committed profile summary holds it
+    """HBM bytes of a stage's kernel launches at the headline workload, as the committed profile summary holds them
     (profiles/issm_fwd_bwd_bidir_fp32_hbm_traffic.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled by
-    the same counters on a plain copy; last column of the kernel's row); None if the summary has no such row."""
+    the same counters on a plain copy; last column of the kernel's rows, added up over the stage's launches -- the chunk
+    backward is launched once per direction, and its algorithmic bytes are counted the same way); None if the summary
+    has no such row."""
     import re
     path = os.path.join(ROOT, "profiles", "issm_fwd_bwd_bidir_fp32_hbm_traffic.md")
     pat = re.compile(KERNEL_OF_STAGE.get(stage, stage) + r"\b")
+    total = None
     try:
         for row in open(path):
             cells = [c.strip() for c in row.strip().strip("|").split("|")]
             if len(cells) >= 4 and pat.search(cells[0]):
-                return float(cells[-1]) * 1e6
+                total = (total or 0.0) + float(cells[-1]) * 1e6
     except (OSError, ValueError):
-        pass
-    return None
+        return None
+    return total
 
 
 def stage_work(ndir, shape=None, elt=4):
