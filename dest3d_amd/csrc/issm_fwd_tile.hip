@@ -108,7 +108,7 @@ __device__ __forceinline__ void unpack4(const typename RawVec<BF>::type& r, floa
   }
 }
 
-template <int PT, bool IOB, bool DTB>
+template <int PT, bool IOB, bool DTB, bool FULLP>
 __global__ __launch_bounds__(NTHREADS, 2) void k_local_tile(KP p, float* __restrict__ states, float* __restrict__ cs_last,
                                                             float* __restrict__ cabt) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -224,10 +224,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_local_tile(KP p, float* __restr
     for (int k = 0; k < 16; ++k) et[k] = __shfl(up[k], last_lane, 64);  // whole-tile decay of the lane's columns
 #pragma unroll
     for (int k = 0; k < 16; k += 2) etmin = fminf(etmin, fminf(et[k], et[k + 1]));
-    if (i == 15) {  // the chunk's total decay (natural logarithm), four adjacent columns per lane
+    {  // the chunk's total decay (natural logarithm), four adjacent columns per lane group.  All 16 lanes of a group
+       // store the same values to the same place: a store under a lane condition sits behind a branch, and the waits
+       // for the requests in flight -- counted in order with the stores -- would then have to assume it away and wait
+       // for every store as well.
       f4 tot;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) tot[r] = (((pc[r] + pc[4 + r]) + pc[8 + r]) + pc[12 + r]) * LN2;
+      for (int r = 0; r < 4; ++r)
+        tot[r] = __shfl((((pc[r] + pc[4 + r]) + pc[8 + r]) + pc[12 + r]) * LN2, last_lane, 64);
       *(f4*)(cdst + n0 + ncol) = tot;
     }
 
@@ -300,9 +304,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_local_tile(KP p, float* __restr
       }
     }
     // S^T block: lane (p = i, kg) holds columns n0 + ncol .. + 3 of state row 16 pt + i
+    if (FULLP) {  // every state row exists: plain stores (see the note at the chunk's total decay)
 #pragma unroll
-    for (int pt = 0; pt < PT; ++pt)
-      if (16 * pt + i < p.P) *(f4*)(sdst + (16 * pt + i) * p.N + n0 + ncol) = sacc[pt];
+      for (int pt = 0; pt < PT; ++pt) *(f4*)(sdst + (16 * pt + i) * p.N + n0 + ncol) = sacc[pt];
+    } else {
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt)
+        if (16 * pt + i < p.P) *(f4*)(sdst + (16 * pt + i) * p.N + n0 + ncol) = sacc[pt];
+    }
   }
 #undef ISSM_REQUEST
 
@@ -370,9 +379,15 @@ int launch_local_tile(const KP& p, float* states, float* cs_last, float* cabt, h
 #define ISSM_LT(PT_, IOB_, DTB_)                                                                            \
   {                                                                                                         \
     const size_t sm = fwd_tile_lds<PT_, !IOB_>();                                                           \
-    constexpr auto kern = &k_local_tile<PT_, IOB_, DTB_>;                                                   \
-    if (int e = set_lds_tile(kern, sm)) return e;                                                           \
-    hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);                \
+    if (p.P == 16 * PT_) {                                                                                  \
+      constexpr auto kern = &k_local_tile<PT_, IOB_, DTB_, true>;                                           \
+      if (int e = set_lds_tile(kern, sm)) return e;                                                         \
+      hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);              \
+    } else {                                                                                                \
+      constexpr auto kern = &k_local_tile<PT_, IOB_, DTB_, false>;                                          \
+      if (int e = set_lds_tile(kern, sm)) return e;                                                         \
+      hipLaunchKernelGGL(kern, dim3(units), dim3(NTHREADS), sm, st, p, states, cs_last, cabt);              \
+    }                                                                                                       \
   }
 #define ISSM_LT_DT(PT_)                                                      \
   {                                                                          \
