@@ -222,8 +222,8 @@ __device__ __forceinline__ float dsoftplus_(float x) { return x <= 20.0f ? sigmo
 // FULLK: K is a multiple of 64, so no load or store needs a bound on k, and every per-lane address is a
 // pointer advanced once per trip plus a compile-time offset.  UNR blocks of 16 k have their loads in flight together.
 template <bool BF, bool FULLK, bool HASW>
-__global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
-  constexpr int UNR = (HASW || !BF) ? 2 : 4;
+__global__ __launch_bounds__(NTHREADS, (BF || !HASW || !FULLK) ? 4 : 3) void k_pgen_bwd(PGenP p) {
+  constexpr int UNR = 2;
   typedef typename std::conditional<BF, uint16_t, float>::type T;
   typedef typename std::conditional<BF, uint2, f4>::type T4;
   __shared__ float wred[4][16 * PG_M];
@@ -343,19 +343,26 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
       const float* pw2 = HASW ? p.weights + t * K + 4 * q : nullptr;
       T* pdd = p.ddist ? (T*)p.ddist + (t * K + i) * PG_M + 4 * q : nullptr;
       float* pdw = (HASW && p.dweights) ? p.dweights + t * K + 4 * q : nullptr;
-      for (int kb = 0; kb < K; kb += 16 * UNR) {
-        T4 ra[UNR], rab[UNR], rr2[UNR], rd[UNR];
-        f4 rw2[UNR];
+      // Two sets of operand registers used in turn: while one set is worked on, the other set's loads are in flight
+      // (K is a multiple of 64, so the number of 16 * UNR-column steps is even; the request after the last step reads
+      // the last step's operands once more instead of sitting under a branch).
+      constexpr int STEP = 16 * UNR;
+      const int nstep = K / STEP;
+      auto request = [&](int is, T4 (&ra)[UNR], T4 (&rab)[UNR], T4 (&rr2)[UNR], T4 (&rd)[UNR], f4 (&rw2)[UNR]) {
+        const int k0 = min(is, nstep - 1) * STEP;
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-          ra[u] = *(const T4*)(pa + 16 * u);
-          if (any_back) rab[u] = *(const T4*)(pab + 16 * u);
-          rd[u] = *(const T4*)(pd + 16 * u * PG_M);
+          ra[u] = *(const T4*)(pa + (ok2 ? k0 : 0) + 16 * u);
+          if (any_back) rab[u] = *(const T4*)(pab + (ok2b ? k0 : 0) + 16 * u);
+          rd[u] = *(const T4*)(pd + (long)(k0 + 16 * u) * PG_M);
           if constexpr (HASW) {
-            rr2[u] = *(const T4*)(pr2 + 16 * u);
-            rw2[u] = *(const f4*)(pw2 + 16 * u);
+            rr2[u] = *(const T4*)(pr2 + (isdt2 ? k0 : 0) + 16 * u);
+            rw2[u] = *(const f4*)(pw2 + k0 + 16 * u);
           }
         }
+      };
+      auto work = [&](int is, T4 (&ra)[UNR], T4 (&rab)[UNR], T4 (&rr2)[UNR], T4 (&rd)[UNR], f4 (&rw2)[UNR]) {
+        const int k0 = is * STEP;
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
           float* S = sg[wave][u];
@@ -392,7 +399,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
             f4 dd = zero4;
 #pragma unroll
             for (int s = 0; s < 3; ++s) dd = mfma4(wA[s], x[s], dd);
-            T* dst = pdd + 16 * u * PG_M;
+            T* dst = pdd + (long)(k0 + 16 * u) * PG_M;
             if constexpr (BF) {
               uint2 w;
               w.x = pack_bf16(dd.x, dd.y);
@@ -406,20 +413,19 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_pgen_bwd(PGenP p) {
             if (pdw != nullptr) {  // uniform: sum over the rows = over the 16 lanes that share q
 #pragma unroll
               for (int v = 0; v < 4; ++v) pw[v] = row_sum16_(pw[v]);
-              if (i == 15) *(f4*)(pdw + 16 * u) = pw;
+              if (i == 15) *(f4*)(pdw + k0 + 16 * u) = pw;
             }
           }
         }
-        const int step = 16 * UNR;
-        pa += ok2 ? step : 0;
-        pab += ok2b ? step : 0;
-        pd += step * PG_M;
-        if (pdd) pdd += step * PG_M;
-        if constexpr (HASW) {
-          pr2 += isdt2 ? step : 0;
-          pw2 += step;
-          if (pdw) pdw += step;
-        }
+      };
+      T4 ra0[UNR], rab0[UNR], rr20[UNR], rd0[UNR], ra1[UNR], rab1[UNR], rr21[UNR], rd1[UNR];
+      f4 rw20[UNR], rw21[UNR];
+      request(0, ra0, rab0, rr20, rd0, rw20);
+      for (int is = 0; is < nstep; is += 2) {
+        request(is + 1, ra1, rab1, rr21, rd1, rw21);
+        work(is, ra0, rab0, rr20, rd0, rw20);
+        request(is + 2, ra0, rab0, rr20, rd0, rw20);
+        work(is + 1, ra1, rab1, rr21, rd1, rw21);
       }
     } else {
       const void* safe = p.W;
