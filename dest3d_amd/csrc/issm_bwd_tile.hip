@@ -41,6 +41,12 @@ struct BwdTileSmem {
   uint16_t dys[NH * CS * LDP];
   uint16_t tm[NH * CS * LDM];
   float dbc[32 * NTHREADS];  // per-lane dB / dC accumulators [k][tid]
+  // bf16 inputs, two head tiles: the group's B and C values of every lane, packed in pairs, [i][tid] (i < 8: B, then C).
+  // They are the same for every head of the group; read from global memory again per head they miss the L2 (the heads'
+  // streams have been through it in between) and were a third of the kernel's reads.  fp32 inputs have no room for them
+  // at two workgroups per CU, wider heads no registers to spare for the change (they spill and lose what it gains).
+  static constexpr bool BCL = !SPLIT && PT == 2;
+  unsigned bc[BCL ? 16 * NTHREADS : 1];
   int bad[4];                // per wave: some column of the head exceeds SPAN_LIMIT
 };
 
@@ -60,6 +66,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
   typedef BwdTileSmem<PT, SPLIT> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
   constexpr int LDP = SM::LDP, LDM = SM::LDM, KT = (PT + 1) / 2;
+  constexpr bool BCL = SM::BCL;
   constexpr int KP_ = PT * 4;  // dS / H values per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
@@ -82,6 +89,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
 #pragma unroll
   for (int k = 0; k < 16; ++k) s.dbc[k * NTHREADS + tid] = s.dbc[(16 + k) * NTHREADS + tid] = 0.0f;
 
+  if constexpr (BCL) {
+    float tb[16], tc[16];
+    lane_load_ln<true>(p.Bm[u.dir], u.b, u.g, n, true, g4, rm, tb);
+    lane_load_ln<true>(p.Cm[u.dir], u.b, u.g, n, true, g4, rm, tc);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      s.bc[i * NTHREADS + tid] = pack_bf16(tb[2 * i], tb[2 * i + 1]);  // exact: the values are bf16 numbers
+      s.bc[(8 + i) * NTHREADS + tid] = pack_bf16(tc[2 * i], tc[2 * i + 1]);
+    }
+  }
+
   // the reversed direction's launch follows the forward one's and shares dt, x, B, C and ddt with it: it walks the
   // heads backwards, so what the first launch touched last (and the last-level cache still holds) is read first
   auto head_of = [&](int hh) { return u.g * p.hpg + (p.dir0 ? p.hpg - 1 - hh : hh); };
@@ -98,7 +116,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
   uint4 l_th0, l_th1, l_tl0, l_tl1;
   f4 l_xv[SPLIT ? PT : 1], l_dv[SPLIT ? PT : 1];
   uint2 l_nx[SPLIT ? 1 : PT], l_ny[SPLIT ? 1 : PT];
-  float l_raw[16], l_A, l_bias, l_gl, l_dsv[KP_], l_hv[KP_], l_Bv[16], l_Cv[16];
+  float l_raw[16], l_A, l_bias, l_gl, l_dsv[KP_], l_hv[KP_], l_Bv[BCL ? 1 : 16], l_Cv[BCL ? 1 : 16];
   auto request = [&](int hnext) {
     constexpr int G4 = 4 * PT;
     int tq = tid;
@@ -144,8 +162,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
     l_gl = g_last[vec_off(p, u.bt, u.c, hnext) + n];  // (every lane of the column; the last lane group uses it)
     lane_load_pn<KP_>(dstates + dst_off(p, u.bt, u.c, hnext), p.P, p.N, n, true, g4, PNF, l_dsv);
     lane_load_pn<KP_>(states + st_off(p, u.bt, u.c, hnext), p.P, p.N, n, true, g4, PNF, l_hv);
-    lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, true, g4, rm, l_Bv);
-    lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, true, g4, rm, l_Cv);
+    if constexpr (!BCL) {
+      lane_load_ln<IOB>(p.Bm[u.dir], u.b, u.g, n, true, g4, rm, l_Bv);
+      lane_load_ln<IOB>(p.Cm[u.dir], u.b, u.g, n, true, g4, rm, l_Cv);
+    }
   };
   request(head_of(0));
 
@@ -226,6 +246,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
       for (int I = 1; I < 5; ++I)
 #pragma unroll
         for (int J = 0; J < I; ++J) E[I][J] = ex2(bs[I] - bs[J]);
+      auto unpk = [](const unsigned (&a)[8], int k) {
+        return __uint_as_float((k & 1) ? (a[k >> 1] & 0xffff0000u) : (a[k >> 1] << 16));
+      };
+      auto half_of = [](unsigned w, int k) { return __uint_as_float((k & 1) ? (w & 0xffff0000u) : (w << 16)); };
       // Cu = C up (operand of the G blocks), Bi = B dt' iup (operand of the F blocks)
       bf4 Ch[4], Bh[4], Cl[4], Bl[4];
 #pragma unroll
@@ -233,7 +257,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int k = 4 * J + j;
-          float cu = l_Cv[k] * up[k], bi = l_Bv[k] * dtp[k] * iup[k];
+          float cu, bi;
+          if constexpr (!BCL) {
+            cu = l_Cv[k] * up[k];
+            bi = l_Bv[k] * dtp[k] * iup[k];
+          } else {  // out of the workgroup's LDS copy of the group's B and C
+            cu = half_of(s.bc[(8 + (k >> 1)) * NTHREADS + tid], k) * up[k];
+            bi = half_of(s.bc[(k >> 1) * NTHREADS + tid], k) * dtp[k] * iup[k];
+          }
           if (SPLIT) {
             cu = trunc16(cu);
             bi = trunc16(bi);
@@ -246,10 +277,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
           }
         }
       // B (and, for bf16 inputs, C) as the column phase needs them: bf16 inputs are bf16 numbers and stay packed, two
-      // to a register; the registers of the requests are then free for the next head's
+      // to a register
       unsigned bvp[8], cvp[8];
       float bvf[SPLIT ? 16 : 1];
-      if constexpr (!SPLIT) {
+      if constexpr (BCL) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          bvp[i] = s.bc[i * NTHREADS + tid];
+          cvp[i] = s.bc[(8 + i) * NTHREADS + tid];
+        }
+      } else if constexpr (!SPLIT) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           bvp[i] = pack_bf16(l_Bv[2 * i], l_Bv[2 * i + 1]);
@@ -259,9 +296,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_tile(KP p, const float* __r
 #pragma unroll
         for (int k = 0; k < 16; ++k) bvf[k] = l_Bv[k];
       }
-      auto unpk = [](const unsigned (&a)[8], int k) {
-        return __uint_as_float((k & 1) ? (a[k >> 1] & 0xffff0000u) : (a[k >> 1] << 16));
-      };
       __builtin_amdgcn_sched_barrier(0);
 
       int cq = cm, gq = g4;
