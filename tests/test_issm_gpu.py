@@ -1056,3 +1056,37 @@ def test_bidirectional_bf16_ddt_is_the_once_rounded_sum_of_the_two_directions():
         frac = ((twice - total).abs() > slack).double().mean().item()
         print(f"    rounded twice, {100 * frac:.1f} % of the elements would miss the bound", flush=True)
         assert frac > 0.01
+
+
+@pytest.mark.parametrize("io_dtype,dt_dtype", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)],
+                         ids=["x_fp32_dt_bf16", "x_bf16_dt_fp32"])
+@pytest.mark.parametrize("L_", [192, 150], ids=["complete_tiles", "ragged"])
+def test_dt_of_another_dtype_than_x(io_dtype, dt_dtype, L_):
+    """dt and x / B / C may have different element types (include/issm.h: io_dtype, dt_dtype): the complete-tile forward
+    kernel reads each in its own type, the chunk backward falls back to the level-hierarchy kernel for the mix.  Inputs
+    are rounded to the types they are passed in, so the oracle sees the same numbers."""
+    _say(f"mixed dtypes x {io_dtype} dt {dt_dtype} L={L_}")
+    d = _problem(2, L_, 4, 32, 128, 2, seed=61, D="h")
+    for k in ("x", "B", "C"):
+        d[k] = d[k].to(io_dtype).float()
+    d["dt"] = d["dt"].to(dt_dtype).float()
+    y_ref, fin_ref, g_ref = _oracle(d, GRAD_NAMES)
+    from dest3d_amd import ISSM_chunk_scan_combined
+    dev = "cuda"
+    cast = lambda t, dt_: None if t is None else t.to(dev, dt_).requires_grad_()
+    ins = dict(x=cast(d["x"], io_dtype), dt=cast(d["dt"], dt_dtype), A=cast(d["A"], torch.float32), B=cast(d["B"], io_dtype),
+               C=cast(d["C"], io_dtype), D=cast(d["D"], torch.float32), dt_bias=cast(d["dt_bias"], torch.float32),
+               h0=cast(d["h0"], torch.float32))
+    y, fin = ISSM_chunk_scan_combined(ins["x"], ins["dt"], ins["A"], ins["B"], ins["C"], 64, D=ins["D"],
+                                      dt_bias=ins["dt_bias"], initial_states=ins["h0"], dt_softplus=True,
+                                      dt_limit=d["dt_limit"], return_final_states=True)
+    assert y.dtype == io_dtype
+    ((y.float() * d["dy"].to(dev)).sum() + (fin * d["dfinal"].to(dev)).sum()).backward()
+    torch.cuda.synchronize()
+    assert ins["dt"].grad.dtype == dt_dtype
+    ft, bt = (FWD32, BWD32) if io_dtype == torch.float32 else (FWD16, BWD16)
+    _check("out", y, y_ref, ft)
+    _check("final_states", fin, fin_ref, ft)
+    for k in ("x", "dt", "A", "B", "C", "D", "dt_bias", "h0"):
+        # a bf16 ddt is rounded to 8 bits whatever the arithmetic behind it
+        _check("d" + k, ins[k].grad, g_ref[k], BWD16 if (k == "dt" and dt_dtype == torch.bfloat16) else bt)
