@@ -18,14 +18,18 @@ FLAGS = [
 ]
 
 
-# Sources whose results are integers decided by a floating-point quotient: compiled with IEEE division (no
-# reciprocal-multiply rewriting), so that a point exactly on a cell boundary lands in the same cell as on the host.
-EXACT_DIVISION = {"hilbert.hip"}
+# Sources whose results are integers decided by floating-point comparisons, compiled without -ffast-math:
+#  - hilbert.hip: a floating-point quotient picks the cell; IEEE division (no reciprocal-multiply rewriting) puts a
+#    point exactly on a cell boundary into the same cell as on the host;
+#  - pointnet2_ops.hip: squared distances pick indices (furthest point, ball membership, three nearest).  Under
+#    -ffast-math the backend fuses multiply and add whatever `#pragma clang fp contract(off)` says, and a distance one
+#    unit in the last place off decides a near-tie differently from a plain fp32 evaluation.
+EXACT_ARITHMETIC = {"hilbert.hip", "pointnet2_ops.hip"}
 
 
 def _compile(src: str) -> str:
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    flags = [f for f in FLAGS if f not in ("-ffast-math", "-fno-finite-math-only")] if src in EXACT_DIVISION else FLAGS
+    flags = [f for f in FLAGS if f not in ("-ffast-math", "-fno-finite-math-only")] if src in EXACT_ARITHMETIC else FLAGS
     cmd = [HIPCC, *flags, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
