@@ -1410,18 +1410,45 @@ __global__ __launch_bounds__(NTHREADS, 2) void k_bwd_chunk_bf_mixed(KP p, const 
 
 // ------------------------------------------------------------------------- dx
 // BF (bf16 inputs): the operands of the product over the state index are bf16 tiles read as matrix fragments of 8
-// adjacent columns; otherwise fp32 tiles.  `prod` (the dy * x products of the skip gradient) is its own small tile.
+// adjacent columns; fp32 inputs: (hi, lo) pairs of such tiles from two head tiles on, fp32 tiles for one.  `prod` (the
+// dy * x products of the skip gradient) is its own small tile for bf16 inputs.
+#ifndef DX_SPLIT_FROM
+#define DX_SPLIT_FROM 2
+#endif
 template <int PT, bool BF>
 struct BwdDxSmem {
   static constexpr int LDPT = PT * 16 + 4;
   static constexpr int LDK = NS + 8;
+  // fp32 inputs: the product over the state index on (hi, lo) bf16 tiles, hi.hi + hi.lo + lo.hi, instead of fp32
+  // matrix instructions, which take the vector ALU's issue slots (28 - 45 % of this kernel's cycles, never beside its
+  // vector work); the bf16 instructions run beside it.  (DX_SPLIT_FROM: head tiles from which this form is used.)
+  static constexpr bool SPL = !BF && PT >= DX_SPLIT_FROM;
+  static constexpr bool B16 = BF || SPL;
+  static constexpr int NH = SPL ? 2 : 1;
   float dys[CS * LDPT];
-  typename std::conditional<BF, uint16_t, float>::type bt[CS * (BF ? LDK : LDN)];        // B dt' exp2(last - cs) [m][n]
-  typename std::conditional<BF, uint16_t, float>::type dss[PT * 16 * (BF ? LDK : LDN)];  // dS [p][n]
-  float prod_own[BF ? CS * LDPT : 4];  // dy * x; with fp32 tiles it takes the place of `bt`
+  typename std::conditional<B16, uint16_t, float>::type bt[NH * CS * (B16 ? LDK : LDN)];        // B dt' exp2(last - cs) [m][n]
+  typename std::conditional<B16, uint16_t, float>::type dss[NH * PT * 16 * (B16 ? LDK : LDN)];  // dS [p][n]
+  float prod_own[BF ? CS * LDPT : 4];  // dy * x; with fp32 inputs it takes the place of `bt`
   __device__ __forceinline__ float* prod() { return BF ? prod_own : reinterpret_cast<float*>(bt); }
-  static constexpr int LDPROD = BF ? LDPT : LDN;
+  static constexpr int LDPROD = B16 ? LDPT : LDN;
+  static_assert(!SPL || sizeof(uint16_t) * NH * CS * LDK >= sizeof(float) * CS * LDPT, "dy * x fits in the place of bt");
 };
+// a (16 PT x 64) slab of fp32 values as (hi, lo) bf16 pairs into LDS hi / lo [p][col], row stride LD
+template <int PT, int LD>
+__device__ __forceinline__ void pn_store_hl(const PnRegs<PT>& r, uint16_t* hi, uint16_t* lo, int tid = threadIdx.x) {
+  typedef PnRegs<PT> R;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    const float w[4] = {r.v[i][0], r.v[i][1], r.v[i][2], r.v[i][3]};
+    bf4 h, l;
+    split4(w, h, l);
+    if (e < R::TOT) {
+      *(bf4*)(hi + pp * LD + c4) = h;
+      *(bf4*)(lo + pp * LD + c4) = l;
+    }
+  }
+}
 template <int PT, int LD>
 __device__ __forceinline__ void pn_store_bf16(const PnRegs<PT>& r, uint16_t* dst, int tid = threadIdx.x) {
   typedef PnRegs<PT> R;
@@ -1498,6 +1525,18 @@ __device__ __forceinline__ void k_bwd_dx_body(const KP& p, const float* __restri
           s.bt[lane_row(k, g4) * LDK + wave * 16 + cm] = (uint16_t)h2;
           s.bt[lane_row(k + 1, g4) * LDK + wave * 16 + cm] = (uint16_t)(h2 >> 16);
         }
+      } else if constexpr (SM::SPL) {
+#pragma unroll
+        for (int k = 0; k < 16; k += 2) {
+          const float b0 = bv[k] * dtp[k] * ex2(last - cs[k]), b1 = bv[k + 1] * dtp[k + 1] * ex2(last - cs[k + 1]);
+          const unsigned h2 = pack_bf16(b0, b1);
+          const unsigned l2 = pack_bf16(b0 - __uint_as_float(h2 << 16), b1 - __uint_as_float(h2 & 0xffff0000u));
+          const int o0 = lane_row(k, g4) * LDK + wave * 16 + cm, o1 = lane_row(k + 1, g4) * LDK + wave * 16 + cm;
+          s.bt[o0] = (uint16_t)h2;
+          s.bt[o1] = (uint16_t)(h2 >> 16);
+          s.bt[CS * LDK + o0] = (uint16_t)l2;
+          s.bt[CS * LDK + o1] = (uint16_t)(l2 >> 16);
+        }
       } else {
 #pragma unroll
         for (int k = 0; k < 16; ++k)
@@ -1505,6 +1544,7 @@ __device__ __forceinline__ void k_bwd_dx_body(const KP& p, const float* __restri
       }
     }
     if constexpr (IOB) pn_store_bf16<PT, LDK>(sv, s.dss);
+    else if constexpr (SM::SPL) pn_store_hl<PT, LDK>(sv, s.dss, s.dss + PT * 16 * LDK);
     else pn_store<PT>(sv, s.dss);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
@@ -1522,6 +1562,15 @@ __device__ __forceinline__ void k_bwd_dx_body(const KP& p, const float* __restri
         const bf8 a = frag8<LDK>(s.bt, wave * 16 + cm, g4, t);
 #pragma unroll
         for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma_bf(a, frag8<LDK>(s.dss, pt * 16 + cm, g4, t), acc[pt]);
+      }
+    } else if constexpr (SM::SPL) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const bf8 ah = frag8<LDK>(s.bt, wave * 16 + cm, g4, t), al = frag8<LDK>(s.bt + CS * LDK, wave * 16 + cm, g4, t);
+#pragma unroll
+        for (int pt = 0; pt < PT; ++pt)
+          acc[pt] = mfma_split(ah, al, frag8<LDK>(s.dss, pt * 16 + cm, g4, t),
+                               frag8<LDK>(s.dss + PT * 16 * LDK, pt * 16 + cm, g4, t), acc[pt]);
       }
     } else {
 #pragma unroll

@@ -156,14 +156,25 @@ __global__ __launch_bounds__(NTHREADS) void k_state_fwd(KP p, float* __restrict_
 
 // ------------------------------------------------------------------ chunk scan
 // BF (bf16 inputs): the operands of the product over the state index are bf16 tiles read as matrix fragments of 8
-// adjacent columns; otherwise fp32 tiles.
+// adjacent columns; fp32 inputs: (hi, lo) pairs of such tiles from two head tiles on, fp32 tiles for one.
+#ifndef SCAN_SPLIT_FROM
+#define SCAN_SPLIT_FROM 2
+#endif
 template <int PT, bool BF>
 struct FwdScanSmem {
   static constexpr int LDPT = PT * 16 + 4;
   static constexpr int LDK = NS + 8;  // row stride of the bf16 tiles
+  // fp32 inputs: the product over the state index on (hi, lo) bf16 tiles, hi.hi + hi.lo + lo.hi, instead of fp32
+  // matrix instructions.  An fp32 matrix instruction takes the vector ALU's issue slots (the two never overlap on this
+  // chip): they were 31 % of the kernel's issue cycles beside 46 % of vector work with two head tiles, 46 % beside
+  // 39 % with four.  Three bf16 instructions per product take a fifth of that and run beside the vector ALU; the
+  // splitting adds a quarter to the vector work.  (SCAN_SPLIT_FROM: head tiles from which this form is used.)
+  static constexpr bool SPL = !BF && PT >= SCAN_SPLIT_FROM;
+  static constexpr bool B16 = BF || SPL;
+  static constexpr int NH = SPL ? 2 : 1;
   float xs[CS * LDPT];                                          // x [s][p]
-  typename std::conditional<BF, uint16_t, float>::type ct[CS * (BF ? LDK : LDN)];       // C * exp2(cs) [l][n]
-  typename std::conditional<BF, uint16_t, float>::type hs[PT * 16 * (BF ? LDK : LDN)];  // H [p][n]
+  typename std::conditional<B16, uint16_t, float>::type ct[NH * CS * (B16 ? LDK : LDN)];       // C * exp2(cs) [l][n]
+  typename std::conditional<B16, uint16_t, float>::type hs[NH * PT * 16 * (B16 ? LDK : LDN)];  // H [p][n]
 };
 // a (16 PT x 64) slab of fp32 values (layout of pn_load) rounded to bf16 into LDS dst[p][col], row stride LD
 template <int PT, int LD>
@@ -173,6 +184,22 @@ __device__ __forceinline__ void pn_store_bf(const PnRegs<PT>& r, uint16_t* dst, 
   for (int i = 0; i < R::CNT; ++i) {
     const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
     if (e < R::TOT) *(uint2*)(dst + pp * LD + c4) = make_uint2(pack_bf16(r.v[i][0], r.v[i][1]), pack_bf16(r.v[i][2], r.v[i][3]));
+  }
+}
+// the same slab as (hi, lo) bf16 pairs
+template <int PT, int LD>
+__device__ __forceinline__ void pn_store_split(const PnRegs<PT>& r, uint16_t* hi, uint16_t* lo, int tid = threadIdx.x) {
+  typedef PnRegs<PT> R;
+#pragma unroll
+  for (int i = 0; i < R::CNT; ++i) {
+    const int e = tid + i * NTHREADS, pp = e / R::Q, c4 = (e % R::Q) * 4;
+    const float w[4] = {r.v[i][0], r.v[i][1], r.v[i][2], r.v[i][3]};
+    bf4 h, l;
+    split4(w, h, l);
+    if (e < R::TOT) {
+      *(bf4*)(hi + pp * LD + c4) = h;
+      *(bf4*)(lo + pp * LD + c4) = l;
+    }
   }
 }
 // the lane's 16 values of one column -> column `col` of a [64][LD] bf16 tile
@@ -240,12 +267,18 @@ __device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __re
 #pragma unroll
         for (int k = 0; k < 16; ++k) ctv[k] = cv[k] * ex2(cs[k]);
         col_store_bf<LDK>(ctv, s.ct, g4, wave * 16 + cm);
+      } else if constexpr (SM::SPL) {
+        float ctv[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) ctv[k] = cv[k] * ex2(cs[k]);
+        op_store<LDK, true>(ctv, s.ct, s.ct + CS * LDK, g4, wave * 16 + cm);
       } else {
 #pragma unroll
         for (int k = 0; k < 16; ++k) s.ct[lane_row(k, g4) * LDN + wave * 16 + cm] = cv[k] * ex2(cs[k]);
       }
     }
     if constexpr (IOB) pn_store_bf<PT, LDK>(hv, s.hs);
+    else if constexpr (SM::SPL) pn_store_split<PT, LDK>(hv, s.hs, s.hs + PT * 16 * LDK);
     else pn_store<PT>(hv, s.hs);
     if (n0 + NS < p.N) {
       n = n0 + NS + wave * 16 + cm;
@@ -257,8 +290,7 @@ __device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __re
       pn_load<PT>(p, hsrc, n0 + NS, hv);
     }
     __syncthreads();
-    // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows.  (fp32 product: both operands change with
-    // every slice and are used once or twice, so a bf16 split costs more vector work than it saves -- measured)
+    // y[l][p] += sum_n Ct[l][n] H[p][n]; wave owns 16 rows
     if constexpr (IOB) {
       // bf16 inputs: one rounding of C exp(cs) and of the entry state to bf16 (the reference stores the entry states
       // in the input dtype and casts its dot operands, issm_combined.py:87, issm_chunk_scan.py:149-190)
@@ -267,6 +299,15 @@ __device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __re
         const bf8 a = op_frag<LDK>(s.ct, wave * 16 + cm, g4, t);
 #pragma unroll
         for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma_bf(a, op_frag<LDK>(s.hs, pt * 16 + cm, g4, t), acc[pt]);
+      }
+    } else if constexpr (SM::SPL) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const bf8 ah = op_frag<LDK>(s.ct, wave * 16 + cm, g4, t), al = op_frag<LDK>(s.ct + CS * LDK, wave * 16 + cm, g4, t);
+#pragma unroll
+        for (int pt = 0; pt < PT; ++pt)
+          acc[pt] = mfma_split(ah, al, op_frag<LDK>(s.hs, pt * 16 + cm, g4, t),
+                               op_frag<LDK>(s.hs + PT * 16 * LDK, pt * 16 + cm, g4, t), acc[pt]);
       }
     } else {
 #pragma unroll
