@@ -358,8 +358,10 @@ __device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __re
     gstore<IOB, 4>(const_cast<void*>(to.ptr), (long)u.b * to.s0 + (long)u.h * to.s2, off, v);
   }
 }
+// fp32 inputs, two head tiles: 128 registers, so that a fourth workgroup lives on the CU (130 without the bound; the
+// nine spilled dwords cost less than the fourth workgroup gives: 52 -> 48.5 us)
 template <int PT, bool IOB, bool DTB, bool FULL>
-__global__ __launch_bounds__(NTHREADS) void k_chunk_scan(KP p, const float* __restrict__ states, const float* __restrict__ cabt, float* __restrict__ out_x) {
+__global__ __launch_bounds__(NTHREADS, (PT <= 2 && FULL && !IOB) ? 4 : 1) void k_chunk_scan(KP p, const float* __restrict__ states, const float* __restrict__ cabt, float* __restrict__ out_x) {
   k_chunk_scan_body<PT, IOB, DTB, FULL>(p, states, cabt, out_x);
 }
 // One launch for a sequence whose last chunk is ragged: complete-tile code for the complete chunks, the general code
