@@ -48,13 +48,15 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_gate(KP p, const float* __rest
 
 // ------------------------------------------------------------ dstates and dM
 // BF (bf16 inputs): the dy and x tiles are kept as bf16 (exact) and every product runs on the bf16 matrix instruction.
+// fp32 inputs: (hi, lo) bf16 pairs of the tiles (hi first), three bf16 instructions per product -- an fp32 matrix
+// instruction would keep the vector ALU from issuing while it runs.
 template <int PT, bool BF>
 struct BwdStSmem {
-  static constexpr int LDPT = PT * 16 + 4;
   static constexpr int LDP = PT * 16 + 8;   // bf16 tiles [l][p]
   static constexpr int LDT = CS + 8;        // transposed dy tile [p][l]
-  typename std::conditional<BF, uint16_t, float>::type dys[CS * (BF ? LDP : LDPT)];
-  typename std::conditional<BF, uint16_t, float>::type xs[CS * (BF ? LDP : LDPT)];
+  static constexpr int NH = BF ? 1 : 2;
+  uint16_t dys[NH * CS * LDP];
+  uint16_t xs[NH * CS * LDP];
   uint16_t dyt_hi[PT * 16 * LDT];             // dy tile transposed, [p][l]: operand of dH
   uint16_t dyt_lo[BF ? 8 : PT * 16 * LDT];
 };
@@ -67,7 +69,7 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
   extern __shared__ __align__(16) unsigned char smem_raw[];
   typedef BwdStSmem<PT, IOB> SM;
   SM& s = *reinterpret_cast<SM*>(smem_raw);
-  constexpr int LDPT = SM::LDPT, LDP = SM::LDP, LDT = SM::LDT;
+  constexpr int LDP = SM::LDP, LDT = SM::LDT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cm = lane & 15, g4 = lane >> 4;
   const Unit u = decode_unit(p, xcd_remap(blockIdx.x, gridDim.x));
@@ -91,8 +93,8 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
       lp_store_bf<PT, LDP>(dv, s.dys, tid);
       lp_store_bf<PT, LDP>(xv, s.xs, tid);
     } else {
-      lp_store<PT>(dv, s.dys, LDPT);
-      lp_store<PT>(xv, s.xs, LDPT);
+      lp_store_split<PT, LDP>(dv, s.dys, s.dys + CS * LDP, tid);
+      lp_store_split<PT, LDP>(xv, s.xs, s.xs + CS * LDP, tid);
     }
     if (dstates) lp_store_split_t<PT, LDT, !IOB>(dv, s.dyt_hi, s.dyt_lo);
   }
@@ -102,18 +104,16 @@ __device__ __forceinline__ void k_bwd_dstates_body(const KP& p, const float* __r
     float* m = dm + sq_off(p, u.bt, u.c, u.h);
     for (int j = 0; j <= wave; ++j) {
       f4 acc = {0, 0, 0, 0};
-      if constexpr (IOB) {
-        constexpr int KT = (PT + 1) / 2;
+      constexpr int KT = (PT + 1) / 2;
 #pragma unroll
-        for (int t = 0; t < KT; ++t) {
-          const bool half = (PT & 1) && t == KT - 1;  // an odd number of 16-column tiles: the last step is half full
-          const bf8 a = half ? split_frag<LDP, true>(s.dys, wave * 16 + cm, g4, t) : split_frag<LDP>(s.dys, wave * 16 + cm, g4, t);
-          const bf8 b = half ? split_frag<LDP, true>(s.xs, j * 16 + cm, g4, t) : split_frag<LDP>(s.xs, j * 16 + cm, g4, t);
-          acc = mfma_bf(a, b, acc);
-        }
-      } else {
-#pragma unroll
-        for (int kb = 0; kb < PT * 16; kb += 16) mma16_mm(acc, s.dys, LDPT, wave * 16, s.xs, LDPT, j * 16, kb, lane);
+      for (int t = 0; t < KT; ++t) {
+        const bool half = (PT & 1) && t == KT - 1;  // an odd number of 16-column tiles: the last step is half full
+        auto frag = [&](const uint16_t* tile, int row) {
+          return half ? split_frag<LDP, true>(tile, row, g4, t) : split_frag<LDP>(tile, row, g4, t);
+        };
+        const bf8 a = frag(s.dys, wave * 16 + cm), b = frag(s.xs, j * 16 + cm);
+        if constexpr (IOB) acc = mfma_bf(a, b, acc);
+        else acc = mfma_split(a, frag(s.dys + CS * LDP, wave * 16 + cm), b, frag(s.xs + CS * LDP, j * 16 + cm), acc);
       }
       {
         // The block goes out as the symmetric bf16 matrix T[i][j] = dM[max(i,j)][min(i,j)] (8 KB at the start of the
@@ -1584,11 +1584,19 @@ __device__ __forceinline__ void k_bwd_dx_body(const KP& p, const float* __restri
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb)
     if (kb >= wave) {  // uniform
+      // the lane's four M values and four dy values are the operands of one K = 16 bf16 instruction as they stand
+      // (k-slot j of lane group g4 <-> row 16 kb + 4 g4 + j), both as (hi, lo) pairs
+      bf4 ah, al;
+      split4(mf[kb], ah, al);
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) {
         const float* bp = s.dys + (16 * kb + 4 * g4) * LDPT + pt * 16 + cm;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[pt] = mfma4(mf[kb][j], bp[j * LDPT], acc[pt]);
+        const float yw[4] = {bp[0], bp[LDPT], bp[2 * LDPT], bp[3 * LDPT]};
+        bf4 bh, bl;
+        split4(yw, bh, bl);
+        acc[pt] = mfma_bf16k(al, bh, acc[pt]);
+        acc[pt] = mfma_bf16k(ah, bl, acc[pt]);  // (also for bf16 inputs: a gated dy is an fp32 product)
+        acc[pt] = mfma_bf16k(ah, bh, acc[pt]);
       }
     }
 

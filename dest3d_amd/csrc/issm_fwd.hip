@@ -321,13 +321,20 @@ __device__ __forceinline__ void k_chunk_scan_body(const KP& p, const float* __re
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb)
     if (kb <= wave) {  // uniform
+      // the lane's four M values and four x values are the operands of one K = 16 bf16 instruction as they stand
+      // (k-slot j of lane group g4 <-> row 16 kb + 4 g4 + j), M as a (hi, lo) pair and, for fp32 inputs, x too
+      const float mw[4] = {mf[kb][0], mf[kb][1], mf[kb][2], mf[kb][3]};
+      bf4 ah, al;
+      split4(mw, ah, al);
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) {
         const float* bp = s.xs + (16 * kb + 4 * g4) * LDPT + pt * 16 + cm;
-        acc[pt] = mfma4(mf[kb][0], bp[0], acc[pt]);
-        acc[pt] = mfma4(mf[kb][1], bp[LDPT], acc[pt]);
-        acc[pt] = mfma4(mf[kb][2], bp[2 * LDPT], acc[pt]);
-        acc[pt] = mfma4(mf[kb][3], bp[3 * LDPT], acc[pt]);
+        const float xw[4] = {bp[0], bp[LDPT], bp[2 * LDPT], bp[3 * LDPT]};
+        bf4 bh, bl;
+        split4(xw, bh, bl);
+        acc[pt] = mfma_bf16k(al, bh, acc[pt]);
+        if constexpr (!IOB) acc[pt] = mfma_bf16k(ah, bl, acc[pt]);  // (bf16 inputs: x is exact, its lo part zero)
+        acc[pt] = mfma_bf16k(ah, bh, acc[pt]);
       }
     }
 
