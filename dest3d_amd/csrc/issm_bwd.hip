@@ -52,9 +52,11 @@ __global__ __launch_bounds__(NTHREADS) void k_bwd_gate(KP p, const float* __rest
 // instruction would keep the vector ALU from issuing while it runs.
 template <int PT, bool BF>
 struct BwdStSmem {
-  static constexpr int LDP = PT * 16 + 8;   // bf16 tiles [l][p]
-  static constexpr int LDT = CS + 8;        // transposed dy tile [p][l]
   static constexpr int NH = BF ? 1 : 2;
+  // bf16 tiles [l][p]; four columns of padding instead of eight where the (hi, lo) tiles of four head tiles would
+  // otherwise take 55 KB and leave two workgroups per CU instead of three
+  static constexpr int LDP = PT * 16 + ((NH == 2 && PT >= 4) ? 4 : 8);
+  static constexpr int LDT = CS + 8;        // transposed dy tile [p][l]
   uint16_t dys[NH * CS * LDP];
   uint16_t xs[NH * CS * LDP];
   uint16_t dyt_hi[PT * 16 * LDT];             // dy tile transposed, [p][l]: operand of dH
