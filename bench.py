@@ -152,8 +152,21 @@ class Runner:
         if not self.fwd_only:
             self.L.check(self.lib.issm_scan_bwd(C.byref(self.a)), "bwd")
 
+    RAMP_MS = 40.0
+
+    def ramp(self):
+        """Untimed: keep the card under this workload's load for RAMP_MS.  After an idle spell (allocations, host work,
+        a fresh process) it runs below its steady clocks for 20 - 30 ms, whatever the number of warm-up steps asked for."""
+        torch = self.torch
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < self.RAMP_MS:
+            for _ in range(4):
+                self.step()
+            torch.cuda.synchronize()
+
     def time_steps(self, steps, warmup):
         torch = self.torch
+        self.ramp()
         for _ in range(warmup):
             self.step()
         torch.cuda.synchronize()
@@ -236,6 +249,16 @@ class Runner:
         for name, fn in stages:
             for _ in range(3):
                 self.L.check(fn(), name)
+            # (allocations and host work leave the card idle, and it then runs the next 20 ms below its steady clocks:
+            # every stage is launched for about that long before it is timed)
+            w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w0.record()
+            for _ in range(3):
+                fn()
+            w1.record()
+            w1.synchronize()
+            for _ in range(min(400, int(25e3 / max(w0.elapsed_time(w1) / 3 * 1e3, 1.0)))):
+                fn()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(reps):
@@ -385,7 +408,7 @@ def cpu_baseline(torch):
             "config0_forward_only_B2_us": round(f * 1e6, 1)}
 
 
-def time_box_dist_layer(torch, steps=10, warmup=3):
+def time_box_dist_layer(torch, steps=10, warmup=15):
     """BoxDistFun + local_weight + MultiHeadISSMScan as ISSMDecoderLayer chains them (models/dest_module.py:283-290)
     at the configs[2] shape, bf16 module, forward + backward, microseconds.  Returns (whole, box_dist forward only)."""
     from dest3d_amd.box_dist import BoxDistFun
@@ -553,7 +576,7 @@ def layer_compulsory_bytes(nlayers=1, with_encoding=False, B=8, L=1024, K=256, d
     return total
 
 
-def time_layer_stack(torch, steps=5, warmup=2, nlayers=6):
+def time_layer_stack(torch, steps=5, warmup=4, nlayers=6):
     """configs[2] as a whole: BoxDistFun + local_weight once, then `nlayers` MultiHeadISSMScan layers as a residual
     stack (models/dest_detector.py:207-235 calls the decoder layers on one shared encoding), bf16, forward + backward
     from a scalar loss, eager; microseconds per step."""
@@ -604,7 +627,7 @@ def caller_rooflines(variants):
     return out
 
 
-def time_module_layer(torch, steps=10, warmup=3, dtype=None, as_graph=False):
+def time_module_layer(torch, steps=10, warmup=25, dtype=None, as_graph=False):
     """One MultiHeadISSMScan-equivalent layer (configs[2]: d_model 288, 8 heads of 36, K = 256 queries, L = 1024
     keys, batch 8, d_dist 16, bf16 unless `dtype` says fp32, float locality weights as mask -- what DEST's decoder layer passes,
     models/dest_module.py:283-290), forward + backward through autograd from given output gradients (as inside a
@@ -676,7 +699,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # After an idle spell the card needs about 20 ms of continuous load to reach its steady clocks (the first steps of a
+    # run take 596 us, the 40th 535): Runner.ramp() covers that before the warm-up steps, whatever their number.
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
     ap.add_argument("--only-layer", action="store_true",
@@ -746,7 +771,7 @@ def main():
     roof["traffic"] = args.traffic if args.traffic is not None else measured_traffic(dom)
     variants, variant_rooflines = {}, {}
     if not args.no_variants:
-        variants["headline_as_hip_graph_replay"] = round(run.time_graph_replays(args.steps, 5), 2)
+        variants["headline_as_hip_graph_replay"] = round(run.time_graph_replays(args.steps, max(args.warmup, 40)), 2)
         del run
         for name, spec in WORKLOADS.items():
             if name == "headline":
@@ -767,7 +792,8 @@ def main():
         variants["detector_six_layers_plus_box_dist_bf16_fwd_bwd"] = round(time_layer_stack(torch), 2)
     line = {
         "metric": "ISSM scan fwd+bwd us/call at B=8,L=1024,N=256", "value": round(us, 2), "unit": "us/call",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "clock_ramp_ms_before_warmup": Runner.RAMP_MS,
+        "ms_per_step": round(us / 1e3, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: " + workload_text("headline"),
                    "variants": {k: workload_text(k) for k in WORKLOADS if k != "headline"}},
