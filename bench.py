@@ -704,6 +704,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-variants", action="store_true", help="time only the headline workload")
+    ap.add_argument("--steps-only", action="store_true",
+                    help="headline workload: the step loop and nothing else (for a kernel trace of the kernels as they run inside a step)")
     ap.add_argument("--only-layer", action="store_true",
                     help="time only the whole detector layer (module forward + backward) and print its JSON line")
     ap.add_argument("--only-box-dist", action="store_true",
@@ -760,6 +762,9 @@ def main():
         return
     run = make_runner(torch, "headline")
     us = run.time_steps(args.steps, args.warmup)
+    if args.steps_only:
+        print(json.dumps({"workload": "headline", "us_per_step": round(us, 2), "steps": args.steps, "warmup": args.warmup}))
+        return
     pct = run.step_percentiles(max(args.steps, 20))
     rep = workload_report(run, us)
     stages, per_stage = rep["stages_us"], rep["stage_roofline"]
