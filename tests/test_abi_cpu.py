@@ -130,3 +130,15 @@ def test_product_does_not_import_the_oracle():
         for f in files:
             if f.endswith(".py"):
                 assert "oracle" not in open(os.path.join(dirpath, f)).read(), f
+
+
+def test_bench_refuses_more_than_one_gpu_and_a_missing_gpu():
+    """bench.py measures one GPU: `--gpus N` above 1 exits with a message that says so, before anything touches a
+    device; without a GPU it exits with a message as well (there is nothing to fall back to)."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one MI355X" in r.stderr and r.stdout.strip() == ""
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")], capture_output=True, text=True, timeout=300)
+        assert r.returncode == 2 and "needs a GPU" in r.stderr
